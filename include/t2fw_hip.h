@@ -1,0 +1,138 @@
+/*
+ * t2fw_hip.h -- C ABI of libt2fw_hip.so: MI355X (gfx950) kernels for the
+ * decaying-fast-weight ("LFW") and delta-rule ("DFW") recurrences.
+ *
+ * This is the boundary a binding of the reference's op layer would call instead of
+ * its CUDA launchers.  Plain pointers and sizes only; no torch types.
+ *
+ *   reference interface replaced                         entry point here
+ *   ---------------------------------------------------  -------------------------
+ *   lfw_forward   (t2fw/csrc/lfw.cpp:28-48) =
+ *     lfw_cuda_forward (t2fw/csrc/lfw_kernel.cu:124-171)
+ *     + output einsum (lfw.cpp:45)                       t2fw_lfw_forward
+ *   lfw_backward  (t2fw/csrc/lfw.cpp:50-96) =
+ *     lfw_cuda_backward (lfw_kernel.cu:173-228)
+ *     + six einsums (lfw.cpp:84-93)                      t2fw_lfw_backward
+ *   T=1 use of lfw_forward in generation
+ *     (tests/benchmark.py:86-88,104-105)                 t2fw_lfw_step
+ *   dfw lfw_forward  (t2fw/csrc/dfw.cpp:27-39,
+ *     dfw_kernel.cu:406-470)                             t2fw_dfw_forward
+ *   dfw lfw_backward (t2fw/csrc/dfw.cpp:41-64,
+ *     dfw_kernel.cu:472-558)                             t2fw_dfw_backward
+ *
+ * Conventions
+ *   - All tensors are dense, row-major, device memory of ONE dtype (dtype code below):
+ *       x, f, out, g_out, d_x, d_f           [B, T, D]
+ *       q, k, f_key, d_q, d_k, d_f_key       [B, T, K]
+ *       s0, next_state, g_state, d_s0        [B, D, K]
+ *       ckpt                                 [B, NC, D, K],  NC = t2fw_lfw_num_ckpt(T, C)
+ *   - ckpt[b, c] is the state at the START of chunk c (time steps [c*C, (c+1)*C)), so
+ *     ckpt[b, 0] == s0[b].  It replaces the reference's [B, T, D, K] "ckpt_states"
+ *     (lfw_kernel.cu:140-144), which stores every step.
+ *   - The library owns no memory and keeps no state between calls.  Scratch space is
+ *     passed by the caller (`workspace`, size from the *_workspace_bytes query; may be
+ *     NULL when the query returns 0).
+ *   - `stream` is a hipStream_t (NULL = the null stream).  Launches are asynchronous;
+ *     the current HIP device must be the one that owns the pointers.
+ *   - Every function returns 0 on success, otherwise one of T2FW_ERR_* ; a message for
+ *     the calling thread's last failure is available from t2fw_last_error().
+ *   - Sizes are 64-bit; B or T may be 0 (no work, next_state = s0).
+ */
+#ifndef T2FW_HIP_H
+#define T2FW_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define T2FW_ABI_VERSION 1
+
+/* dtype codes (reference dispatch: AT_DISPATCH_FLOATING_TYPES_AND_HALF,
+ * lfw_kernel.cu:157 -> fp64/fp32/fp16; bf16 is added here) */
+#define T2FW_F32 0
+#define T2FW_F16 1
+#define T2FW_BF16 2
+#define T2FW_F64 3
+
+/* error codes */
+#define T2FW_OK 0
+#define T2FW_ERR_NULL_POINTER 1
+#define T2FW_ERR_BAD_DTYPE 2
+#define T2FW_ERR_BAD_SHAPE 3
+#define T2FW_ERR_MISALIGNED 4
+#define T2FW_ERR_UNSUPPORTED 5
+#define T2FW_ERR_WORKSPACE 6
+#define T2FW_ERR_HIP 7
+
+/* kernel-path selection for the `flags` argument */
+#define T2FW_FLAG_AUTO 0        /* fastest path that supports the shape/dtype      */
+#define T2FW_FLAG_FORCE_SCAN 1  /* exact per-step scan kernels only (any shape)     */
+
+int t2fw_abi_version(void);
+const char *t2fw_last_error(void);
+
+/* Number of checkpoints per batch row: ceil(T / C), at least 1. */
+int64_t t2fw_lfw_num_ckpt(int64_t T, int32_t C);
+
+/* Bytes of caller-provided scratch the forward / backward calls need (0 = none). */
+size_t t2fw_lfw_workspace_bytes(int64_t B, int64_t T, int64_t D, int64_t K,
+                                int32_t C, int32_t dtype, int32_t flags);
+
+/*
+ * Forward scan.  S_t = S_{t-1} * (f_t (x) f_key_t) + x_t (x) k_t ;  out_t = S_t q_t ;
+ * next_state = S_{T-1}.  Replaces lfw_forward (lfw.cpp:28-48).
+ * ckpt may be NULL (inference: no checkpoints are written); otherwise C >= 1.
+ */
+int t2fw_lfw_forward(const void *x, const void *f, const void *q, const void *k,
+                     const void *f_key, const void *s0,
+                     void *out, void *next_state, void *ckpt,
+                     int64_t B, int64_t T, int64_t D, int64_t K,
+                     int32_t C, int32_t dtype, int32_t flags,
+                     void *workspace, size_t workspace_bytes, void *stream);
+
+/*
+ * Backward pass: recomputes the states inside each chunk from ckpt, runs the
+ * reverse-time adjoint scan and writes all six gradients.  Replaces lfw_backward
+ * (lfw.cpp:50-96); gradient order as returned there (lfw.cpp:95).
+ */
+int t2fw_lfw_backward(const void *g_out, const void *g_state,
+                      const void *x, const void *f, const void *q, const void *k,
+                      const void *f_key, const void *s0, const void *ckpt,
+                      void *d_x, void *d_f, void *d_q, void *d_k, void *d_f_key,
+                      void *d_s0,
+                      int64_t B, int64_t T, int64_t D, int64_t K,
+                      int32_t C, int32_t dtype, int32_t flags,
+                      void *workspace, size_t workspace_bytes, void *stream);
+
+/*
+ * One generation step (T = 1) that may update the state in place
+ * (next_state == s0 is allowed).  x,f,out [B,D]; q,k,f_key [B,K].
+ */
+int t2fw_lfw_step(const void *x, const void *f, const void *q, const void *k,
+                  const void *f_key, const void *s0, void *out, void *next_state,
+                  int64_t B, int64_t D, int64_t K, int32_t dtype, void *stream);
+
+/*
+ * Delta rule.  out_t = S_{t-1} q_t ; delta_t = v_t - S_{t-1} k_t ;
+ * S_t = S_{t-1} + delta_t (x) k_t.   q,k,d_q,d_k [B,T,M]; v,out,delta,g_out,d_v [B,T,D];
+ * s0,final_state,g_state,d_s0 [B,D,M].  Replaces dfw.cpp:27-39 / :41-64.
+ */
+int t2fw_dfw_forward(const void *q, const void *k, const void *v, const void *s0,
+                     void *out, void *final_state, void *delta,
+                     int64_t B, int64_t T, int64_t D, int64_t M,
+                     int32_t dtype, void *stream);
+
+int t2fw_dfw_backward(const void *g_out, const void *g_state,
+                      const void *q, const void *k, const void *delta,
+                      const void *final_state,
+                      void *d_q, void *d_k, void *d_v, void *d_s0,
+                      int64_t B, int64_t T, int64_t D, int64_t M,
+                      int32_t dtype, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* T2FW_HIP_H */

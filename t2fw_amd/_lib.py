@@ -1,0 +1,74 @@
+"""ctypes binding of libt2fw_hip.so (C ABI declared in include/t2fw_hip.h).
+
+torch is imported first so that the library binds to the HIP runtime torch already
+loaded; stream handles from torch are then valid in the library.  There is no CPU
+fallback: a missing library is an ImportError-like RuntimeError at first use.
+"""
+import ctypes
+import os
+
+import torch  # noqa: F401  (must be loaded before the HIP library)
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "lib", "libt2fw_hip.so")
+
+ABI_VERSION = 1
+
+F32, F16, BF16, F64 = 0, 1, 2, 3
+DTYPE_CODE = {torch.float32: F32, torch.float16: F16, torch.bfloat16: BF16, torch.float64: F64}
+
+FLAG_AUTO = 0
+FLAG_FORCE_SCAN = 1
+
+_vp, _i64, _i32, _sz = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int32, ctypes.c_size_t
+
+# name -> (restype, argtypes); mirrors include/t2fw_hip.h one to one
+SIGNATURES = {
+    "t2fw_abi_version": (ctypes.c_int, []),
+    "t2fw_last_error": (ctypes.c_char_p, []),
+    "t2fw_lfw_num_ckpt": (_i64, [_i64, _i32]),
+    "t2fw_lfw_workspace_bytes": (_sz, [_i64, _i64, _i64, _i64, _i32, _i32, _i32]),
+    "t2fw_lfw_forward": (ctypes.c_int, [_vp] * 9 + [_i64] * 4 + [_i32] * 3 + [_vp, _sz, _vp]),
+    "t2fw_lfw_backward": (ctypes.c_int, [_vp] * 15 + [_i64] * 4 + [_i32] * 3 + [_vp, _sz, _vp]),
+    "t2fw_lfw_step": (ctypes.c_int, [_vp] * 8 + [_i64] * 3 + [_i32, _vp]),
+    "t2fw_dfw_forward": (ctypes.c_int, [_vp] * 7 + [_i64] * 4 + [_i32, _vp]),
+    "t2fw_dfw_backward": (ctypes.c_int, [_vp] * 10 + [_i64] * 4 + [_i32, _vp]),
+}
+
+_lib = None
+
+
+def load():
+    """Load the shared library (once).  Raises RuntimeError when it has not been built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise RuntimeError(
+            "t2fw: %s is missing -- build it with `python -m t2fw_amd.build` "
+            "(there is no CPU fallback)" % LIB_PATH)
+    lib = ctypes.CDLL(LIB_PATH)
+    for name, (res, args) in SIGNATURES.items():
+        fn = getattr(lib, name)
+        fn.restype = res
+        fn.argtypes = args
+    got = lib.t2fw_abi_version()
+    if got != ABI_VERSION:
+        raise RuntimeError("t2fw: library ABI version %d, binding expects %d" % (got, ABI_VERSION))
+    _lib = lib
+    return lib
+
+
+def check(rc):
+    """Turn a nonzero return code into RuntimeError carrying the library's message."""
+    if rc != 0:
+        msg = load().t2fw_last_error()
+        raise RuntimeError("t2fw error %d: %s" % (rc, msg.decode() if msg else "?"))
+
+
+def ptr(t):
+    return ctypes.c_void_p(t.data_ptr()) if t is not None else ctypes.c_void_p(0)
+
+
+def current_stream_handle(device):
+    return ctypes.c_void_p(torch.cuda.current_stream(device).cuda_stream)

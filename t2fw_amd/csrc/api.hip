@@ -1,0 +1,178 @@
+// C ABI of libt2fw_hip.so: argument validation and kernel-path selection.
+// Declarations and the reference interfaces they replace: include/t2fw_hip.h.
+#include "common.hpp"
+#include "lfw_scan.hpp"
+
+#include <cstring>
+
+namespace t2fw {
+
+namespace {
+thread_local char g_err[512] = "";
+}
+
+int fail(int code, const char *fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+int check_hip(hipError_t e, const char *what) {
+    if (e == hipSuccess) return T2FW_OK;
+    return fail(T2FW_ERR_HIP, "%s: %s", what, hipGetErrorString(e));
+}
+
+namespace {
+
+size_t elem_size(int dtype) {
+    switch (dtype) {
+        case T2FW_F32: return 4;
+        case T2FW_F16: return 2;
+        case T2FW_BF16: return 2;
+        case T2FW_F64: return 8;
+    }
+    return 0;
+}
+
+struct NamedPtr {
+    const char *name;
+    const void *ptr;
+};
+
+int check_ptrs(const NamedPtr *v, int n, size_t es) {
+    for (int i = 0; i < n; ++i) {
+        if (v[i].ptr == nullptr) return fail(T2FW_ERR_NULL_POINTER, "%s is a null pointer", v[i].name);
+        if (reinterpret_cast<uintptr_t>(v[i].ptr) % es != 0)
+            return fail(T2FW_ERR_MISALIGNED, "%s is not aligned to the %zu-byte element size", v[i].name, es);
+    }
+    return T2FW_OK;
+}
+
+int check_dims(int64_t B, int64_t T, int64_t D, int64_t K) {
+    if (B < 0 || T < 0) return fail(T2FW_ERR_BAD_SHAPE, "B=%lld and T=%lld must be non-negative", (long long)B, (long long)T);
+    if (D < 1 || K < 1) return fail(T2FW_ERR_BAD_SHAPE, "D=%lld and K=%lld must be positive", (long long)D, (long long)K);
+    // every tensor must be addressable with 63-bit element offsets
+    const long double big = (long double)B * (long double)(T > 0 ? T : 1) * (long double)D * (long double)K;
+    if (big > 4.0e18L) return fail(T2FW_ERR_BAD_SHAPE, "B*T*D*K is too large");
+    return T2FW_OK;
+}
+
+}  // namespace
+}  // namespace t2fw
+
+using namespace t2fw;
+
+extern "C" {
+
+int t2fw_abi_version(void) { return T2FW_ABI_VERSION; }
+
+const char *t2fw_last_error(void) { return g_err; }
+
+int64_t t2fw_lfw_num_ckpt(int64_t T, int32_t C) {
+    if (C < 1 || T <= 0) return 1;
+    return (T + C - 1) / C;
+}
+
+size_t t2fw_lfw_workspace_bytes(int64_t B, int64_t T, int64_t D, int64_t K, int32_t C, int32_t dtype,
+                                int32_t flags) {
+    (void)B; (void)T; (void)D; (void)K; (void)C; (void)dtype; (void)flags;
+    return 0;
+}
+
+int t2fw_lfw_forward(const void *x, const void *f, const void *q, const void *k, const void *f_key,
+                     const void *s0, void *out, void *next_state, void *ckpt, int64_t B, int64_t T,
+                     int64_t D, int64_t K, int32_t C, int32_t dtype, int32_t flags, void *workspace,
+                     size_t workspace_bytes, void *stream) {
+    (void)workspace; (void)workspace_bytes; (void)flags;
+    const size_t es = elem_size(dtype);
+    if (es == 0) return fail(T2FW_ERR_BAD_DTYPE, "unknown dtype code %d", dtype);
+    int rc = check_dims(B, T, D, K);
+    if (rc) return rc;
+    if (ckpt != nullptr && C < 1) return fail(T2FW_ERR_BAD_SHAPE, "checkpoint interval C=%d must be >= 1", C);
+    if (B == 0) return T2FW_OK;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    {
+        const NamedPtr sp[] = {{"s0", s0}, {"next_state", next_state}};
+        if ((rc = check_ptrs(sp, 2, es))) return rc;
+        if (ckpt != nullptr && reinterpret_cast<uintptr_t>(ckpt) % es != 0)
+            return fail(T2FW_ERR_MISALIGNED, "ckpt is not aligned to the %zu-byte element size", es);
+    }
+    if (T == 0) {   // no steps: the state passes through
+        const size_t bytes = (size_t)(B * D * K) * es;
+        if (next_state != s0 &&
+            (rc = check_hip(hipMemcpyAsync(next_state, s0, bytes, hipMemcpyDeviceToDevice, st), "state copy")))
+            return rc;
+        if (ckpt != nullptr &&
+            (rc = check_hip(hipMemcpyAsync(ckpt, s0, bytes, hipMemcpyDeviceToDevice, st), "checkpoint copy")))
+            return rc;
+        return T2FW_OK;
+    }
+    const NamedPtr ptrs[] = {{"x", x}, {"f", f}, {"q", q}, {"k", k}, {"f_key", f_key}, {"out", out}};
+    if ((rc = check_ptrs(ptrs, 6, es))) return rc;
+
+    ScanFwdArgs a{};
+    a.x = x; a.f = f; a.q = q; a.k = k; a.f_key = f_key; a.s0 = s0;
+    a.out = out; a.next_state = next_state; a.ckpt = ckpt;
+    a.row_select = nullptr;
+    a.B = B; a.T = T; a.D = D; a.K = K;
+    a.C = ckpt ? C : 1;
+    a.NC = ckpt ? t2fw_lfw_num_ckpt(T, C) : 1;
+    return scan_forward(a, dtype, st);
+}
+
+int t2fw_lfw_backward(const void *g_out, const void *g_state, const void *x, const void *f, const void *q,
+                      const void *k, const void *f_key, const void *s0, const void *ckpt, void *d_x,
+                      void *d_f, void *d_q, void *d_k, void *d_f_key, void *d_s0, int64_t B, int64_t T,
+                      int64_t D, int64_t K, int32_t C, int32_t dtype, int32_t flags, void *workspace,
+                      size_t workspace_bytes, void *stream) {
+    (void)workspace; (void)workspace_bytes; (void)flags; (void)s0;
+    const size_t es = elem_size(dtype);
+    if (es == 0) return fail(T2FW_ERR_BAD_DTYPE, "unknown dtype code %d", dtype);
+    int rc = check_dims(B, T, D, K);
+    if (rc) return rc;
+    if (C < 1) return fail(T2FW_ERR_BAD_SHAPE, "checkpoint interval C=%d must be >= 1", C);
+    if (B == 0) return T2FW_OK;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    {
+        const NamedPtr sp[] = {{"g_state", g_state}, {"d_s0", d_s0}};
+        if ((rc = check_ptrs(sp, 2, es))) return rc;
+    }
+    if (T == 0) {
+        if (d_s0 != g_state)
+            return check_hip(hipMemcpyAsync(d_s0, g_state, (size_t)(B * D * K) * es, hipMemcpyDeviceToDevice, st),
+                             "state-gradient copy");
+        return T2FW_OK;
+    }
+    const NamedPtr ptrs[] = {{"g_out", g_out}, {"x", x}, {"f", f}, {"q", q}, {"k", k}, {"f_key", f_key},
+                             {"ckpt", ckpt}, {"d_x", d_x}, {"d_f", d_f}, {"d_q", d_q}, {"d_k", d_k},
+                             {"d_f_key", d_f_key}};
+    if ((rc = check_ptrs(ptrs, 12, es))) return rc;
+
+    ScanBwdArgs a{};
+    a.g_out = g_out; a.g_state = g_state; a.x = x; a.f = f; a.q = q; a.k = k; a.f_key = f_key; a.ckpt = ckpt;
+    a.d_x = d_x; a.d_f = d_f; a.d_q = d_q; a.d_k = d_k; a.d_f_key = d_f_key; a.d_s0 = d_s0;
+    a.row_select = nullptr;
+    a.B = B; a.T = T; a.D = D; a.K = K; a.C = C;
+    a.NC = t2fw_lfw_num_ckpt(T, C);
+    return scan_backward(a, dtype, st);
+}
+
+int t2fw_lfw_step(const void *x, const void *f, const void *q, const void *k, const void *f_key, const void *s0,
+                  void *out, void *next_state, int64_t B, int64_t D, int64_t K, int32_t dtype, void *stream) {
+    return t2fw_lfw_forward(x, f, q, k, f_key, s0, out, next_state, nullptr, B, 1, D, K, 1, dtype,
+                            T2FW_FLAG_AUTO, nullptr, 0, stream);
+}
+
+int t2fw_dfw_forward(const void *, const void *, const void *, const void *, void *, void *, void *, int64_t,
+                     int64_t, int64_t, int64_t, int32_t, void *) {
+    return fail(T2FW_ERR_UNSUPPORTED, "delta-rule forward is not built yet");
+}
+
+int t2fw_dfw_backward(const void *, const void *, const void *, const void *, const void *, const void *, void *,
+                      void *, void *, void *, int64_t, int64_t, int64_t, int64_t, int32_t, void *) {
+    return fail(T2FW_ERR_UNSUPPORTED, "delta-rule backward is not built yet");
+}
+
+}  // extern "C"

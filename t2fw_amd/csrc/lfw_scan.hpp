@@ -1,0 +1,27 @@
+// Argument blocks and host entry points of the exact scan kernels (lfw_scan.hip).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <cstdint>
+
+namespace t2fw {
+
+struct ScanFwdArgs {
+    const void *x, *f, *q, *k, *f_key, *s0;
+    void *out, *next_state, *ckpt;      // ckpt may be null
+    const int32_t *row_select;          // null, or per batch row: 0 = skip the row
+    int64_t B, T, D, K, NC;
+    int32_t C, kg, tb, ntiles;
+};
+
+struct ScanBwdArgs {
+    const void *g_out, *g_state, *x, *f, *q, *k, *f_key, *ckpt;
+    void *d_x, *d_f, *d_q, *d_k, *d_f_key, *d_s0;
+    const int32_t *row_select;
+    int64_t B, T, D, K, NC;
+    int32_t C, kg, use_sub, ntiles;
+};
+
+int scan_forward(const ScanFwdArgs &a, int dtype, hipStream_t stream);
+int scan_backward(const ScanBwdArgs &a, int dtype, hipStream_t stream);
+
+}  // namespace t2fw

@@ -1,0 +1,145 @@
+"""Autograd boundary of the decay rule: same call as the reference's
+``LFWFunction.apply(value, forget, query, key, f_key, state)``
+(t2fw/functional_lfw.py:31-78), backed by the HIP kernels in libt2fw_hip.so.
+
+Differences from the reference that a caller can observe:
+  * the state is stored only every ``C`` steps (``[B, ceil(T/C), D, K]``) instead of
+    every step (``[B, T, D, K]``, t2fw/csrc/lfw_kernel.cu:140-144); backward recomputes
+    inside each chunk.  ``next_state`` is its own ``[B, D, K]`` tensor, not a view.
+  * bf16 is accepted in addition to fp64/fp32/fp16.
+  * kernels run on the current torch stream and on the inputs' device.
+"""
+import os
+
+import torch
+
+from . import _lib
+
+DEFAULT_CKPT_INTERVAL = 64
+
+
+def _ckpt_interval():
+    v = os.environ.get("T2FW_CKPT_INTERVAL")
+    return int(v) if v else DEFAULT_CKPT_INTERVAL
+
+
+def _check_input(t, name):
+    # mirrors CHECK_INPUT of t2fw/csrc/lfw.cpp:24-26 (TORCH_CHECK -> RuntimeError)
+    if not t.is_cuda:
+        raise RuntimeError("%s must be a CUDA tensor" % name)
+    if not t.is_contiguous():
+        raise RuntimeError("%s must be contiguous" % name)
+
+
+def _dtype_code(dtype):
+    try:
+        return _lib.DTYPE_CODE[dtype]
+    except KeyError:
+        raise RuntimeError("t2fw: unsupported dtype %s" % dtype)
+
+
+class LFWFunction(torch.autograd.Function):
+    """Decay update rule S_t = S_{t-1} * (f_t (x) f_key_t) + x_t (x) k_t, o_t = S_t q_t.
+    Inputs are already gated (no sigmoid is applied here), as in the reference."""
+
+    @staticmethod
+    def forward(ctx, value, forget, query, key, f_key, state):
+        """Return: (outputs [B,T,D], final state [B,D,K])"""
+        # same asserts as t2fw/functional_lfw.py:42-49
+        assert value.shape == forget.shape
+        assert query.shape == key.shape
+        assert query.shape == f_key.shape
+        assert forget.dtype == value.dtype
+        assert query.dtype == value.dtype
+        assert f_key.dtype == value.dtype
+        assert state.dtype == value.dtype
+        assert key.dtype == value.dtype
+        for t, n in ((value, "x"), (forget, "f"), (query, "query"), (key, "key"),
+                     (f_key, "f_key"), (state, "state")):
+            _check_input(t, n)
+        if value.dim() != 3 or query.dim() != 3 or state.dim() != 3:
+            raise RuntimeError("t2fw: expected x,f [B,T,D]; q,k,f_key [B,T,K]; state [B,D,K]")
+        B, T, D = value.shape
+        K = query.shape[2]
+        if query.shape[0] != B or query.shape[1] != T or tuple(state.shape) != (B, D, K):
+            raise RuntimeError("t2fw: inconsistent shapes x %s, query %s, state %s"
+                               % (tuple(value.shape), tuple(query.shape), tuple(state.shape)))
+        code = _dtype_code(value.dtype)
+        lib = _lib.load()
+        need_grad = any(ctx.needs_input_grad)
+        C = _ckpt_interval()
+        dev = value.device
+        with torch.cuda.device(dev):
+            outputs = torch.empty_like(value)
+            next_state = torch.empty_like(state)
+            ckpt = None
+            if need_grad:
+                nc = lib.t2fw_lfw_num_ckpt(T, C)
+                ckpt = torch.empty((B, nc, D, K), dtype=value.dtype, device=dev)
+            ws_bytes = lib.t2fw_lfw_workspace_bytes(B, T, D, K, C, code, _lib.FLAG_AUTO)
+            ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev) if ws_bytes else None
+            _lib.check(lib.t2fw_lfw_forward(
+                _lib.ptr(value), _lib.ptr(forget), _lib.ptr(query), _lib.ptr(key), _lib.ptr(f_key),
+                _lib.ptr(state), _lib.ptr(outputs), _lib.ptr(next_state), _lib.ptr(ckpt),
+                B, T, D, K, C, code, _lib.FLAG_AUTO, _lib.ptr(ws), ws_bytes,
+                _lib.current_stream_handle(dev)))
+        if need_grad:
+            ctx.save_for_backward(value, forget, query, key, f_key, state, ckpt)
+            ctx.ckpt_interval = C
+        return outputs, next_state
+
+    @staticmethod
+    def backward(ctx, grad_output, grad_state):
+        value, forget, query, key, f_key, state, ckpt = ctx.saved_tensors
+        # t2fw/functional_lfw.py:71-72
+        assert grad_state.dtype == value.dtype
+        assert grad_output.dtype == value.dtype
+        grad_output = grad_output.contiguous()
+        grad_state = grad_state.contiguous()
+        B, T, D = value.shape
+        K = query.shape[2]
+        code = _dtype_code(value.dtype)
+        lib = _lib.load()
+        C = ctx.ckpt_interval
+        dev = value.device
+        with torch.cuda.device(dev):
+            d_x = torch.empty_like(value)
+            d_f = torch.empty_like(forget)
+            d_q = torch.empty_like(query)
+            d_k = torch.empty_like(key)
+            d_fk = torch.empty_like(f_key)
+            d_s = torch.empty_like(state)
+            ws_bytes = lib.t2fw_lfw_workspace_bytes(B, T, D, K, C, code, _lib.FLAG_AUTO)
+            ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev) if ws_bytes else None
+            _lib.check(lib.t2fw_lfw_backward(
+                _lib.ptr(grad_output), _lib.ptr(grad_state), _lib.ptr(value), _lib.ptr(forget),
+                _lib.ptr(query), _lib.ptr(key), _lib.ptr(f_key), _lib.ptr(state), _lib.ptr(ckpt),
+                _lib.ptr(d_x), _lib.ptr(d_f), _lib.ptr(d_q), _lib.ptr(d_k), _lib.ptr(d_fk), _lib.ptr(d_s),
+                B, T, D, K, C, code, _lib.FLAG_AUTO, _lib.ptr(ws), ws_bytes,
+                _lib.current_stream_handle(dev)))
+        # order of t2fw/csrc/lfw.cpp:95
+        return d_x, d_f, d_q, d_k, d_fk, d_s
+
+
+def lfw_step(x, f, query, key, f_key, state, out=None, inplace=True):
+    """One generation step (T = 1) without autograd: x,f [B,D]; query,key,f_key [B,K];
+    state [B,D,K] updated in place when ``inplace``.  Returns (out [B,D], state).
+    The reference does this through the T=1 forward (tests/benchmark.py:104-105), which
+    allocates a new state tensor per step."""
+    for t, n in ((x, "x"), (f, "f"), (query, "query"), (key, "key"), (f_key, "f_key"), (state, "state")):
+        _check_input(t, n)
+        assert t.dtype == x.dtype
+    B, D = x.shape
+    K = query.shape[1]
+    assert tuple(state.shape) == (B, D, K) and f.shape == x.shape
+    assert key.shape == query.shape and f_key.shape == query.shape
+    lib = _lib.load()
+    dev = x.device
+    with torch.cuda.device(dev):
+        if out is None:
+            out = torch.empty_like(x)
+        nxt = state if inplace else torch.empty_like(state)
+        _lib.check(lib.t2fw_lfw_step(
+            _lib.ptr(x), _lib.ptr(f), _lib.ptr(query), _lib.ptr(key), _lib.ptr(f_key), _lib.ptr(state),
+            _lib.ptr(out), _lib.ptr(nxt), B, D, K, _dtype_code(x.dtype), _lib.current_stream_handle(dev)))
+    return out, nxt
