@@ -1,0 +1,256 @@
+#!/usr/bin/env python3
+"""Benchmark of the LFW hot path on one MI355X.
+
+A "step" is one forward + backward pass of the decay-rule recurrence over one batch of
+synthetic input already resident in HBM, at the headline configuration
+(B*H=96, T=1024, D=K=64, fp16 I/O, checkpoint interval 64).  Prints ONE JSON line.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg3|cfg2|cfg4|cfg5]
+                    [--no-cpu-baseline]
+
+value      = B*T*steps / wall time of the timed region, in Mtokens/s (token = one
+             (batch row, time step) pair), driving the C ABI directly with preallocated
+             outputs; `autograd_api` repeats it through LFWFunction.apply + backward.
+roofline   = algorithmic bytes of the dominant launch / its mean duration measured with
+             events on the launch stream, against 8 TB/s.
+cpu_baseline = the TorchScript restatement of the reference loop (oracle/), fp32,
+             forward + autograd backward, timed on this host's cores on a bounded sample.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+
+WORKLOADS = {
+    # name: (B, T, D, K, dtype, gate_mean, state_std, backward)
+    "cfg2": dict(B=96, T=1024, D=64, K=64, dtype="float16", gate_mean=2.0, state_std=0.0, backward=False),
+    "cfg3": dict(B=96, T=1024, D=64, K=64, dtype="float16", gate_mean=2.0, state_std=0.0, backward=True),
+    "cfg4": dict(B=128, T=8192, D=64, K=64, dtype="bfloat16", gate_mean=3.0, state_std=0.1, backward=True),
+    "cfg5": dict(B=49152, T=1, D=64, K=64, dtype="float16", gate_mean=2.0, state_std=0.0, backward=False),
+}
+
+
+def algorithmic_bytes(B, T, D, K, es, C, backward):
+    """Bytes one pass must move: forward reads x,f,q,k,f_key + s0, writes out +
+    next_state (+ checkpoints when a backward follows); backward reads the five inputs,
+    g_out, checkpoints and g_state, writes five gradients and d_s0."""
+    tok = B * T
+    nc = (T + C - 1) // C
+    fwd = tok * (3 * D + 3 * K) * es + 2 * B * D * K * es
+    if not backward:
+        return fwd, 0
+    fwd += B * nc * D * K * es
+    bwd = tok * (3 * D + 3 * K) * es + B * nc * D * K * es + tok * (2 * D + 3 * K) * es + 2 * B * D * K * es
+    return fwd, bwd
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--workload", default="cfg3", choices=sorted(WORKLOADS))
+    ap.add_argument("--ckpt-interval", type=int, default=64)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--force-scan", action="store_true", help="exact scan kernels only")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build measures one GPU only (the path shards over the batch with no "
+              "exchange); run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    from t2fw_amd import _lib
+    from tests.lfw_cases import make_config_inputs
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(1)
+    lib = _lib.load()
+    w = WORKLOADS[args.workload]
+    B, T, D, K = w["B"], w["T"], w["D"], w["K"]
+    dtype = getattr(torch, w["dtype"])
+    es = torch.empty((), dtype=dtype).element_size()
+    C = args.ckpt_interval
+    backward = w["backward"]
+    flags = _lib.FLAG_FORCE_SCAN if args.force_scan else _lib.FLAG_AUTO
+    code = _lib.DTYPE_CODE[dtype]
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+
+    # several independent input sets so that consecutive steps do not re-read the same
+    # lines out of the 256 MB last-level cache
+    per_set = (5 * B * T * D + (B * T * D if backward else 0)) * es * (2 if backward else 1) + 2 * B * T * D * es
+    nsets = max(2, min(16, int(1.2e9 // max(per_set, 1)) + 1))
+    sets = []
+    nc = lib.t2fw_lfw_num_ckpt(T, C)
+    ws_bytes = lib.t2fw_lfw_workspace_bytes(B, T, D, K, C, code, flags)
+    for i in range(nsets):
+        x, f, q, k, fk, s, go, gs = make_config_inputs(B, T, D, K, dtype, seed=i, gate_mean=w["gate_mean"],
+                                                        state_std=w["state_std"])
+        ins = [t.to(dev) for t in (x, f, q, k, fk, s)]
+        d = dict(ins=ins, out=torch.empty_like(ins[0]), nxt=torch.empty_like(ins[5]),
+                 ws=torch.empty(max(ws_bytes, 1), dtype=torch.uint8, device=dev))
+        if backward:
+            d["ckpt"] = torch.empty(B, nc, D, K, dtype=dtype, device=dev)
+            d["go"], d["gs"] = go.to(dev), gs.to(dev)
+            d["grads"] = [torch.empty_like(t) for t in ins]
+        sets.append(d)
+    stream = _lib.current_stream_handle(dev)
+
+    def fwd(d):
+        _lib.check(lib.t2fw_lfw_forward(*[_lib.ptr(t) for t in d["ins"]], _lib.ptr(d["out"]), _lib.ptr(d["nxt"]),
+                                        _lib.ptr(d.get("ckpt")), B, T, D, K, C, code, flags,
+                                        _lib.ptr(d["ws"]), ws_bytes, stream))
+
+    def bwd(d):
+        i = d["ins"]
+        g = d["grads"]
+        _lib.check(lib.t2fw_lfw_backward(_lib.ptr(d["go"]), _lib.ptr(d["gs"]), *[_lib.ptr(t) for t in i],
+                                         _lib.ptr(d["ckpt"]), *[_lib.ptr(t) for t in g], B, T, D, K, C, code,
+                                         flags, _lib.ptr(d["ws"]), ws_bytes, stream))
+
+    def step(i):
+        d = sets[i % nsets]
+        fwd(d)
+        if backward:
+            bwd(d)
+
+    for i in range(args.warmup):
+        step(i)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        step(i)
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    ms_per_step = wall / args.steps * 1e3
+    mtok = B * T * args.steps / wall / 1e6
+
+    # per-launch durations with events on the launch stream (same stream torch uses)
+    nrep = min(args.steps, 100)
+    ev = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(nrep)]
+    for i in range(nrep):
+        d = sets[i % nsets]
+        ev[i][0].record()
+        fwd(d)
+        ev[i][1].record()
+        if backward:
+            bwd(d)
+        ev[i][2].record()
+    torch.cuda.synchronize()
+    fwd_ms = sorted(e[0].elapsed_time(e[1]) for e in ev)
+    bwd_ms = sorted(e[1].elapsed_time(e[2]) for e in ev)
+    fwd_avg = sum(fwd_ms) / nrep
+    bwd_avg = sum(bwd_ms) / nrep
+    fwd_bytes, bwd_bytes = algorithmic_bytes(B, T, D, K, es, C, backward)
+    if backward and bwd_avg >= fwd_avg:
+        dom, dom_bytes, dom_ms = "backward", bwd_bytes, bwd_avg
+    else:
+        dom, dom_bytes, dom_ms = "forward", fwd_bytes, fwd_avg
+    achieved = dom_bytes / (dom_ms * 1e-3) / 1e9
+    traffic = None
+    tpath = os.path.join(ROOT, "profiles", "traffic_%s.json" % args.workload)
+    if os.path.exists(tpath):
+        try:
+            traffic = json.load(open(tpath)).get(dom)
+        except Exception:
+            traffic = None
+    roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic, "kernel": dom,
+                "algorithmic_bytes": dom_bytes, "avg_launch_ms": round(dom_ms, 5)}
+    whole = (fwd_bytes + bwd_bytes) / (ms_per_step * 1e-3) / 1e9
+
+    # the same step through the autograd API (allocations and Python dispatch included)
+    autograd = None
+    if backward:
+        from t2fw.functional_lfw import LFWFunction
+        os.environ["T2FW_CKPT_INTERVAL"] = str(C)
+        leaves = [[t.detach().clone().requires_grad_(True) for t in d["ins"]] for d in sets[:2]]
+
+        def astep(i):
+            ins = leaves[i % 2]
+            o, n = LFWFunction.apply(*ins)
+            torch.autograd.backward([o, n], [sets[i % 2]["go"], sets[i % 2]["gs"]])
+            for t in ins:
+                t.grad = None
+        for i in range(5):
+            astep(i)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        n_a = min(args.steps, 50)
+        for i in range(n_a):
+            astep(i)
+        torch.cuda.synchronize()
+        autograd = {"ms_per_step": round((time.perf_counter() - t0) / n_a * 1e3, 4)}
+        autograd["value"] = round(B * T / autograd["ms_per_step"] / 1e3, 1)
+
+    cpu = None
+    if not args.no_cpu_baseline:
+        cpu = cpu_baseline(w, backward)
+
+    line = {
+        "metric": "fwd+bwd Mtokens/s + % HBM roofline, B*H=96 T=1024 d=kdim=64 fp16" if args.workload == "cfg3"
+                  else "Mtokens/s (%s)" % args.workload,
+        "value": round(mtok, 1), "unit": "Mtokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": {"float16": "fp16", "bfloat16": "bf16"}[w["dtype"]] + " I/O, fp32 state",
+        "data": "synthetic",
+        "config": {"workload": "%s: B=%d T=%d D=%d K=%d %s %s, checkpoint interval %d" % (
+            args.workload, B, T, D, K, w["dtype"], "fwd+bwd" if backward else "fwd", C),
+            "input_sets_rotated": nsets, "path": "scan" if args.force_scan else "auto"},
+        "whole_step_algorithmic_GBs": round(whole, 1),
+        "whole_step_roofline_frac": round(whole / HBM_PEAK_GBS, 4),
+        "forward_avg_ms": round(fwd_avg, 5), "backward_avg_ms": round(bwd_avg, 5) if backward else None,
+        "autograd_api": autograd,
+        "roofline": roofline,
+        "cpu_baseline": cpu,
+    }
+    if cpu:
+        line["speedup_vs_cpu"] = round(mtok / cpu["value"], 1) if cpu["value"] else None
+    print(json.dumps(line))
+
+
+def cpu_baseline(w, backward):
+    """TorchScript restatement of the reference loop, fp32, on this host's cores.
+    Bounded sample: a slice of the batch (rows are independent, so cost is linear in B)."""
+    import torch
+    from oracle.lfw_ref import lfw_reference_script
+    from tests.lfw_cases import make_config_inputs
+    B, T, D, K = w["B"], w["T"], w["D"], w["K"]
+    Bs = min(B, 24)
+    Ts = min(T, 1024)
+    x, f, q, k, fk, s, go, gs = make_config_inputs(Bs, Ts, D, K, torch.float32, seed=0, gate_mean=w["gate_mean"],
+                                                    state_std=w["state_std"])
+    ins = [t.clone().requires_grad_(backward) for t in (x, f, q, k, fk, s)]
+
+    def run():
+        o, n = lfw_reference_script(*ins)
+        if backward:
+            torch.autograd.backward([o, n], [go, gs])
+            for t in ins:
+                t.grad = None
+    run()   # warm-up (TorchScript profiling runs)
+    run()
+    t0 = time.perf_counter()
+    reps = 0
+    while reps < 3 or (time.perf_counter() - t0 < 10.0 and reps < 20):
+        run()
+        reps += 1
+    dt = (time.perf_counter() - t0) / reps
+    return {"value": round(Bs * Ts / dt / 1e6, 4), "unit": "Mtokens/s", "cores": torch.get_num_threads(),
+            "kind": "port",
+            "sample": "TorchScript loop (oracle/lfw_ref.py), fp32, %s, B=%d of %d rows, T=%d of %d, "
+                      "%d reps, %.2f s each; host reports %d cpus" % (
+                          "fwd+autograd bwd" if backward else "fwd", Bs, B, Ts, T, reps, dt, os.cpu_count())}
+
+
+if __name__ == "__main__":
+    main()
