@@ -70,6 +70,9 @@ extern "C" {
 /* kernel-path selection for the `flags` argument */
 #define T2FW_FLAG_AUTO 0        /* fastest path that supports the shape/dtype      */
 #define T2FW_FLAG_FORCE_SCAN 1  /* exact per-step scan kernels only (any shape)     */
+#define T2FW_FLAG_FP16_OPERANDS 2 /* fp16 tensors: fp16 (not bf16) matrix-core operands;
+                                     more mantissa, but rows whose 16-step gate products
+                                     fall below 2^-8 take the exact scan path          */
 
 int t2fw_abi_version(void);
 const char *t2fw_last_error(void);

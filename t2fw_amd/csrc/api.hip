@@ -2,8 +2,10 @@
 // Declarations and the reference interfaces they replace: include/t2fw_hip.h.
 #include "common.hpp"
 #include "lfw_scan.hpp"
+#include "lfw_chunk.hpp"
 
 #include <cstring>
+#include <initializer_list>
 
 namespace t2fw {
 
@@ -50,6 +52,19 @@ int check_ptrs(const NamedPtr *v, int n, size_t es) {
     return T2FW_OK;
 }
 
+bool aligned16(std::initializer_list<const void *> ps) {
+    for (const void *p : ps)
+        if (p != nullptr && reinterpret_cast<uintptr_t>(p) % 16 != 0) return false;
+    return true;
+}
+
+// The chunked matrix-core kernels cover D = K = 64 with 16-bit tensors.
+bool chunk_shape_ok(int64_t D, int64_t K, int32_t dtype, int32_t flags) {
+    return (flags & T2FW_FLAG_FORCE_SCAN) == 0 && D == 64 && K == 64 && (dtype == T2FW_F16 || dtype == T2FW_BF16);
+}
+
+size_t row_flag_bytes(int64_t B) { return (size_t)((B * 4 + 255) / 256 * 256); }
+
 int check_dims(int64_t B, int64_t T, int64_t D, int64_t K) {
     if (B < 0 || T < 0) return fail(T2FW_ERR_BAD_SHAPE, "B=%lld and T=%lld must be non-negative", (long long)B, (long long)T);
     if (D < 1 || K < 1) return fail(T2FW_ERR_BAD_SHAPE, "D=%lld and K=%lld must be positive", (long long)D, (long long)K);
@@ -77,7 +92,8 @@ int64_t t2fw_lfw_num_ckpt(int64_t T, int32_t C) {
 
 size_t t2fw_lfw_workspace_bytes(int64_t B, int64_t T, int64_t D, int64_t K, int32_t C, int32_t dtype,
                                 int32_t flags) {
-    (void)B; (void)T; (void)D; (void)K; (void)C; (void)dtype; (void)flags;
+    (void)T; (void)C;
+    if (B > 0 && chunk_shape_ok(D, K, dtype, flags)) return row_flag_bytes(B);
     return 0;
 }
 
@@ -85,7 +101,6 @@ int t2fw_lfw_forward(const void *x, const void *f, const void *q, const void *k,
                      const void *s0, void *out, void *next_state, void *ckpt, int64_t B, int64_t T,
                      int64_t D, int64_t K, int32_t C, int32_t dtype, int32_t flags, void *workspace,
                      size_t workspace_bytes, void *stream) {
-    (void)workspace; (void)workspace_bytes; (void)flags;
     const size_t es = elem_size(dtype);
     if (es == 0) return fail(T2FW_ERR_BAD_DTYPE, "unknown dtype code %d", dtype);
     int rc = check_dims(B, T, D, K);
@@ -119,6 +134,21 @@ int t2fw_lfw_forward(const void *x, const void *f, const void *q, const void *k,
     a.B = B; a.T = T; a.D = D; a.K = K;
     a.C = ckpt ? C : 1;
     a.NC = ckpt ? t2fw_lfw_num_ckpt(T, C) : 1;
+
+    if (chunk_shape_ok(D, K, dtype, flags) && (ckpt == nullptr || C % 32 == 0) &&
+        aligned16({x, f, q, k, f_key, s0, out, next_state, ckpt})) {
+        if (workspace == nullptr || workspace_bytes < row_flag_bytes(B))
+            return fail(T2FW_ERR_WORKSPACE, "workspace of %zu bytes needed, %zu given", row_flag_bytes(B),
+                        workspace_bytes);
+        ChunkFwdArgs c{};
+        c.x = x; c.f = f; c.q = q; c.k = k; c.f_key = f_key; c.s0 = s0;
+        c.out = out; c.next_state = next_state; c.ckpt = ckpt;
+        c.row_flags = static_cast<int32_t *>(workspace);
+        c.B = B; c.T = T; c.NC = a.NC; c.C = a.C;
+        const int op = (dtype == T2FW_F16 && (flags & T2FW_FLAG_FP16_OPERANDS)) ? 1 : 0;
+        if ((rc = chunk_forward(c, dtype, op, st))) return rc;
+        a.row_select = c.row_flags;      // rows the chunked form could not take
+    }
     return scan_forward(a, dtype, st);
 }
 
@@ -127,7 +157,7 @@ int t2fw_lfw_backward(const void *g_out, const void *g_state, const void *x, con
                       void *d_f, void *d_q, void *d_k, void *d_f_key, void *d_s0, int64_t B, int64_t T,
                       int64_t D, int64_t K, int32_t C, int32_t dtype, int32_t flags, void *workspace,
                       size_t workspace_bytes, void *stream) {
-    (void)workspace; (void)workspace_bytes; (void)flags; (void)s0;
+    (void)s0;
     const size_t es = elem_size(dtype);
     if (es == 0) return fail(T2FW_ERR_BAD_DTYPE, "unknown dtype code %d", dtype);
     int rc = check_dims(B, T, D, K);
@@ -156,6 +186,21 @@ int t2fw_lfw_backward(const void *g_out, const void *g_state, const void *x, con
     a.row_select = nullptr;
     a.B = B; a.T = T; a.D = D; a.K = K; a.C = C;
     a.NC = t2fw_lfw_num_ckpt(T, C);
+
+    if (chunk_shape_ok(D, K, dtype, flags) && (C == 32 || C == 64) &&
+        aligned16({g_out, g_state, x, f, q, k, f_key, ckpt, d_x, d_f, d_q, d_k, d_f_key, d_s0})) {
+        if (workspace == nullptr || workspace_bytes < row_flag_bytes(B))
+            return fail(T2FW_ERR_WORKSPACE, "workspace of %zu bytes needed, %zu given", row_flag_bytes(B),
+                        workspace_bytes);
+        ChunkBwdArgs c{};
+        c.g_out = g_out; c.g_state = g_state; c.x = x; c.f = f; c.q = q; c.k = k; c.f_key = f_key; c.ckpt = ckpt;
+        c.d_x = d_x; c.d_f = d_f; c.d_q = d_q; c.d_k = d_k; c.d_f_key = d_f_key; c.d_s0 = d_s0;
+        c.row_flags = static_cast<int32_t *>(workspace);
+        c.B = B; c.T = T; c.NC = a.NC; c.C = C;
+        const int op = (dtype == T2FW_F16 && (flags & T2FW_FLAG_FP16_OPERANDS)) ? 1 : 0;
+        if ((rc = chunk_backward(c, dtype, op, st))) return rc;
+        a.row_select = c.row_flags;      // rows the chunked form could not take
+    }
     return scan_backward(a, dtype, st);
 }
 

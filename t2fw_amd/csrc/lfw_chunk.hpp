@@ -1,0 +1,137 @@
+// Chunked (matrix-core) form of the decay-rule recurrence for D = K = 64, 16-bit I/O.
+//
+// The rank-1-separable gate lets a block of L = 16 steps be written as small dense
+// contractions.  With a_t[d] = prod_{r<=t} f_r[d], b_t[k] = prod_{r<=t} fkey_r[k] (products
+// from the block start), suffix products ca_t = a_L/a_t, cb_t = b_L/b_t and
+//   qs_t = q_t*b_t,  kh_t = k_t*cb_t,  kt_t = kh_t/b_L (= k_t/b_t),
+//   xh_t = x_t*ca_t, xt_t = xh_t/a_L (= x_t/a_t),  gs_t = g_t*a_t
+// the block is
+//   P[t,s]  = qs_t . kt_s                       (t >= s)
+//   o_t     = a_t * ( S0 qs_t + sum_{s<=t} P[t,s] xt_s )
+//   S_L     = (a_L (x) b_L) * S0 + sum_s xh_s (x) kh_s
+// Only the intra-block terms use an inverse (1/b_L, 1/a_L over 16 steps); everything that
+// crosses block boundaries is scaled by factors <= 1, so the form holds for any gates in
+// (0, 1] whose 16-step products stay above 2^-100.  Rows that violate this (or have gates
+// outside (0, 1]) are flagged and recomputed by the exact scan kernels.
+//
+// All contractions run on MFMA with 16-bit operands (type OP) and fp32 accumulation; the
+// state itself is carried in fp32 accumulator registers for the whole sequence.
+#pragma once
+
+#include "common.hpp"
+
+namespace t2fw {
+
+struct ChunkFwdArgs {
+    const void *x, *f, *q, *k, *f_key, *s0;
+    void *out, *next_state, *ckpt;     // ckpt may be null
+    int32_t *row_flags;                // [B]: set to 1 for rows the exact kernels must redo
+    int64_t B, T, NC;
+    int32_t C;                         // checkpoint interval, multiple of 32
+};
+
+struct ChunkBwdArgs {
+    const void *g_out, *g_state, *x, *f, *q, *k, *f_key, *ckpt;
+    void *d_x, *d_f, *d_q, *d_k, *d_f_key, *d_s0;
+    int32_t *row_flags;
+    int64_t B, T, NC;
+    int32_t C;
+};
+
+// op: 0 = bf16 operands, 1 = fp16 operands (fp16 I/O only)
+int chunk_forward(const ChunkFwdArgs &a, int dtype, int op, hipStream_t stream);
+int chunk_backward(const ChunkBwdArgs &a, int dtype, int op, hipStream_t stream);
+
+#if defined(__HIPCC__)
+
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+typedef float floatx2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x4_t __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x2_t __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x4_t __attribute__((ext_vector_type(4)));
+typedef _Float16 f16x8_t __attribute__((ext_vector_type(8)));
+typedef short short4_t __attribute__((ext_vector_type(4)));
+typedef unsigned short u16;
+typedef unsigned int u32;
+
+// The register allocator may place an MFMA's destination on top of its A or B source
+// registers (it only forbids that for results wider than four registers).  On gfx950 the
+// 16x16 forms then return wrong values in the overlapped result elements, so the wrappers
+// below keep A and B alive past the instruction: the empty asm reads them together with the
+// result, which forces three distinct register ranges and emits nothing.
+typedef unsigned int u32x4_t __attribute__((ext_vector_type(4)));
+typedef unsigned int u32x2_t __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ void mfma_keep_sources(floatx4 &d, const uint4 &a, const uint4 &b) {
+    const u32x4_t av = {a.x, a.y, a.z, a.w}, bv = {b.x, b.y, b.z, b.w};
+    asm("" : "+v"(d) : "v"(av), "v"(bv));
+}
+__device__ __forceinline__ void mfma_keep_sources(floatx4 &d, const uint2 &a, const uint2 &b) {
+    const u32x2_t av = {a.x, a.y}, bv = {b.x, b.y};
+    asm("" : "+v"(d) : "v"(av), "v"(bv));
+}
+#define T2FW_MFMA_KEEP_SOURCES(d, a, b)
+
+// 16-bit element types as raw bits + conversions ---------------------------------------
+struct Bf16 {
+    static constexpr u16 ONE_BITS = 0x3F80;
+    // smallest 16-step gate product accepted with operands of this type: the inverse
+    // 1/product scales the intra-block operands and must stay far from overflow
+    static constexpr float MIN_PRODUCT = 7.8886090522101181e-31f;   // 2^-100
+    static __device__ __forceinline__ float to_f32(u16 v) { return __uint_as_float((u32)v << 16); }
+    static __device__ __forceinline__ u32 pack2(float lo, float hi) {
+        floatx2 v = {lo, hi};
+        return __builtin_bit_cast(u32, __builtin_convertvector(v, bf16x2_t));
+    }
+    static __device__ __forceinline__ floatx4 mfma32(uint4 a, uint4 b, floatx4 c) {
+        floatx4 d = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a),
+                                                            __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
+        T2FW_MFMA_KEEP_SOURCES(d, a, b);
+        return d;
+    }
+    static __device__ __forceinline__ floatx4 mfma16(uint2 a, uint2 b, floatx4 c) {
+        floatx4 d = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(short4_t, a),
+                                                              __builtin_bit_cast(short4_t, b), c, 0, 0, 0);
+        T2FW_MFMA_KEEP_SOURCES(d, a, b);
+        return d;
+    }
+};
+
+struct Fp16 {
+    static constexpr u16 ONE_BITS = 0x3C00;
+    static constexpr float MIN_PRODUCT = 0.00390625f;               // 2^-8
+    static __device__ __forceinline__ float to_f32(u16 v) { return (float)__builtin_bit_cast(_Float16, v); }
+    static __device__ __forceinline__ u32 pack2(float lo, float hi) {
+        floatx2 v = {lo, hi};
+        return __builtin_bit_cast(u32, __builtin_convertvector(v, f16x2_t));
+    }
+    static __device__ __forceinline__ floatx4 mfma32(uint4 a, uint4 b, floatx4 c) {
+        floatx4 d = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8_t, a),
+                                                           __builtin_bit_cast(f16x8_t, b), c, 0, 0, 0);
+        T2FW_MFMA_KEEP_SOURCES(d, a, b);
+        return d;
+    }
+    static __device__ __forceinline__ floatx4 mfma16(uint2 a, uint2 b, floatx4 c) {
+        floatx4 d = __builtin_amdgcn_mfma_f32_16x16x16f16(__builtin_bit_cast(f16x4_t, a),
+                                                          __builtin_bit_cast(f16x4_t, b), c, 0, 0, 0);
+        T2FW_MFMA_KEEP_SOURCES(d, a, b);
+        return d;
+    }
+};
+
+template <typename E> __device__ __forceinline__ u16 cvt1(float v) { return (u16)(E::pack2(v, 0.f) & 0xffffu); }
+
+constexpr int CH_THREADS = 256;
+constexpr int CH_L = 16;        // block length
+constexpr int CH_STEP = 32;     // tokens prepared per iteration (two blocks)
+constexpr int CH_N = 64;        // D = K = 64
+
+// LDS strides (in elements) chosen so the MFMA operand reads are bank-conflict free
+constexpr int TS = 72;          // token-major tiles [32 tokens][64 ch] of 16-bit: row stride
+constexpr int CS = 36;          // channel-major tiles [64 ch][32 tokens] of 16-bit / fp32: row stride
+constexpr int OS = 68;          // output tile [32 tokens][64 ch] of 16-bit: row stride
+
+#endif  // __HIPCC__
+
+}  // namespace t2fw

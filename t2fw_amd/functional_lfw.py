@@ -23,6 +23,13 @@ def _ckpt_interval():
     return int(v) if v else DEFAULT_CKPT_INTERVAL
 
 
+def _flags():
+    """Kernel-path flags (include/t2fw_hip.h): 0 = automatic, 1 = exact scan kernels only,
+    2 = fp16 matrix-core operands for fp16 tensors.  Overridable with T2FW_FLAGS."""
+    v = os.environ.get("T2FW_FLAGS")
+    return int(v) if v else _lib.FLAG_AUTO
+
+
 def _check_input(t, name):
     # mirrors CHECK_INPUT of t2fw/csrc/lfw.cpp:24-26 (TORCH_CHECK -> RuntimeError)
     if not t.is_cuda:
@@ -68,6 +75,7 @@ class LFWFunction(torch.autograd.Function):
         lib = _lib.load()
         need_grad = any(ctx.needs_input_grad)
         C = _ckpt_interval()
+        flags = _flags()
         dev = value.device
         with torch.cuda.device(dev):
             outputs = torch.empty_like(value)
@@ -76,16 +84,17 @@ class LFWFunction(torch.autograd.Function):
             if need_grad:
                 nc = lib.t2fw_lfw_num_ckpt(T, C)
                 ckpt = torch.empty((B, nc, D, K), dtype=value.dtype, device=dev)
-            ws_bytes = lib.t2fw_lfw_workspace_bytes(B, T, D, K, C, code, _lib.FLAG_AUTO)
+            ws_bytes = lib.t2fw_lfw_workspace_bytes(B, T, D, K, C, code, flags)
             ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev) if ws_bytes else None
             _lib.check(lib.t2fw_lfw_forward(
                 _lib.ptr(value), _lib.ptr(forget), _lib.ptr(query), _lib.ptr(key), _lib.ptr(f_key),
                 _lib.ptr(state), _lib.ptr(outputs), _lib.ptr(next_state), _lib.ptr(ckpt),
-                B, T, D, K, C, code, _lib.FLAG_AUTO, _lib.ptr(ws), ws_bytes,
+                B, T, D, K, C, code, flags, _lib.ptr(ws), ws_bytes,
                 _lib.current_stream_handle(dev)))
         if need_grad:
             ctx.save_for_backward(value, forget, query, key, f_key, state, ckpt)
             ctx.ckpt_interval = C
+            ctx.flags = flags
         return outputs, next_state
 
     @staticmethod
@@ -101,6 +110,7 @@ class LFWFunction(torch.autograd.Function):
         code = _dtype_code(value.dtype)
         lib = _lib.load()
         C = ctx.ckpt_interval
+        flags = ctx.flags
         dev = value.device
         with torch.cuda.device(dev):
             d_x = torch.empty_like(value)
@@ -109,13 +119,13 @@ class LFWFunction(torch.autograd.Function):
             d_k = torch.empty_like(key)
             d_fk = torch.empty_like(f_key)
             d_s = torch.empty_like(state)
-            ws_bytes = lib.t2fw_lfw_workspace_bytes(B, T, D, K, C, code, _lib.FLAG_AUTO)
+            ws_bytes = lib.t2fw_lfw_workspace_bytes(B, T, D, K, C, code, flags)
             ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev) if ws_bytes else None
             _lib.check(lib.t2fw_lfw_backward(
                 _lib.ptr(grad_output), _lib.ptr(grad_state), _lib.ptr(value), _lib.ptr(forget),
                 _lib.ptr(query), _lib.ptr(key), _lib.ptr(f_key), _lib.ptr(state), _lib.ptr(ckpt),
                 _lib.ptr(d_x), _lib.ptr(d_f), _lib.ptr(d_q), _lib.ptr(d_k), _lib.ptr(d_fk), _lib.ptr(d_s),
-                B, T, D, K, C, code, _lib.FLAG_AUTO, _lib.ptr(ws), ws_bytes,
+                B, T, D, K, C, code, flags, _lib.ptr(ws), ws_bytes,
                 _lib.current_stream_handle(dev)))
         # order of t2fw/csrc/lfw.cpp:95
         return d_x, d_f, d_q, d_k, d_fk, d_s

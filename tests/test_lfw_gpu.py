@@ -15,24 +15,47 @@ from tests.lfw_cases import (err_stats, make_config_inputs, make_reference_test_
 
 pytestmark = pytest.mark.gpu
 
-# stated tolerances per dtype: |got-ref| <= rtol*|ref| + afrac*max|ref|
+# Stated tolerances: |got-ref| <= rtol*|ref| + afrac*max|ref|.
+# Exact scan kernels (fp32 state, result rounded once to the I/O dtype):
 TOL = {
     torch.float16: (2e-3, 1e-3),
     torch.bfloat16: (1.6e-2, 8e-3),
     torch.float32: (2e-5, 2e-5),
     torch.float64: (1e-12, 1e-12),
 }
+# Chunked matrix-core kernels (D = K = 64, 16-bit tensors): operands of the contractions are
+# rounded to bf16 (2^-9 relative), accumulation is fp32.  The gate gradients are differences
+# of products of such quantities and carry a wider bound.
+TOL_CHUNK = (2e-2, 1e-2)
+TOL_CHUNK_GATE = (4e-2, 4e-2)
 
 
-def assert_close(got, ref, dtype, what, scale=1.0):
-    rtol, afrac = TOL[dtype]
+def on_chunk_path(dtype, D, K):
+    import os
+    return D == 64 and K == 64 and dtype in (torch.float16, torch.bfloat16) and \
+        not (int(os.environ.get("T2FW_FLAGS", "0")) & 1)
+
+
+def gate_grad_floor(inputs, go, r_out, r_grads):
+    """Natural magnitude of the terms whose difference forms f*d_f and fkey*d_fkey
+    (g.o - x.dx and q.dq - k.dk): the absolute error of the chunked kernels scales with
+    these, also where the exact gradient happens to vanish (e.g. a zero initial state)."""
+    x, f, q, k, fk, s = [t.double() for t in inputs]
+    d_x, d_f, d_q, d_k, d_fk, d_s = [torch.as_tensor(t).double() for t in r_grads]
+    fl_f = float(((go.double() * torch.as_tensor(r_out).double()).abs() + (x * d_x).abs()).max()) if x.numel() else 0.0
+    fl_k = float(((q * d_q).abs() + (k * d_k).abs()).max()) if q.numel() else 0.0
+    return {"d_f": fl_f, "d_f_key": fl_k}
+
+
+def assert_close(got, ref, dtype, what, scale=1.0, tol=None, floor=0.0):
+    rtol, afrac = tol if tol is not None else TOL[dtype]
     got = got.detach().double().cpu()
     ref = torch.as_tensor(ref).double()
     assert got.shape == ref.shape, (what, got.shape, ref.shape)
     if ref.numel() == 0:
         return
     assert torch.isfinite(got).all(), what + " has non-finite values"
-    bound = scale * (rtol * ref.abs() + afrac * ref.abs().max())
+    bound = scale * (rtol * ref.abs() + afrac * max(float(ref.abs().max()), floor))
     bad = (got - ref).abs() > bound
     assert not bad.any(), "%s: %d/%d outside tolerance, max-abs err %.3e (max|ref| %.3e)" % (
         what, int(bad.sum()), ref.numel(), float((got - ref).abs().max()), float(ref.abs().max()))
@@ -62,11 +85,15 @@ def check_all(inputs, go, gs, dtype, scale=1.0):
     out, nxt, grads = run_autograd(inputs, go, gs)
     r_out, r_nxt, r_grads = oracle_all(inputs, go, gs)
     assert out.dtype == dtype and nxt.dtype == dtype
-    assert_close(out, r_out, dtype, "outputs", scale)
-    assert_close(nxt, r_nxt, dtype, "next_state", scale)
+    chunk = on_chunk_path(dtype, inputs[0].shape[2], inputs[2].shape[2])
+    tol = TOL_CHUNK if chunk else None
+    floors = gate_grad_floor(inputs, go, r_out, r_grads) if chunk else {}
+    assert_close(out, r_out, dtype, "outputs", scale, tol)
+    assert_close(nxt, r_nxt, dtype, "next_state", scale, tol)
     for n, g, r in zip(NAMES, grads, r_grads):
         assert g.dtype == dtype
-        assert_close(g, r, dtype, n, scale)
+        assert_close(g, r, dtype, n, scale, (TOL_CHUNK_GATE if n in ("d_f", "d_f_key") else TOL_CHUNK) if chunk else None,
+                     floors.get(n, 0.0))
     # outer bound: the reference's own tolerances (tests/test_lfw.py:65,92)
     if dtype == torch.float16:
         assert torch.allclose(out.double().cpu(), torch.as_tensor(r_out), atol=1e-2, rtol=1e-1)
@@ -105,6 +132,14 @@ def test_checkpoint_interval_any_value(C, monkeypatch):
     x, f, q, k, fk, s, go, gs = make_config_inputs(2, 150, 64, 64, torch.float16, seed=9,
                                                     gate_mean=2.0, state_std=0.3)
     check_all((x, f, q, k, fk, s), go, gs, torch.float16)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_scan_kernels_at_the_matrix_core_shape(dtype, monkeypatch):
+    # D = K = 64 through the exact scan kernels only (the row-level fallback of the chunked path)
+    monkeypatch.setenv("T2FW_FLAGS", "1")
+    x, f, q, k, fk, s, go, gs = make_config_inputs(3, 200, 64, 64, dtype, seed=12, state_std=0.3)
+    check_all((x, f, q, k, fk, s), go, gs, dtype)
 
 
 def test_checkpoints_hold_chunk_start_states():
