@@ -56,23 +56,13 @@ typedef short short4_t __attribute__((ext_vector_type(4)));
 typedef unsigned short u16;
 typedef unsigned int u32;
 
-// The register allocator may place an MFMA's destination on top of its A or B source
-// registers (it only forbids that for results wider than four registers).  On gfx950 the
-// 16x16 forms then return wrong values in the overlapped result elements, so the wrappers
-// below keep A and B alive past the instruction: the empty asm reads them together with the
-// result, which forces three distinct register ranges and emits nothing.
-typedef unsigned int u32x4_t __attribute__((ext_vector_type(4)));
-typedef unsigned int u32x2_t __attribute__((ext_vector_type(2)));
-__device__ __forceinline__ void mfma_keep_sources(floatx4 &d, const uint4 &a, const uint4 &b) {
-    const u32x4_t av = {a.x, a.y, a.z, a.w}, bv = {b.x, b.y, b.z, b.w};
-    asm("" : "+v"(d) : "v"(av), "v"(bv));
-}
-__device__ __forceinline__ void mfma_keep_sources(floatx4 &d, const uint2 &a, const uint2 &b) {
-    const u32x2_t av = {a.x, a.y}, bv = {b.x, b.y};
-    asm("" : "+v"(d) : "v"(av), "v"(bv));
-}
-#define T2FW_MFMA_KEEP_SOURCES(d, a, b)
-
+// MFMA chaining rule used by the kernels: an accumulator is only ever chained (result fed back
+// as the C operand) through MFMAs of the SAME form.  The result of a 16x16x32 chain and the
+// result of a 16x16x16 product are combined with VALU adds, never by feeding one form's
+// result straight into the other form's C operand: with only three instructions between a
+// 16x16x32 and a dependent 16x16x16 the latter was observed to read a partly written C on
+// gfx950 (two of the four result elements wrong); VALU reads of MFMA results are interlocked
+// by the compiler's wait states.
 // 16-bit element types as raw bits + conversions ---------------------------------------
 struct Bf16 {
     static constexpr u16 ONE_BITS = 0x3F80;
@@ -85,16 +75,12 @@ struct Bf16 {
         return __builtin_bit_cast(u32, __builtin_convertvector(v, bf16x2_t));
     }
     static __device__ __forceinline__ floatx4 mfma32(uint4 a, uint4 b, floatx4 c) {
-        floatx4 d = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a),
+        return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a),
                                                             __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
-        T2FW_MFMA_KEEP_SOURCES(d, a, b);
-        return d;
     }
     static __device__ __forceinline__ floatx4 mfma16(uint2 a, uint2 b, floatx4 c) {
-        floatx4 d = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(short4_t, a),
+        return __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(short4_t, a),
                                                               __builtin_bit_cast(short4_t, b), c, 0, 0, 0);
-        T2FW_MFMA_KEEP_SOURCES(d, a, b);
-        return d;
     }
 };
 
@@ -107,16 +93,12 @@ struct Fp16 {
         return __builtin_bit_cast(u32, __builtin_convertvector(v, f16x2_t));
     }
     static __device__ __forceinline__ floatx4 mfma32(uint4 a, uint4 b, floatx4 c) {
-        floatx4 d = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8_t, a),
+        return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8_t, a),
                                                            __builtin_bit_cast(f16x8_t, b), c, 0, 0, 0);
-        T2FW_MFMA_KEEP_SOURCES(d, a, b);
-        return d;
     }
     static __device__ __forceinline__ floatx4 mfma16(uint2 a, uint2 b, floatx4 c) {
-        floatx4 d = __builtin_amdgcn_mfma_f32_16x16x16f16(__builtin_bit_cast(f16x4_t, a),
+        return __builtin_amdgcn_mfma_f32_16x16x16f16(__builtin_bit_cast(f16x4_t, a),
                                                           __builtin_bit_cast(f16x4_t, b), c, 0, 0, 0);
-        T2FW_MFMA_KEEP_SOURCES(d, a, b);
-        return d;
     }
 };
 

@@ -485,10 +485,10 @@ __device__ __forceinline__ void bwd_matrix_waves(const ChunkBwdArgs &p, unsigned
                 // o' and dq' use the block-start state
                 floatx4 oa = OPE::mfma32(cat(ld2(QT + po), ld2(QT + po + 16)), cat(svd[i][0], svd[i][1]), zero);
                 oa = OPE::mfma32(cat(ld2(QT + po + 32), ld2(QT + po + 48)), cat(svd[i][2], svd[i][3]), oa);
-                oa = OPE::mfma16(pa_o, xtc, oa);
+                oa += OPE::mfma16(pa_o, xtc, zero);
                 floatx4 dqa = OPE::mfma32(cat(ld2(GT + po), ld2(GT + po + 16)), cat(svk[i][0], svk[i][1]), zero);
                 dqa = OPE::mfma32(cat(ld2(GT + po + 32), ld2(GT + po + 48)), cat(svk[i][2], svk[i][3]), dqa);
-                dqa = OPE::mfma16(pa_q, ktc, dqa);
+                dqa += OPE::mfma16(pa_q, ktc, zero);
                 // dx' and dk' use the adjoint entering the block, scaled to the block end on one side
                 floatx4 ga[4], gb[4];
                 uint2 gap[4], gbp[4];
@@ -501,10 +501,10 @@ __device__ __forceinline__ void bwd_matrix_waves(const ChunkBwdArgs &p, unsigned
                 }
                 floatx4 dxa = OPE::mfma32(cat(ld2(KH + po), ld2(KH + po + 16)), cat(gap[0], gap[1]), zero);
                 dxa = OPE::mfma32(cat(ld2(KH + po + 32), ld2(KH + po + 48)), cat(gap[2], gap[3]), dxa);
-                dxa = OPE::mfma16(pa_x, gtc, dxa);
+                dxa += OPE::mfma16(pa_x, gtc, zero);
                 floatx4 dka = OPE::mfma32(cat(ld2(XH + po), ld2(XH + po + 16)), cat(gbp[0], gbp[1]), zero);
                 dka = OPE::mfma32(cat(ld2(XH + po + 32), ld2(XH + po + 48)), cat(gbp[2], gbp[3]), dka);
-                dka = OPE::mfma16(pa_k, qtc, dka);
+                dka += OPE::mfma16(pa_k, qtc, zero);
                 // adjoint of the previous block: Gb <- (a_L (x) b_L) * Gb + sum_t gs_t (x) qs_t
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {

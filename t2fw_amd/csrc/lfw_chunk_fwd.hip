@@ -287,12 +287,13 @@ __device__ __forceinline__ void fwd_matrix_waves(const ChunkFwdArgs &p, unsigned
             floatx4 o = {0.f, 0.f, 0.f, 0.f};
             o = OPE::mfma32(make_uint4(q0.x, q0.y, q1.x, q1.y), make_uint4(s0p.x, s0p.y, s1p.x, s1p.y), o);
             o = OPE::mfma32(make_uint4(q2.x, q2.y, q3.x, q3.y), make_uint4(s2p.x, s2p.y, s3p.x, s3p.y), o);
-            o = OPE::mfma16(pa, *reinterpret_cast<const uint2 *>(XT + d * CS + tok0 + 4 * g), o);
+            const floatx4 zero = {0.f, 0.f, 0.f, 0.f};
+            const floatx4 oi = OPE::mfma16(pa, *reinterpret_cast<const uint2 *>(XT + d * CS + tok0 + 4 * g), zero);
             const float4 as = *reinterpret_cast<const float4 *>(AS + d * CS + tok0 + 4 * g);
-            OUT[(tok0 + 4 * g + 0) * OS + d] = cvt1<IOE>(o[0] * as.x);
-            OUT[(tok0 + 4 * g + 1) * OS + d] = cvt1<IOE>(o[1] * as.y);
-            OUT[(tok0 + 4 * g + 2) * OS + d] = cvt1<IOE>(o[2] * as.z);
-            OUT[(tok0 + 4 * g + 3) * OS + d] = cvt1<IOE>(o[3] * as.w);
+            OUT[(tok0 + 4 * g + 0) * OS + d] = cvt1<IOE>((o[0] + oi[0]) * as.x);
+            OUT[(tok0 + 4 * g + 1) * OS + d] = cvt1<IOE>((o[1] + oi[1]) * as.y);
+            OUT[(tok0 + 4 * g + 2) * OS + d] = cvt1<IOE>((o[2] + oi[2]) * as.z);
+            OUT[(tok0 + 4 * g + 3) * OS + d] = cvt1<IOE>((o[3] + oi[3]) * as.w);
             // S_L = (a_L (x) b_L) * S0 + sum_s xh_s (x) kh_s
             const float aL = AL[hh * CH_N + d];
             const uint2 xh = *reinterpret_cast<const uint2 *>(XH + d * CS + tok0 + 4 * g);
