@@ -28,6 +28,18 @@
 // (t2fw/csrc/lfw_kernel.cu:61-102, t2fw/csrc/lfw.cpp:84-93).
 #include "lfw_chunk.hpp"
 
+// Build-time diagnostic (-DT2FW_PHASE_TIMERS): workgroup 0 accumulates shader-clock ticks
+// per phase into row_flags[64..]; off in the shipped library.
+#ifdef T2FW_PHASE_TIMERS
+#define PHASE_BEGIN() unsigned long long ph_t = __builtin_amdgcn_s_memtime(); unsigned long long ph_acc[4] = {0, 0, 0, 0}
+#define PHASE_MARK(i) { const unsigned long long ph_n = __builtin_amdgcn_s_memtime(); ph_acc[i] += ph_n - ph_t; ph_t = ph_n; }
+#define PHASE_END(slot) if (b == 0 && (tid & 63) == 0) { for (int ph_i = 0; ph_i < 4; ++ph_i) p.row_flags[64 + (slot) * 8 + ph_i * 2] = (int)(ph_acc[ph_i] & 0x7fffffff); }
+#else
+#define PHASE_BEGIN()
+#define PHASE_MARK(i)
+#define PHASE_END(slot)
+#endif
+
 namespace t2fw {
 namespace {
 
@@ -61,37 +73,35 @@ static_assert(BWD_SMEM <= 160 * 1024, "backward stage buffers exceed the LDS of 
 // Chunks are visited from the last one down; a chunk with nb blocks takes nb "R" stages
 // (blocks 0..nb-1) followed by nb "B" stages (blocks nb-1..0).
 struct StageInfo {
-    int64_t chunk;
+    int chunk;
     int block;      // block inside the chunk
     bool bmode;     // false: recompute sweep, true: backward sweep
-    bool valid;
 };
 
+// 32-bit arithmetic only; NB is a power of two, so the divisions are shifts.
 template <int NB> struct Schedule {
-    int64_t NC, total;
-    int nb_last;
-    __device__ Schedule(int64_t T, int64_t NC_, int C) : NC(NC_) {
-        const int64_t len_last = T - (NC_ - 1) * C;
-        nb_last = (int)((len_last + CH_L - 1) / CH_L);
-        total = 2 * nb_last + (NC_ - 1) * 2 * NB;
+    int NC, total, nb_last;
+    __device__ Schedule(int64_t T, int64_t NC_, int C) {
+        NC = (int)NC_;
+        const int len_last = (int)(T - (NC_ - 1) * C);
+        nb_last = (len_last + CH_L - 1) / CH_L;
+        total = 2 * nb_last + (NC - 1) * 2 * NB;
     }
-    __device__ StageInfo at(int64_t s) const {
+    __device__ StageInfo at(int s) const {
         StageInfo r;
-        r.valid = s >= 0 && s < total;
-        int64_t local;
-        int nb;
+        int local, nb;
         if (s < 2 * nb_last) {
             r.chunk = NC - 1;
             local = s;
             nb = nb_last;
         } else {
-            const int64_t s2 = s - 2 * nb_last;
-            r.chunk = NC - 2 - s2 / (2 * NB);
-            local = s2 % (2 * NB);
+            const unsigned s2 = (unsigned)(s - 2 * nb_last);
+            r.chunk = NC - 2 - (int)(s2 / (2u * NB));
+            local = (int)(s2 % (2u * NB));
             nb = NB;
         }
         r.bmode = local >= nb;
-        r.block = r.bmode ? (int)(2 * nb - 1 - local) : (int)local;
+        r.block = r.bmode ? 2 * nb - 1 - local : local;
         return r;
     }
 };
@@ -245,10 +255,10 @@ __device__ __forceinline__ void bwd_prep_waves(const ChunkBwdArgs &p, unsigned c
                              reinterpret_cast<u16 *>(p.d_q), reinterpret_cast<u16 *>(p.d_k),
                              reinterpret_cast<u16 *>(p.d_f_key)};
     const Schedule<NB> sched(T, p.NC, p.C);
-    const int64_t total = sched.total;
+    const int total = sched.total;
     u32 bad = 0;
     if (tid == 0) p.row_flags[b] = 0;
-    auto tok0_of = [&](const StageInfo &si) -> int64_t { return si.chunk * p.C + (int64_t)si.block * CH_L; };
+    auto tok0_of = [&](const StageInfo &si) -> int64_t { return (int64_t)si.chunk * p.C + si.block * CH_L; };
 
     // raw inputs of stage m live in RAW[m & 1]; `st` carries the next stage to be written
     BStage st;
@@ -270,7 +280,7 @@ __device__ __forceinline__ void bwd_prep_waves(const ChunkBwdArgs &p, unsigned c
         __syncthreads();
     }
 
-    auto store_out = [&](int64_t s) {       // gradients of B stage s: LDS tiles -> global, 16 B pieces
+    auto store_out = [&](int s) {       // gradients of B stage s: LDS tiles -> global, 16 B pieces
         const StageInfo si = sched.at(s);
         if (!si.bmode) return;
         const unsigned char *outp = smem + BOFF_OUT + (s & 1) * BOUT_BYTES;
@@ -289,20 +299,28 @@ __device__ __forceinline__ void bwd_prep_waves(const ChunkBwdArgs &p, unsigned c
         }
     };
 
-    for (int64_t s = 0; s < total; ++s) {
-        if (s > 0) store_out(s - 1);
+    PHASE_BEGIN();
+    for (int s = 0; s < total; ++s) {
+        // consume last iteration's loads first (everything still in flight is at least most of an
+        // iteration old), then issue this iteration's stores, then the next loads
         if (s + 2 < total) bstage_store(st, smem + BOFF_RAW + (s & 1) * BRAW_BYTES, sched.at(s + 2).bmode, tid);
+        PHASE_MARK(1);
+        if (s > 0) store_out(s - 1);
         if (s + 3 < total) {
             const StageInfo s3 = sched.at(s + 3);
             bstage_load<IOE>(st, src, row_base, T, tok0_of(s3), s3.bmode, tid);
         }
+        PHASE_MARK(0);
         if (s + 1 < total)
             bwd_prep<IOE, OPE>(smem + BOFF_RAW + ((s + 1) & 1) * BRAW_BYTES, smem + ((s + 1) & 1) * STAGE_BYTES, role, c,
                                sched.at(s + 1).bmode, bad);
+        PHASE_MARK(2);
         __syncthreads();
+        PHASE_MARK(3);
     }
     store_out(total - 1);
     if (bad) p.row_flags[b] = 1;
+    PHASE_END(4 + (tid >> 6));
 }
 
 // helpers of the matrix waves ----------------------------------------------------------------
@@ -392,6 +410,7 @@ __device__ __forceinline__ void bwd_matrix_waves(const ChunkBwdArgs &p, unsigned
     int64_t s = 0;
     __syncthreads();      // raw inputs of the first stages are in LDS
     __syncthreads();      // operand tiles of stage 0 are in LDS
+    PHASE_BEGIN();
 
     for (int64_t chunk = NC - 1; chunk >= 0; --chunk) {
         const int nb = chunk == NC - 1 ? nb_last : NB;
@@ -421,7 +440,9 @@ __device__ __forceinline__ void bwd_matrix_waves(const ChunkBwdArgs &p, unsigned
                     Sd[j] = OPE::mfma16(ld2(KHc + (16 * j + r) * CC + 4 * g), xh_d, Sd[j]);
                     Sk[j] = OPE::mfma16(ld2(XHc + (16 * j + r) * CC + 4 * g), kh_k, Sk[j]);
                 }
+                PHASE_MARK(0);
                 __syncthreads();
+                PHASE_MARK(3);
                 ++s;
             }
         }
@@ -554,7 +575,9 @@ __device__ __forceinline__ void bwd_matrix_waves(const ChunkBwdArgs &p, unsigned
                         DFK[(4 * g + ii) * OS + ch] = cvt1<IOE>(dv[ii] * rkv[ii]);
                     }
                 }
+                PHASE_MARK(1);
                 __syncthreads();
+                PHASE_MARK(2);
                 ++s;
             }
         }
@@ -565,6 +588,7 @@ __device__ __forceinline__ void bwd_matrix_waves(const ChunkBwdArgs &p, unsigned
 #pragma unroll
         for (int j = 0; j < 4; ++j) *reinterpret_cast<uint2 *>(ds + ch * CH_N + 16 * j + 4 * g) = pack4v<IOE>(Gd[j]);
     }
+    PHASE_END(tid >> 6);
 }
 
 template <typename IOE, typename OPE, int NB>
