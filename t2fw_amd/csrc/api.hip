@@ -3,6 +3,7 @@
 #include "common.hpp"
 #include "lfw_scan.hpp"
 #include "lfw_chunk.hpp"
+#include "dfw_scan.hpp"
 
 #include <cstring>
 #include <initializer_list>
@@ -210,14 +211,59 @@ int t2fw_lfw_step(const void *x, const void *f, const void *q, const void *k, co
                             T2FW_FLAG_AUTO, nullptr, 0, stream);
 }
 
-int t2fw_dfw_forward(const void *, const void *, const void *, const void *, void *, void *, void *, int64_t,
-                     int64_t, int64_t, int64_t, int32_t, void *) {
-    return fail(T2FW_ERR_UNSUPPORTED, "delta-rule forward is not built yet");
+int t2fw_dfw_forward(const void *q, const void *k, const void *v, const void *s0, void *out, void *final_state,
+                     void *delta, int64_t B, int64_t T, int64_t D, int64_t M, int32_t dtype, void *stream) {
+    const size_t es = elem_size(dtype);
+    if (es == 0) return fail(T2FW_ERR_BAD_DTYPE, "unknown dtype code %d", dtype);
+    int rc = check_dims(B, T, D, M);
+    if (rc) return rc;
+    if (B == 0) return T2FW_OK;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    {
+        const NamedPtr sp[] = {{"s0", s0}, {"final_state", final_state}};
+        if ((rc = check_ptrs(sp, 2, es))) return rc;
+    }
+    if (T == 0) {
+        if (final_state != s0)
+            return check_hip(hipMemcpyAsync(final_state, s0, (size_t)(B * D * M) * es, hipMemcpyDeviceToDevice, st),
+                             "state copy");
+        return T2FW_OK;
+    }
+    const NamedPtr ptrs[] = {{"q", q}, {"k", k}, {"v", v}, {"out", out}, {"delta", delta}};
+    if ((rc = check_ptrs(ptrs, 5, es))) return rc;
+    DfwFwdArgs a{};
+    a.q = q; a.k = k; a.v = v; a.s0 = s0; a.out = out; a.final_state = final_state; a.delta = delta;
+    a.B = B; a.T = T; a.D = D; a.M = M;
+    return dfw_forward(a, dtype, st);
 }
 
-int t2fw_dfw_backward(const void *, const void *, const void *, const void *, const void *, const void *, void *,
-                      void *, void *, void *, int64_t, int64_t, int64_t, int64_t, int32_t, void *) {
-    return fail(T2FW_ERR_UNSUPPORTED, "delta-rule backward is not built yet");
+int t2fw_dfw_backward(const void *g_out, const void *g_state, const void *q, const void *k, const void *delta,
+                      const void *final_state, void *d_q, void *d_k, void *d_v, void *d_s0, int64_t B, int64_t T,
+                      int64_t D, int64_t M, int32_t dtype, void *stream) {
+    const size_t es = elem_size(dtype);
+    if (es == 0) return fail(T2FW_ERR_BAD_DTYPE, "unknown dtype code %d", dtype);
+    int rc = check_dims(B, T, D, M);
+    if (rc) return rc;
+    if (B == 0) return T2FW_OK;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    {
+        const NamedPtr sp[] = {{"g_state", g_state}, {"d_s0", d_s0}};
+        if ((rc = check_ptrs(sp, 2, es))) return rc;
+    }
+    if (T == 0) {
+        if (d_s0 != g_state)
+            return check_hip(hipMemcpyAsync(d_s0, g_state, (size_t)(B * D * M) * es, hipMemcpyDeviceToDevice, st),
+                             "state-gradient copy");
+        return T2FW_OK;
+    }
+    const NamedPtr ptrs[] = {{"g_out", g_out}, {"q", q}, {"k", k}, {"delta", delta}, {"final_state", final_state},
+                             {"d_q", d_q}, {"d_k", d_k}, {"d_v", d_v}};
+    if ((rc = check_ptrs(ptrs, 8, es))) return rc;
+    DfwBwdArgs a{};
+    a.g_out = g_out; a.g_state = g_state; a.q = q; a.k = k; a.delta = delta; a.final_state = final_state;
+    a.d_q = d_q; a.d_k = d_k; a.d_v = d_v; a.d_s0 = d_s0;
+    a.B = B; a.T = T; a.D = D; a.M = M;
+    return dfw_backward(a, dtype, st);
 }
 
 }  // extern "C"

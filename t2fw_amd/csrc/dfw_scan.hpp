@@ -1,0 +1,25 @@
+// Argument blocks and host entry points of the delta-rule kernels (dfw_scan.hip).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <cstdint>
+
+namespace t2fw {
+
+struct DfwFwdArgs {
+    const void *q, *k, *v, *s0;
+    void *out, *final_state, *delta;
+    int64_t B, T, D, M;
+    int32_t kg, tb, ntiles;
+};
+
+struct DfwBwdArgs {
+    const void *g_out, *g_state, *q, *k, *delta, *final_state;
+    void *d_q, *d_k, *d_v, *d_s0;
+    int64_t B, T, D, M;
+    int32_t kg, tb, ntiles;
+};
+
+int dfw_forward(const DfwFwdArgs &a, int dtype, hipStream_t stream);
+int dfw_backward(const DfwBwdArgs &a, int dtype, hipStream_t stream);
+
+}  // namespace t2fw

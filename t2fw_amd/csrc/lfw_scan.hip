@@ -16,98 +16,13 @@
 // and t2fw/csrc/lfw.cpp:84-93 (backward).
 #include "common.hpp"
 #include "lfw_scan.hpp"
+#include "scan_tile.hpp"
 
 namespace t2fw {
 
 namespace {
 
-constexpr int PFC = 8;   // prefetch slots per thread per column-side array
-constexpr int PFR = 4;   // prefetch slots per thread per row-side array
-
-__device__ __forceinline__ int ilog2(int v) { return 31 - __clz(v); }
-
-// Geometry derived on the device from (kg, kpl): all powers of two.
-struct Tile {
-    int kg, rows, KP;        // lanes per row, rows per workgroup, padded columns
-    int CW, SP, lncc;        // column staging: lanes across columns, steps per pass, log2(KP/CW)
-    int SPR;                 // row staging: steps per pass
-    int r, kgi, k0;          // this lane's row, position in the row, first column
-    __device__ Tile(int kg_, int kpl) {
-        kg = kg_;
-        rows = SCAN_THREADS / kg;
-        KP = kg * kpl;
-        CW = KP < SCAN_THREADS ? KP : SCAN_THREADS;
-        SP = SCAN_THREADS / CW;
-        lncc = ilog2(KP / CW);
-        SPR = SCAN_THREADS / rows;
-        r = threadIdx.x / kg;
-        kgi = threadIdx.x % kg;
-        k0 = kgi * kpl;
-    }
-};
-
-// Prefetch registers for one time block: NCA column-side and NRA row-side arrays.
-template <typename IO, int NCA, int NRA> struct Prefetch {
-    IO c[NCA][PFC];
-    IO r[NRA][PFR];
-};
-
-// Issue the global loads of a block of n steps starting at step t0 of batch row b.
-// colp[a] are [B,T,ncols] arrays, rowp[a] are [B,T,nrows] arrays; this workgroup
-// needs all columns and rows [row0, row0 + rows).
-template <typename IO, int NCA, int NRA>
-__device__ __forceinline__ void block_load(Prefetch<IO, NCA, NRA> &pf, const Tile &g,
-                                           const IO *const (&colp)[NCA],
-                                           const IO *const (&rowp)[NRA],
-                                           int64_t b, int64_t T, int64_t t0, int n,
-                                           int64_t ncols, int64_t nrows, int64_t row0) {
-    const int csub = threadIdx.x % g.CW, tsub = threadIdx.x / g.CW;
-    const int64_t cbase = (b * T + t0) * ncols;
-#pragma unroll
-    for (int m = 0; m < PFC; ++m) {
-        const int tt = tsub + g.SP * (m >> g.lncc);
-        const int c = csub + g.CW * (m & ((1 << g.lncc) - 1));
-        const bool ok = tt < n && c < ncols;
-#pragma unroll
-        for (int a = 0; a < NCA; ++a)
-            pf.c[a][m] = ok ? colp[a][cbase + (int64_t)tt * ncols + c] : IO(0);
-    }
-    const int rsub = threadIdx.x % g.rows, tsr = threadIdx.x / g.rows;
-    const int64_t rbase = (b * T + t0) * nrows + row0;
-#pragma unroll
-    for (int m = 0; m < PFR; ++m) {
-        const int tt = tsr + g.SPR * m;
-        const bool ok = tt < n && row0 + rsub < nrows;
-#pragma unroll
-        for (int a = 0; a < NRA; ++a)
-            pf.r[a][m] = ok ? rowp[a][rbase + (int64_t)tt * nrows + rsub] : IO(0);
-    }
-}
-
-// Write the prefetched block into LDS: colL[(tt*NCA + a)*KP + c], rowL[(tt*NRA + a)*rows + r]
-template <typename IO, typename Acc, int NCA, int NRA>
-__device__ __forceinline__ void block_store(const Prefetch<IO, NCA, NRA> &pf, const Tile &g,
-                                            Acc *colL, Acc *rowL, int tb) {
-    const int csub = threadIdx.x % g.CW, tsub = threadIdx.x / g.CW;
-#pragma unroll
-    for (int m = 0; m < PFC; ++m) {
-        const int tt = tsub + g.SP * (m >> g.lncc);
-        const int c = csub + g.CW * (m & ((1 << g.lncc) - 1));
-        if (tt < tb) {
-#pragma unroll
-            for (int a = 0; a < NCA; ++a) colL[(tt * NCA + a) * g.KP + c] = to_acc(pf.c[a][m]);
-        }
-    }
-    const int rsub = threadIdx.x % g.rows, tsr = threadIdx.x / g.rows;
-#pragma unroll
-    for (int m = 0; m < PFR; ++m) {
-        const int tt = tsr + g.SPR * m;
-        if (tt < tb) {
-#pragma unroll
-            for (int a = 0; a < NRA; ++a) rowL[(tt * NRA + a) * g.rows + rsub] = to_acc(pf.r[a][m]);
-        }
-    }
-}
+using namespace scan;
 
 // ------------------------------------------------------------------------------------
 // forward
