@@ -73,6 +73,8 @@ def main():
     if not torch.cuda.is_available():
         print("bench.py: no GPU visible", file=sys.stderr)
         sys.exit(1)
+    if args.workload == "cfg5":
+        return bench_generation(args)
     lib = _lib.load()
     w = WORKLOADS[args.workload]
     B, T, D, K = w["B"], w["T"], w["D"], w["K"]
@@ -215,6 +217,64 @@ def main():
     }
     if cpu:
         line["speedup_vs_cpu"] = round(mtok / cpu["value"], 1) if cpu["value"] else None
+    print(json.dumps(line))
+
+
+def bench_generation(args):
+    """cfg5: O(1) generation steps at serving batch, the state carried in place.  A "step" is
+    one call of t2fw_lfw_step over the whole batch; bytes = state read + write + six vectors."""
+    import torch
+    from t2fw_amd import _lib
+    from tests.lfw_cases import make_config_inputs
+    lib = _lib.load()
+    w = WORKLOADS["cfg5"]
+    B, D, K = w["B"], w["D"], w["K"]
+    dtype = getattr(torch, w["dtype"])
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    nvec = 8
+    x, f, q, k, fk, s, _, _ = make_config_inputs(B, nvec, D, K, dtype, seed=0, gate_mean=w["gate_mean"])
+    vec = [[a[:, i].contiguous().to(dev) for a in (x, f, q, k, fk)] for i in range(nvec)]
+    state = s.to(dev)
+    out = torch.empty(B, D, dtype=dtype, device=dev)
+    stream = _lib.current_stream_handle(dev)
+    code = _lib.DTYPE_CODE[dtype]
+
+    def step(i):
+        v = vec[i % nvec]
+        _lib.check(lib.t2fw_lfw_step(*[_lib.ptr(t) for t in v], _lib.ptr(state), _lib.ptr(out), _lib.ptr(state),
+                                     B, D, K, code, stream))
+    for i in range(args.warmup):
+        step(i)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        step(i)
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    ev = [torch.cuda.Event(enable_timing=True) for _ in range(2)]
+    nrep = min(args.steps, 100)
+    ev[0].record()
+    for i in range(nrep):
+        step(i)
+    ev[1].record()
+    torch.cuda.synchronize()
+    kern_ms = ev[0].elapsed_time(ev[1]) / nrep
+    es = 2
+    nbytes = B * (2 * D * K * es + (3 * D + 3 * K) * es)
+    achieved = nbytes / (kern_ms * 1e-3) / 1e9
+    line = {
+        "metric": "generation steps: Mtokens/s and state GB/s (cfg5)", "value": round(B * args.steps / wall / 1e6, 1),
+        "unit": "Mtokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(wall / args.steps * 1e3, 5), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "fp16 I/O, fp32 arithmetic", "data": "synthetic",
+        "config": {"workload": "cfg5: B=%d T=1 D=%d K=%d float16, state carried in place over consecutive calls" % (B, D, K)},
+        "state_GBs": round(2 * B * D * K * es / (kern_ms * 1e-3) / 1e9, 1),
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None, "kernel": "lfw_step_kernel",
+                     "algorithmic_bytes": nbytes, "avg_launch_ms": round(kern_ms, 5)},
+        "cpu_baseline": None,
+    }
     print(json.dumps(line))
 
 

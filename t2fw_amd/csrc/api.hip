@@ -4,6 +4,7 @@
 #include "lfw_scan.hpp"
 #include "lfw_chunk.hpp"
 #include "dfw_scan.hpp"
+#include "lfw_step.hpp"
 
 #include <cstring>
 #include <initializer_list>
@@ -207,8 +208,25 @@ int t2fw_lfw_backward(const void *g_out, const void *g_state, const void *x, con
 
 int t2fw_lfw_step(const void *x, const void *f, const void *q, const void *k, const void *f_key, const void *s0,
                   void *out, void *next_state, int64_t B, int64_t D, int64_t K, int32_t dtype, void *stream) {
+    const size_t es = elem_size(dtype);
+    if (es == 0) return fail(T2FW_ERR_BAD_DTYPE, "unknown dtype code %d", dtype);
+    int rc = check_dims(B, 1, D, K);
+    if (rc) return rc;
+    if (B == 0) return T2FW_OK;
+    const NamedPtr ptrs[] = {{"x", x}, {"f", f}, {"q", q}, {"k", k}, {"f_key", f_key}, {"s0", s0}, {"out", out},
+                             {"next_state", next_state}};
+    if ((rc = check_ptrs(ptrs, 8, es))) return rc;
+    if (D == 64 && K == 64 && (dtype == T2FW_F16 || dtype == T2FW_BF16) &&
+        aligned16({x, f, q, k, f_key, s0, out, next_state})) {
+        StepArgs a{};
+        a.x = x; a.f = f; a.q = q; a.k = k; a.f_key = f_key; a.s0 = s0; a.out = out; a.next_state = next_state;
+        a.B = B;
+        return step_forward(a, dtype, static_cast<hipStream_t>(stream));
+    }
+    // general shapes: the exact scan kernel with T = 1 (each lane reads its state elements before
+    // it writes them, so updating in place is safe there too)
     return t2fw_lfw_forward(x, f, q, k, f_key, s0, out, next_state, nullptr, B, 1, D, K, 1, dtype,
-                            T2FW_FLAG_AUTO, nullptr, 0, stream);
+                            T2FW_FLAG_FORCE_SCAN, nullptr, 0, stream);
 }
 
 int t2fw_dfw_forward(const void *q, const void *k, const void *v, const void *s0, void *out, void *final_state,
