@@ -26,22 +26,12 @@
 //
 // Replaces lfw_cuda_bwd_kernel and the six einsums of the reference
 // (t2fw/csrc/lfw_kernel.cu:61-102, t2fw/csrc/lfw.cpp:84-93).
-#include "lfw_chunk.hpp"
-
-// Build-time diagnostic (-DT2FW_PHASE_TIMERS): workgroup 0 accumulates shader-clock ticks
-// per phase into row_flags[64..]; off in the shipped library.
-#ifdef T2FW_PHASE_TIMERS
-#define PHASE_BEGIN() unsigned long long ph_t = __builtin_amdgcn_s_memtime(); unsigned long long ph_acc[4] = {0, 0, 0, 0}
-#define PHASE_MARK(i) { const unsigned long long ph_n = __builtin_amdgcn_s_memtime(); ph_acc[i] += ph_n - ph_t; ph_t = ph_n; }
-#define PHASE_END(slot) if (b == 0 && (tid & 63) == 0) { for (int ph_i = 0; ph_i < 4; ++ph_i) p.row_flags[64 + (slot) * 8 + ph_i * 2] = (int)(ph_acc[ph_i] & 0x7fffffff); }
-#else
-#define PHASE_BEGIN()
-#define PHASE_MARK(i)
-#define PHASE_END(slot)
-#endif
+#include "lfw_chunk_bwd_dev.hpp"
 
 namespace t2fw {
 namespace {
+
+using namespace bwd;
 
 constexpr int BWD_THREADS = 512;
 constexpr int CC = 20;   // channel-major 16-token tiles: row stride in elements
@@ -69,84 +59,42 @@ constexpr int BOFF_RAW = BOFF_OUT + 2 * BOUT_BYTES;
 constexpr int BWD_SMEM = BOFF_RAW + 2 * BRAW_BYTES;
 static_assert(BWD_SMEM <= 160 * 1024, "backward stage buffers exceed the LDS of one CU");
 
-// ---- stage schedule ----------------------------------------------------------------------
-// Chunks are visited from the last one down; a chunk with nb blocks takes nb "R" stages
-// (blocks 0..nb-1) followed by nb "B" stages (blocks nb-1..0).
-struct StageInfo {
-    int chunk;
-    int block;      // block inside the chunk
-    bool bmode;     // false: recompute sweep, true: backward sweep
-};
-
-// 32-bit arithmetic only; NB is a power of two, so the divisions are shifts.
-template <int NB> struct Schedule {
-    int NC, total, nb_last;
-    __device__ Schedule(int64_t T, int64_t NC_, int C) {
-        NC = (int)NC_;
-        const int len_last = (int)(T - (NC_ - 1) * C);
-        nb_last = (len_last + CH_L - 1) / CH_L;
-        total = 2 * nb_last + (NC - 1) * 2 * NB;
-    }
-    __device__ StageInfo at(int s) const {
-        StageInfo r;
-        int local, nb;
-        if (s < 2 * nb_last) {
-            r.chunk = NC - 1;
-            local = s;
-            nb = nb_last;
-        } else {
-            const unsigned s2 = (unsigned)(s - 2 * nb_last);
-            r.chunk = NC - 2 - (int)(s2 / (2u * NB));
-            local = (int)(s2 % (2u * NB));
-            nb = NB;
-        }
-        r.bmode = local >= nb;
-        r.block = r.bmode ? 2 * nb - 1 - local : local;
-        return r;
-    }
-};
-
 // ---- raw staging -------------------------------------------------------------------------
+// A stage's raw inputs are R_NUM arrays of [16 tokens][64 channels]: 768 pieces of 16 bytes,
+// three per prep thread.  Everything that does not depend on the stage is worked out once per
+// thread (PieceMap), so that issuing a stage's loads costs a handful of instructions.
 struct BStage {
     uint4 v[3];
 };
 
-template <typename IOE>
-__device__ __forceinline__ void bstage_load(BStage &st, const u16 *const (&src)[R_NUM], int64_t row_base,
-                                            int64_t T, int64_t t0, bool bmode, int tid) {
+struct PieceMap {
+    const u16 *ld[3];     // source of raw piece m at token offset 0 of this batch row
+    u16 *st[3];           // destination of gradient piece m at token offset 0 (null: no such piece)
+    int arr[3];           // raw array index of piece m
+    int tok[3];           // token inside the block
+    u32 fill[3];          // identity fill for steps past the end of the sequence
+    int out_off[3];       // byte offset of gradient piece m inside one OUT buffer
+};
+
+__device__ __forceinline__ void bstage_load(BStage &st, const PieceMap &pm, int64_t T, int64_t t0, bool bmode) {
     const int narr = bmode ? R_NUM : 4;
 #pragma unroll
     for (int m = 0; m < 3; ++m) {
-        const int p = tid + 256 * m;            // piece index: [array][token][8 pieces]
-        const int a = p >> 7, tok = (p >> 3) & 15, piece = p & 7;
-        if (a < narr) {
-            const int64_t t = t0 + tok;
-            if (t < T) {
-                st.v[m] = *reinterpret_cast<const uint4 *>(src[a] + (row_base + t) * CH_N + 8 * piece);
-            } else {
-                // steps past the end act as identity: gates 1, everything else 0
-                const u32 fill = (a == R_FK || a == R_F) ? (u32)IOE::ONE_BITS * 0x10001u : 0u;
-                st.v[m] = make_uint4(fill, fill, fill, fill);
-            }
+        if (pm.arr[m] < narr) {
+            if (t0 + pm.tok[m] < T)
+                st.v[m] = *reinterpret_cast<const uint4 *>(pm.ld[m] + t0 * CH_N);
+            else
+                st.v[m] = make_uint4(pm.fill[m], pm.fill[m], pm.fill[m], pm.fill[m]);
         }
     }
 }
 
-__device__ __forceinline__ void bstage_store(const BStage &st, unsigned char *raw, bool bmode, int tid) {
+__device__ __forceinline__ void bstage_store(const BStage &st, const PieceMap &pm, unsigned char *raw, bool bmode,
+                                             int tid) {
     const int narr = bmode ? R_NUM : 4;
 #pragma unroll
-    for (int m = 0; m < 3; ++m) {
-        const int p = tid + 256 * m;
-        if ((p >> 7) < narr) *reinterpret_cast<uint4 *>(raw + p * 16) = st.v[m];
-    }
-}
-
-template <typename E> __device__ __forceinline__ uint2 packq(float a, float b, float c, float d) {
-    return make_uint2(E::pack2(a, b), E::pack2(c, d));
-}
-
-template <typename E> __device__ __forceinline__ uint2 pack4v(const floatx4 &v) {
-    return make_uint2(E::pack2(v[0], v[1]), E::pack2(v[2], v[3]));
+    for (int m = 0; m < 3; ++m)
+        if (pm.arr[m] < narr) *reinterpret_cast<uint4 *>(raw + (tid + 256 * m) * 16) = st.v[m];
 }
 
 // column of one raw array for channel c
@@ -154,16 +102,6 @@ __device__ __forceinline__ void raw_col(u16 (&dst)[CH_L], const unsigned char *r
     const u16 *base = reinterpret_cast<const u16 *>(raw + array * BRAW_ARRAY) + c;
 #pragma unroll
     for (int t = 0; t < CH_L; ++t) dst[t] = base[t * CH_N];
-}
-
-template <typename IOE> __device__ __forceinline__ u32 gate_check(const u16 (&g)[CH_L]) {
-    u16 mx = 0;
-#pragma unroll
-    for (int t = 0; t < CH_L; ++t) {
-        const u16 m1 = (u16)(g[t] - 1);      // gates must lie in (0, 1]: 0 < bits <= bits(1.0)
-        mx = m1 > mx ? m1 : mx;
-    }
-    return (mx >= IOE::ONE_BITS) ? 1u : 0u;
 }
 
 template <typename OPE>
@@ -260,20 +198,38 @@ __device__ __forceinline__ void bwd_prep_waves(const ChunkBwdArgs &p, unsigned c
     if (tid == 0) p.row_flags[b] = 0;
     auto tok0_of = [&](const StageInfo &si) -> int64_t { return (int64_t)si.chunk * p.C + si.block * CH_L; };
 
-    // raw inputs of stage m live in RAW[m & 1]; `st` carries the next stage to be written
-    BStage st;
+    PieceMap pm;
+#pragma unroll
+    for (int m = 0; m < 3; ++m) {
+        const int pi = tid + 256 * m;              // [array or gradient][token][8 pieces]
+        const int a = pi >> 7, tok = (pi >> 3) & 15, piece = pi & 7;
+        const int64_t off = (row_base + tok) * CH_N + 8 * piece;
+        pm.arr[m] = a;
+        pm.tok[m] = tok;
+        pm.ld[m] = src[a] + off;                   // a <= 5 for every piece
+        pm.fill[m] = (a == R_FK || a == R_F) ? (u32)IOE::ONE_BITS * 0x10001u : 0u;
+        pm.st[m] = a < O_NUM ? dst[a] + off : nullptr;
+        pm.out_off[m] = a * BOUT_TILE + (tok * OS + 8 * piece) * 2;
+    }
+
+    // raw inputs of stage m live in RAW[m & 1]; stA / stB carry the even / odd stages two ahead
+    BStage stA, stB;
     {
         const StageInfo s0 = sched.at(0);
-        bstage_load<IOE>(st, src, row_base, T, tok0_of(s0), s0.bmode, tid);
-        bstage_store(st, smem + BOFF_RAW, s0.bmode, tid);
+        bstage_load(stA, pm, T, tok0_of(s0), s0.bmode);
+        bstage_store(stA, pm, smem + BOFF_RAW, s0.bmode, tid);
         if (total > 1) {
             const StageInfo s1 = sched.at(1);
-            bstage_load<IOE>(st, src, row_base, T, tok0_of(s1), s1.bmode, tid);
-            bstage_store(st, smem + BOFF_RAW + BRAW_BYTES, s1.bmode, tid);
+            bstage_load(stB, pm, T, tok0_of(s1), s1.bmode);
+            bstage_store(stB, pm, smem + BOFF_RAW + BRAW_BYTES, s1.bmode, tid);
         }
         if (total > 2) {
             const StageInfo s2 = sched.at(2);
-            bstage_load<IOE>(st, src, row_base, T, tok0_of(s2), s2.bmode, tid);
+            bstage_load(stA, pm, T, tok0_of(s2), s2.bmode);
+        }
+        if (total > 3) {
+            const StageInfo s3 = sched.at(3);
+            bstage_load(stB, pm, T, tok0_of(s3), s3.bmode);
         }
         __syncthreads();
         bwd_prep<IOE, OPE>(smem + BOFF_RAW, smem, role, c, s0.bmode, bad);
@@ -287,28 +243,24 @@ __device__ __forceinline__ void bwd_prep_waves(const ChunkBwdArgs &p, unsigned c
         const int64_t t0 = tok0_of(si);
 #pragma unroll
         for (int m = 0; m < 3; ++m) {
-            const int pi = tid + 256 * m;          // [output][token][8 pieces]
-            const int o = pi >> 7, tok = (pi >> 3) & 15, piece = pi & 7;
-            if (o < O_NUM && t0 + tok < T) {
-                const u16 *tile = reinterpret_cast<const u16 *>(outp + o * BOUT_TILE) + tok * OS + 8 * piece;
+            if (pm.st[m] != nullptr && t0 + pm.tok[m] < T) {
+                const u16 *tile = reinterpret_cast<const u16 *>(outp + pm.out_off[m]);
                 const uint2 lo = *reinterpret_cast<const uint2 *>(tile);
                 const uint2 hi = *reinterpret_cast<const uint2 *>(tile + 4);
-                *reinterpret_cast<uint4 *>(dst[o] + (row_base + t0 + tok) * CH_N + 8 * piece) =
-                    make_uint4(lo.x, lo.y, hi.x, hi.y);
+                *reinterpret_cast<uint4 *>(pm.st[m] + t0 * CH_N) = make_uint4(lo.x, lo.y, hi.x, hi.y);
             }
         }
     };
 
     PHASE_BEGIN();
-    for (int s = 0; s < total; ++s) {
-        // consume last iteration's loads first (everything still in flight is at least most of an
-        // iteration old), then issue this iteration's stores, then the next loads
-        if (s + 2 < total) bstage_store(st, smem + BOFF_RAW + (s & 1) * BRAW_BYTES, sched.at(s + 2).bmode, tid);
+    auto iteration = [&](int s, BStage &st) {       // st holds stage s+2, then takes stage s+4
+        PHASE_SELECT(sched.at(s).bmode ? 0 : 4);
+        if (s + 2 < total) bstage_store(st, pm, smem + BOFF_RAW + (s & 1) * BRAW_BYTES, sched.at(s + 2).bmode, tid);
         PHASE_MARK(1);
         if (s > 0) store_out(s - 1);
-        if (s + 3 < total) {
-            const StageInfo s3 = sched.at(s + 3);
-            bstage_load<IOE>(st, src, row_base, T, tok0_of(s3), s3.bmode, tid);
+        if (s + 4 < total) {
+            const StageInfo s4 = sched.at(s + 4);
+            bstage_load(st, pm, T, tok0_of(s4), s4.bmode);
         }
         PHASE_MARK(0);
         if (s + 1 < total)
@@ -317,6 +269,10 @@ __device__ __forceinline__ void bwd_prep_waves(const ChunkBwdArgs &p, unsigned c
         PHASE_MARK(2);
         __syncthreads();
         PHASE_MARK(3);
+    };
+    for (int s = 0; s < total; s += 2) {
+        iteration(s, stA);
+        if (s + 1 < total) iteration(s + 1, stB);
     }
     store_out(total - 1);
     if (bad) p.row_flags[b] = 1;
@@ -333,31 +289,6 @@ __device__ __forceinline__ const u16 *cm_tile(const unsigned char *stage, int ti
 __device__ __forceinline__ const float *cf_tile(const unsigned char *stage, int tile) {
     return reinterpret_cast<const float *>(stage + OFF_CF + tile * CF_TILE);
 }
-__device__ __forceinline__ uint2 ld2(const u16 *p) { return *reinterpret_cast<const uint2 *>(p); }
-__device__ __forceinline__ uint4 ld4(const u16 *p) { return *reinterpret_cast<const uint4 *>(p); }
-__device__ __forceinline__ uint4 cat(uint2 a, uint2 b) { return make_uint4(a.x, a.y, b.x, b.y); }
-
-template <typename E> __device__ __forceinline__ void unpack4(uint2 v, float (&o)[4]) {
-    o[0] = E::to_f32((u16)(v.x & 0xffff));
-    o[1] = E::to_f32((u16)(v.x >> 16));
-    o[2] = E::to_f32((u16)(v.y & 0xffff));
-    o[3] = E::to_f32((u16)(v.y >> 16));
-}
-
-// Reverse running sum over the 16 tokens of a block: lane (g, r) holds d[i] for token 4g+i of its channel;
-// returns the inclusive suffix sums plus `carry`, and updates carry to the value at token 0.
-__device__ __forceinline__ void reverse_running_sum(float (&d)[4], float &carry, int g, int r) {
-    d[2] += d[3];
-    d[1] += d[2];
-    d[0] += d[1];
-    const float tot = d[0];
-    const float t16 = __shfl_down(tot, 16, 64), t32 = __shfl_down(tot, 32, 64), t48 = __shfl_down(tot, 48, 64);
-    const float higher = (g < 3 ? t16 : 0.f) + (g < 2 ? t32 : 0.f) + (g < 1 ? t48 : 0.f) + carry;
-#pragma unroll
-    for (int i = 0; i < 4; ++i) d[i] += higher;
-    carry = __shfl(d[0], r, 64);
-}
-
 template <typename IOE, typename OPE, int NB>
 __device__ __forceinline__ void bwd_matrix_waves(const ChunkBwdArgs &p, unsigned char *smem, int tid, int64_t b) {
     const int w = tid >> 6, l = tid & 63, r = l & 15, g = l >> 4;
