@@ -73,6 +73,10 @@ extern "C" {
 #define T2FW_FLAG_FP16_OPERANDS 2 /* fp16 tensors: fp16 (not bf16) matrix-core operands;
                                      more mantissa, but rows whose 16-step gate products
                                      fall below 2^-8 take the exact scan path          */
+#define T2FW_FLAG_BWD_WHOLE_ROW 4 /* backward, matrix-core path: one workgroup per batch row  */
+#define T2FW_FLAG_BWD_SPLIT 8     /* backward, matrix-core path: two workgroups per batch row
+                                     (value side / key side).  With neither bit the library
+                                     splits when twice the batch fits the device's CUs.      */
 
 int t2fw_abi_version(void);
 const char *t2fw_last_error(void);

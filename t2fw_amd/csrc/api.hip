@@ -65,6 +65,14 @@ bool chunk_shape_ok(int64_t D, int64_t K, int32_t dtype, int32_t flags) {
     return (flags & T2FW_FLAG_FORCE_SCAN) == 0 && D == 64 && K == 64 && (dtype == T2FW_F16 || dtype == T2FW_BF16);
 }
 
+// compute units of the current device (-1 on error)
+int compute_units() {
+    int dev = 0, n = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return -1;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return -1;
+    return n;
+}
+
 size_t row_flag_bytes(int64_t B) { return (size_t)((B * 4 + 255) / 256 * 256); }
 
 int check_dims(int64_t B, int64_t T, int64_t D, int64_t K) {
@@ -200,7 +208,13 @@ int t2fw_lfw_backward(const void *g_out, const void *g_state, const void *x, con
         c.row_flags = static_cast<int32_t *>(workspace);
         c.B = B; c.T = T; c.NC = a.NC; c.C = C;
         const int op = (dtype == T2FW_F16 && (flags & T2FW_FLAG_FP16_OPERANDS)) ? 1 : 0;
-        if ((rc = chunk_backward(c, dtype, op, st))) return rc;
+        bool split = (flags & T2FW_FLAG_BWD_SPLIT) != 0 && T < CHUNK_SPLIT_MAX_T;
+        if ((flags & (T2FW_FLAG_BWD_SPLIT | T2FW_FLAG_BWD_WHOLE_ROW)) == 0) {
+            const int cus = compute_units();
+            if (cus < 0) return fail(T2FW_ERR_HIP, "could not read the device's compute-unit count");
+            split = 2 * ((B + 7) / 8 * 8) <= cus && T < CHUNK_SPLIT_MAX_T;
+        }
+        if ((rc = split ? chunk_backward_split(c, dtype, op, st) : chunk_backward(c, dtype, op, st))) return rc;
         a.row_select = c.row_flags;      // rows the chunked form could not take
     }
     return scan_backward(a, dtype, st);

@@ -41,6 +41,9 @@ struct ChunkBwdArgs {
 // op: 0 = bf16 operands, 1 = fp16 operands (fp16 I/O only)
 int chunk_forward(const ChunkFwdArgs &a, int dtype, int op, hipStream_t stream);
 int chunk_backward(const ChunkBwdArgs &a, int dtype, int op, hipStream_t stream);
+// same result from two workgroups per batch row (one per side of the state); for batches that leave CUs idle
+int chunk_backward_split(const ChunkBwdArgs &a, int dtype, int op, hipStream_t stream);
+constexpr int64_t CHUNK_SPLIT_MAX_T = 1 << 24;      // the split kernel addresses a batch row with 32-bit offsets
 
 #if defined(__HIPCC__)
 
