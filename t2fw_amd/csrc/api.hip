@@ -208,11 +208,12 @@ int t2fw_lfw_backward(const void *g_out, const void *g_state, const void *x, con
         c.row_flags = static_cast<int32_t *>(workspace);
         c.B = B; c.T = T; c.NC = a.NC; c.C = C;
         const int op = (dtype == T2FW_F16 && (flags & T2FW_FLAG_FP16_OPERANDS)) ? 1 : 0;
-        bool split = (flags & T2FW_FLAG_BWD_SPLIT) != 0 && T < CHUNK_SPLIT_MAX_T;
+        const bool split_ok = T < CHUNK_SPLIT_MAX_T && T % 16 == 0;
+        bool split = (flags & T2FW_FLAG_BWD_SPLIT) != 0 && split_ok;
         if ((flags & (T2FW_FLAG_BWD_SPLIT | T2FW_FLAG_BWD_WHOLE_ROW)) == 0) {
             const int cus = compute_units();
             if (cus < 0) return fail(T2FW_ERR_HIP, "could not read the device's compute-unit count");
-            split = 2 * ((B + 7) / 8 * 8) <= cus && T < CHUNK_SPLIT_MAX_T;
+            split = 2 * ((B + 7) / 8 * 8) <= cus && split_ok;
         }
         if ((rc = split ? chunk_backward_split(c, dtype, op, st) : chunk_backward(c, dtype, op, st))) return rc;
         a.row_select = c.row_flags;      // rows the chunked form could not take

@@ -15,9 +15,12 @@
 //   d_own_gate_t = RG_t * (carry + sum_{r>=t} o'_r AS_r - v'_r VT_r)
 //   d_V_t = IP_t * (v'_t + AS_t P[t,t])        d_A_t = PP_t * (o'_t + VT_t P[t,t])   (side 1 only)
 //   Gb <- L_own[c] L_other[e] Gb[c,e] + sum_t AS_t[c] AOS_t[e]
-// Used when twice the batch fits the CUs of the device: the 12-wave workgroups (4 matrix
-// waves + 8 prep waves, two per role, each taking 8 of a block's 16 tokens) halve the
-// instructions on every wave's critical path compared with the whole-row kernel.
+// Used when twice the batch fits the CUs of the device and T is a multiple of 16: the 12-wave
+// workgroups (4 matrix waves + 8 prep waves, two per role, each taking 8 of a block's 16
+// tokens) halve the instructions on every wave's critical path compared with the whole-row
+// kernel.  The recompute sweep of a chunk takes two blocks per stage (all eight prep waves
+// build the few tiles it needs), raw inputs go from global memory straight to the prep
+// waves' registers two stages ahead, and the matrix waves store the gradients themselves.
 //
 // Replaces lfw_cuda_bwd_kernel and the six einsums of the reference
 // (t2fw/csrc/lfw_kernel.cu:61-102, t2fw/csrc/lfw.cpp:84-93).
@@ -29,7 +32,6 @@ namespace {
 using namespace bwd;
 
 constexpr int SP_THREADS = 768;
-constexpr int SP_PREP = 512;
 constexpr int CC = 20;   // channel-major 16-token tiles: row stride in elements
 
 // ---- LDS layout of one stage buffer (bytes) ----------------------------------------------
@@ -37,91 +39,82 @@ constexpr int TM_TILE = CH_L * TS * 2;       // token-major 16-bit tile [16][TS]
 constexpr int CM_TILE = CH_N * CC * 2;       // channel-major 16-bit tile [64][CC]
 constexpr int CF_TILE = CH_N * CC * 4;       // channel-major fp32 tile [64][CC]
 enum { TM_AOS = 0, TM_VOT, TM_VOH, TM_NUM };
+// B stages use the named tiles; an R stage covers two blocks j = 0, 1 and uses tiles 2j (VOH) and 2j+1 (VH)
 enum { CM_AOS = 0, CM_VOH, CM_AS, CM_VT, CM_VH, CM_NUM };
 enum { F_RG = 0, F_IP, F_PP, F_NUM };        // 1/own gate, 1/own prefix, own prefix
 constexpr int OFF_TM = 0;
 constexpr int OFF_CM = OFF_TM + TM_NUM * TM_TILE;
 constexpr int OFF_CF = OFF_CM + CM_NUM * CM_TILE;
-constexpr int OFF_LX = OFF_CF + F_NUM * CF_TILE;           // 16-step product of the other side's gate [64] f32
-constexpr int OFF_LO = OFF_LX + CH_N * 4;                  // 16-step product of the own gate [64] f32
-constexpr int STAGE_BYTES = OFF_LO + CH_N * 4;
-constexpr int RAW_ARRAY = CH_L * CH_N * 2;                 // [16][64] u16
-enum { R_GO = 0, R_VO, R_GW, R_VW, R_AO, R_AW, R_NUM };   // R stages need the first four only
-constexpr int RAW_BYTES = R_NUM * RAW_ARRAY;
-constexpr int SOFF_RAW = 2 * STAGE_BYTES;
-constexpr int SP_SMEM = SOFF_RAW + 2 * RAW_BYTES;
+// 16-step gate products, [block j of an R stage][other side, own side][64] f32 (B stages: j = 0)
+constexpr int OFF_LV = OFF_CF + F_NUM * CF_TILE;
+constexpr int STAGE_BYTES = OFF_LV + 4 * CH_N * 4;
+constexpr int SP_SMEM = 2 * STAGE_BYTES;
 static_assert(SP_SMEM <= 160 * 1024, "backward stage buffers exceed the LDS of one CU");
 static_assert(STAGE_BYTES % 16 == 0, "stage buffers must keep 16-byte alignment");
+
+__device__ __forceinline__ float *lv_vec(unsigned char *stage, int j, int own) {
+    return reinterpret_cast<float *>(stage + OFF_LV) + (2 * j + own) * CH_N;
+}
+__device__ __forceinline__ const float *lv_vec(const unsigned char *stage, int j, int own) {
+    return reinterpret_cast<const float *>(stage + OFF_LV) + (2 * j + own) * CH_N;
+}
 
 // Position of channel c = 16j + 4g + e inside a token-major row: 16g + 4j + e.  The 16 values a
 // lane contracts against its own accumulators (channels 16j + 4g + e, j = 0..3) are then
 // contiguous.  Products between two token-major tiles are indifferent to the order.
 __device__ __forceinline__ int tm_pos(int c) { return 16 * ((c >> 2) & 3) + 4 * (c >> 4) + (c & 3); }
 
-struct Side {
-    const u16 *src[R_NUM];      // raw arrays in the order of R_*
-};
-
-__device__ __forceinline__ Side make_side(const ChunkBwdArgs &p, int side) {
-    Side s;
-    const u16 *x = reinterpret_cast<const u16 *>(p.x), *f = reinterpret_cast<const u16 *>(p.f);
-    const u16 *g = reinterpret_cast<const u16 *>(p.g_out), *k = reinterpret_cast<const u16 *>(p.k);
-    const u16 *fk = reinterpret_cast<const u16 *>(p.f_key), *q = reinterpret_cast<const u16 *>(p.q);
-    if (side == 0) {
-        s.src[R_GO] = fk; s.src[R_VO] = k; s.src[R_GW] = f; s.src[R_VW] = x; s.src[R_AO] = q; s.src[R_AW] = g;
-    } else {
-        s.src[R_GO] = f; s.src[R_VO] = x; s.src[R_GW] = fk; s.src[R_VW] = k; s.src[R_AO] = g; s.src[R_AW] = q;
+// ---- stage schedule ----------------------------------------------------------------------
+// Chunks are visited from the last one down; a chunk with nb blocks takes ceil(nb/2) "R"
+// stages of two blocks each (forward in time), then nb "B" stages (blocks nb-1..0).
+// A stage is one int: (first token of its first block) * 2 + (1 for a B stage).
+template <int NB> struct SplitSchedule {
+    static constexpr unsigned PER_CHUNK = NB / 2 + NB;
+    int NC, C, total, nb_last, st_last;
+    __device__ SplitSchedule(int64_t T, int64_t NC_, int C_) {
+        NC = (int)NC_;
+        C = C_;
+        const int len_last = (int)(T - (NC_ - 1) * C_);
+        nb_last = (len_last + CH_L - 1) / CH_L;
+        st_last = (nb_last + 1) / 2 + nb_last;
+        total = st_last + (NC - 1) * (int)PER_CHUNK;
     }
-    return s;
-}
-
-// ---- raw staging -------------------------------------------------------------------------
-// A stage's raw inputs are R_NUM arrays of [16 tokens][64 channels]: 768 pieces of 16 bytes;
-// prep thread i moves pieces i and (for i < 256, B stages only) i + 512.  R stages need pieces
-// 0..511 only.  A wave's pieces come from one array, so the array base stays in scalar
-// registers and a piece is addressed by a 32-bit element offset inside the batch row.  Loads
-// are issued at the top of an iteration and parked in LDS at its end, so the wait for them
-// overlaps the tile building in between; they are unconditional (clamped token, identity fill
-// selected afterwards), which keeps the hardware memory counters exact.
-constexpr int NPIECE = 2;
-struct RawRegs {
-    uint4 v[NPIECE];
-    bool valid;
+    __device__ int at(int s) const {
+        int chunk, local, nb;
+        if (s < st_last) {
+            chunk = NC - 1;
+            local = s;
+            nb = nb_last;
+        } else {
+            const unsigned s2 = (unsigned)(s - st_last);
+            chunk = NC - 2 - (int)(s2 / PER_CHUNK);
+            local = (int)(s2 % PER_CHUNK);
+            nb = NB;
+        }
+        const int nr = (nb + 1) / 2;
+        const bool bmode = local >= nr;
+        const int block = bmode ? nb - 1 - (local - nr) : 2 * local;
+        return ((chunk * C + block * CH_L) << 1) | (bmode ? 1 : 0);
+    }
 };
 
-// element a of a small pointer table, a wave-uniform: scalar selects that keep the pointers' provenance
-template <typename P> __device__ __forceinline__ P pick(int a, P p0, P p1, P p2, P p3, P p4, P p5) {
-    return a == 0 ? p0 : a == 1 ? p1 : a == 2 ? p2 : a == 3 ? p3 : a == 4 ? p4 : p5;
-}
-
-struct PieceMap {
-    const u16 *ld[NPIECE];   // this batch row of the array raw piece m comes from (wave-uniform)
-    int tok;                 // token inside the block (the same for both pieces)
-    u32 col;                 // element offset of the piece inside a token's 64 channels
-    u32 fill;                // identity fill of piece 0 for steps past the end of the sequence (piece 1: zero)
-    bool second;             // this thread also moves piece i + 512 (wave-uniform)
+// ---- raw inputs --------------------------------------------------------------------------
+// A prep thread works on one channel and eight tokens; it needs the gate at those tokens, the
+// gate at the block's other eight tokens and one value (or adjoint) array at its own tokens:
+// 24 two-byte loads, coalesced over the wave's 64 channels.  They go straight to registers,
+// two stages ahead of their use, from a wave-uniform base with immediate token offsets.
+struct RawSet {
+    u16 gown[8], goth[8], val[8];
 };
 
-__device__ __forceinline__ void raw_load(RawRegs &st, const PieceMap &pm, int T, int t0, bool bmode) {
-    const int t = t0 + pm.tok;
-    st.valid = t < T;
-    const u32 off = (u32)(st.valid ? t : T - 1) * CH_N + pm.col;
-    st.v[0] = *reinterpret_cast<const uint4 *>(pm.ld[0] + off);
-    if (pm.second && bmode) st.v[1] = *reinterpret_cast<const uint4 *>(pm.ld[1] + off);
-}
-
-__device__ __forceinline__ void raw_store(const RawRegs &st, const PieceMap &pm, unsigned char *raw, bool bmode, int tid) {
-    const u32 fl = pm.fill;
-    *reinterpret_cast<uint4 *>(raw + tid * 16) = st.valid ? st.v[0] : make_uint4(fl, fl, fl, fl);
-    if (pm.second && bmode)
-        *reinterpret_cast<uint4 *>(raw + (tid + SP_PREP) * 16) = st.valid ? st.v[1] : make_uint4(0u, 0u, 0u, 0u);
-}
-
-// eight consecutive tokens (from t0) of channel c of one raw array
-__device__ __forceinline__ void raw_col8(u16 (&dst)[8], const unsigned char *raw, int array, int c, int t0) {
-    const u16 *base = reinterpret_cast<const u16 *>(raw + array * RAW_ARRAY) + t0 * CH_N + c;
+__device__ __forceinline__ void raw_issue(RawSet &r, const u16 *gate, const u16 *val, int h, int c) {
+    const u16 *go = gate + 8 * h * CH_N + c, *gx = gate + 8 * (1 - h) * CH_N + c, *va = val + 8 * h * CH_N + c;
 #pragma unroll
-    for (int t = 0; t < 8; ++t) dst[t] = base[t * CH_N];
+    for (int t = 0; t < 8; ++t) {
+        r.gown[t] = go[t * CH_N];
+        r.goth[t] = gx[t * CH_N];
+        r.val[t] = va[t * CH_N];
+    }
 }
 
 template <typename IOE> __device__ __forceinline__ u32 gate_check8(const u16 (&g)[8]) {
@@ -154,36 +147,66 @@ __device__ __forceinline__ void write_cf8(unsigned char *stage, int tile, int c,
     cf[1] = make_float4(v[4], v[5], v[6], v[7]);
 }
 
-// One prep wave: one role, tokens 8h..8h+7 of the block, channel c.
+// Raw inputs as floats: the registers of the RawSet are free again after this.
+struct RawF {
+    float gown[8], goth_prod, val[8];
+    u32 bad;      // own gates outside (0, 1]
+};
+
+template <typename IOE> __device__ __forceinline__ RawF raw_take(const RawSet &r) {
+    RawF f;
+    f.bad = gate_check8<IOE>(r.gown);
+    float po = 1.0f;
+#pragma unroll
+    for (int t = 0; t < 8; ++t) {
+        f.gown[t] = IOE::to_f32(r.gown[t]);
+        f.val[t] = IOE::to_f32(r.val[t]);
+        po *= IOE::to_f32(r.goth[t]);
+    }
+    f.goth_prod = po;
+    return f;
+}
+
+// Gate-suffix scalings of one half block: hat = v * prod_{r>t} gate_r, til = hat / total,
+// inv = 1 / prod_{r<=t} gate_r; returns the 16-step product.
+template <typename OPE>
+__device__ __forceinline__ float suffix_scale(const RawF &f, int h, float (&hat)[8], float (&til)[8], float (&inv)[8],
+                                              u32 &bad) {
+    float pown = 1.0f;
+#pragma unroll
+    for (int t = 0; t < 8; ++t) pown *= f.gown[t];
+    const float tot = pown * f.goth_prod;
+    bad |= f.bad | ((tot >= OPE::MIN_PRODUCT) ? 0u : 1u);
+    const float itot = __builtin_amdgcn_rcpf(tot);
+    float sfx = h ? 1.0f : f.goth_prod;
+#pragma unroll
+    for (int t = 7; t >= 0; --t) {
+        inv[t] = sfx * itot;
+        hat[t] = f.val[t] * sfx;
+        til[t] = hat[t] * itot;
+        sfx *= f.gown[t];
+    }
+    return tot;
+}
+
+// B stage, one prep wave: one role, tokens 8h..8h+7 of the block, channel c.
 //   role 0: other gate prefix -> AOS (token- and channel-major)
 //   role 1: other gate suffix -> VOH (both layouts), VOT (token-major), L_other
 //   role 2: own gate prefix   -> AS, 1/gate, prefix (side 1)
 //   role 3: own gate suffix   -> VH, VT, 1/prefix, L_own
-// R stages need VOH and VH channel-major and the two 16-step products only.
-template <typename IOE, typename OPE>
-__device__ __forceinline__ void split_prep(const unsigned char *raw, unsigned char *stage, int role, int h, int c,
-                                           bool bmode, bool want_pp, u32 &bad) {
+template <typename OPE>
+__device__ __forceinline__ void prep_b(const RawF &f, unsigned char *stage, int role, int h, int c, bool want_pp,
+                                       u32 &bad) {
     const bool other = role < 2;
-    const bool prefix_role = (role & 1) == 0;
-    if (!bmode && prefix_role) return;
     const int t0 = 8 * h;
-    const int garr = other ? R_GO : R_GW;
-    u16 gown[8], goth[8], ar[8];
-    raw_col8(gown, raw, garr, c, t0);
-    raw_col8(ar, raw, prefix_role ? (other ? R_AO : R_AW) : (other ? R_VO : R_VW), c, t0);
-    if (prefix_role) {
-        float run = 1.0f;
-        if (h) {
-            raw_col8(goth, raw, garr, c, 0);
-#pragma unroll
-            for (int t = 0; t < 8; ++t) run *= IOE::to_f32(goth[t]);
-        }
+    if ((role & 1) == 0) {
+        float run = h ? f.goth_prod : 1.0f;
         float pre[8], v[8];
 #pragma unroll
         for (int t = 0; t < 8; ++t) {
-            run *= IOE::to_f32(gown[t]);
+            run *= f.gown[t];
             pre[t] = run;
-            v[t] = IOE::to_f32(ar[t]) * run;
+            v[t] = f.val[t] * run;
         }
         if (other) {
             write_tm8<OPE>(stage, TM_AOS, c, t0, v);
@@ -191,132 +214,108 @@ __device__ __forceinline__ void split_prep(const unsigned char *raw, unsigned ch
         } else {
             float rg[8];
 #pragma unroll
-            for (int t = 0; t < 8; ++t) rg[t] = __builtin_amdgcn_rcpf(IOE::to_f32(gown[t]));
+            for (int t = 0; t < 8; ++t) rg[t] = __builtin_amdgcn_rcpf(f.gown[t]);
             write_cm8<OPE>(stage, CM_AS, c, t0, v);
             write_cf8(stage, F_RG, c, t0, rg);
             if (want_pp) write_cf8(stage, F_PP, c, t0, pre);
         }
     } else {
-        raw_col8(goth, raw, garr, c, 8 - t0);
-        bad |= gate_check8<IOE>(gown);
-        float gate[8];
-        float pown = 1.0f, poth = 1.0f;
-#pragma unroll
-        for (int t = 0; t < 8; ++t) {
-            gate[t] = IOE::to_f32(gown[t]);
-            pown *= gate[t];
-            poth *= IOE::to_f32(goth[t]);
-        }
-        const float tot = pown * poth;
-        bad |= (tot >= OPE::MIN_PRODUCT) ? 0u : 1u;
-        const float itot = __builtin_amdgcn_rcpf(tot);
         float hat[8], til[8], inv[8];
-        float sfx = h ? 1.0f : poth;
-#pragma unroll
-        for (int t = 7; t >= 0; --t) {
-            inv[t] = sfx * itot;                            // 1 / prefix_t
-            hat[t] = IOE::to_f32(ar[t]) * sfx;
-            til[t] = hat[t] * itot;
-            sfx *= gate[t];
-        }
-        write_cm8<OPE>(stage, other ? CM_VOH : CM_VH, c, t0, hat);
-        if (h == 0) reinterpret_cast<float *>(stage + (other ? OFF_LX : OFF_LO))[c] = tot;
-        if (bmode) {
-            if (other) {
-                write_tm8<OPE>(stage, TM_VOH, c, t0, hat);
-                write_tm8<OPE>(stage, TM_VOT, c, t0, til);
-            } else {
-                write_cm8<OPE>(stage, CM_VT, c, t0, til);
-                write_cf8(stage, F_IP, c, t0, inv);
-            }
+        const float tot = suffix_scale<OPE>(f, h, hat, til, inv, bad);
+        if (h == 0) lv_vec(stage, 0, other ? 0 : 1)[c] = tot;
+        if (other) {
+            write_cm8<OPE>(stage, CM_VOH, c, t0, hat);
+            write_tm8<OPE>(stage, TM_VOH, c, t0, hat);
+            write_tm8<OPE>(stage, TM_VOT, c, t0, til);
+        } else {
+            write_cm8<OPE>(stage, CM_VH, c, t0, hat);
+            write_cm8<OPE>(stage, CM_VT, c, t0, til);
+            write_cf8(stage, F_IP, c, t0, inv);
         }
     }
+}
+
+// R stage, one prep wave: block j of the pair, own or other side, tokens 8h..8h+7, channel c:
+// the suffix-scaled values (channel-major) and the 16-step gate product.
+template <typename OPE>
+__device__ __forceinline__ void prep_r(const RawF &f, unsigned char *stage, int j, int own, int h, int c, u32 &bad) {
+    float hat[8], til[8], inv[8];
+    const float tot = suffix_scale<OPE>(f, h, hat, til, inv, bad);
+    if (h == 0) lv_vec(stage, j, own)[c] = tot;
+    write_cm8<OPE>(stage, 2 * j + own, c, 8 * h, hat);
 }
 
 template <typename IOE, typename OPE, int NB>
 __device__ __forceinline__ void split_prep_waves(const ChunkBwdArgs &p, unsigned char *smem, int tid, int64_t b,
                                                  int side) {
-    // wave pw: SIMD-balanced assignment of (role, token half); roles 1 and 3 are the heavier ones
-    const int pw = tid >> 6, c = tid & 63;
+    const int pw = __builtin_amdgcn_readfirstlane(tid >> 6), c = tid & 63;
+    // B stages: SIMD-balanced assignment of (role, token half); roles 1 and 3 are the heavier ones
     const int h = pw >> 2;
     const int role = (h ? (pw ^ 1) : pw) & 3;
-    const int T = (int)p.T;                              // the launcher admits T < 2^24 only
-    const int64_t row_base = b * p.T;
-    const Side sd = make_side(p, side);
-    const Schedule<NB> sched(p.T, p.NC, p.C);
+    // R stages: (block of the pair, side, token half)
+    const int rj = (pw >> 1) & 1, rown = pw & 1;
+    const int T = (int)p.T;                              // the launcher admits T < 2^24, T % 16 == 0 only
+    const int64_t row_off = b * p.T * CH_N;
+    // this batch row of: other gate, other value, own gate, own value, other adjoint, own adjoint
+    const u16 *const x = reinterpret_cast<const u16 *>(p.x) + row_off, *const f = reinterpret_cast<const u16 *>(p.f) + row_off;
+    const u16 *const g = reinterpret_cast<const u16 *>(p.g_out) + row_off, *const k = reinterpret_cast<const u16 *>(p.k) + row_off;
+    const u16 *const fk = reinterpret_cast<const u16 *>(p.f_key) + row_off, *const q = reinterpret_cast<const u16 *>(p.q) + row_off;
+    const u16 *const GO = side == 0 ? fk : f, *const VO = side == 0 ? k : x, *const GW = side == 0 ? f : fk;
+    const u16 *const VW = side == 0 ? x : k, *const AO = side == 0 ? q : g, *const AW = side == 0 ? g : q;
+    // the two arrays this wave reads in B stages and in R stages
+    const u16 *const b_gate = role < 2 ? GO : GW;
+    const u16 *const b_val = role == 0 ? AO : role == 1 ? VO : role == 2 ? AW : VW;
+    const u16 *const r_gate = rown ? GW : GO;
+    const u16 *const r_val = rown ? VW : VO;
+    const SplitSchedule<NB> sched(p.T, p.NC, p.C);
     const int total = sched.total;
     u32 bad = 0;
-    // a stage as one int: first token of its block * 2 + (1 for a B stage)
-    auto stage_at = [&](int s) -> int {
-        const StageInfo si = sched.at(s);
-        return ((si.chunk * p.C + si.block * CH_L) << 1) | (si.bmode ? 1 : 0);
+
+    auto issue = [&](RawSet &r, int st) {          // raw inputs of stage st (wave-uniform) -> registers
+        const int tok = st >> 1;
+        if (st & 1) {
+            raw_issue(r, b_gate + (u32)tok * CH_N, b_val + (u32)tok * CH_N, h, c);
+        } else {
+            // the second block of the last pair may lie past the end: read the last block instead
+            // (its tiles are never used)
+            const int t2 = min(tok + rj * CH_L, T - CH_L);
+            raw_issue(r, r_gate + (u32)t2 * CH_N, r_val + (u32)t2 * CH_N, h, c);
+        }
+    };
+    // builds the tiles of stage s (= st); r then takes stage s+2, and st that stage's descriptor
+    auto prepare = [&](RawSet &r, int s, int &st_io) {
+        const int st = st_io;
+        const RawF fr = raw_take<IOE>(r);
+        if (s + 2 < total) {
+            st_io = sched.at(s + 2);
+            issue(r, st_io);
+        }
+        unsigned char *stage = smem + (s & 1) * STAGE_BYTES;
+        if (st & 1)
+            prep_b<OPE>(fr, stage, role, h, c, side == 1, bad);
+        else
+            prep_r<OPE>(fr, stage, rj, rown, h, c, bad);
     };
 
-    PieceMap pm;
-    {
-        const int a0 = __builtin_amdgcn_readfirstlane(pw >> 1);   // pieces are ordered [array][token][8 pieces]
-        pm.tok = (tid >> 3) & 15;
-        pm.col = 8u * (tid & 7);
-        pm.second = a0 < 2;
-        pm.ld[0] = pick(a0, sd.src[0], sd.src[1], sd.src[2], sd.src[3], sd.src[4], sd.src[5]) + row_base * CH_N;
-        pm.ld[1] = (a0 == 0 ? sd.src[4] : sd.src[5]) + row_base * CH_N;
-        pm.fill = (a0 == R_GO || a0 == R_GW) ? (u32)IOE::ONE_BITS * 0x10001u : 0u;
-    }
-
-    // raw inputs of stage m live in RAW[m & 1]; stA / stB carry the even / odd stages, loaded two
-    // iterations before they are parked in LDS (HBM latency is of the order of one iteration)
-    RawRegs stA, stB;
-    int cur = stage_at(0), nxt = cur;                  // stages s and s+1 of the loop below
-    {
-        raw_load(stA, pm, T, cur >> 1, cur & 1);
-        raw_store(stA, pm, smem + SOFF_RAW, cur & 1, tid);
-        if (total > 1) {
-            nxt = stage_at(1);
-            raw_load(stB, pm, T, nxt >> 1, nxt & 1);
-            raw_store(stB, pm, smem + SOFF_RAW + RAW_BYTES, nxt & 1, tid);
-        }
-        __syncthreads();
-        split_prep<IOE, OPE>(smem + SOFF_RAW, smem, role, h, c, cur & 1, side == 1, bad);
-        __syncthreads();
-    }
-    int inA = cur, inB = cur;                          // the stages whose raw inputs stA / stB hold
-    if (total > 2) {
-        inA = stage_at(2);
-        raw_load(stA, pm, T, inA >> 1, inA & 1);
-    }
-    if (total > 3) {
-        inB = stage_at(3);
-        raw_load(stB, pm, T, inB >> 1, inB & 1);
-    }
-
+    RawSet setA, setB;
+    int stA = sched.at(0), stB = total > 1 ? sched.at(1) : stA;
+    issue(setA, stA);
+    if (total > 1) issue(setB, stB);
     PHASE_BEGIN();
-#define T2FW_SPLIT_ITERATION(s_, st, in)                                                                              \
-    {                                                                                                                  \
-        const int s = (s_);             /* st holds stage s+2 (= in), then takes stage s+4 */                          \
-        PHASE_SELECT((cur & 1) ? 0 : 4);                                                                               \
-        PHASE_MARK(0);                                                                                                 \
-        if (s + 1 < total)                                                                                             \
-            split_prep<IOE, OPE>(smem + SOFF_RAW + ((s + 1) & 1) * RAW_BYTES, smem + ((s + 1) & 1) * STAGE_BYTES,      \
-                                 role, h, c, nxt & 1, side == 1, bad);                                                 \
-        PHASE_MARK(2);                                                                                                 \
-        cur = nxt;                                                                                                     \
-        if (s + 2 < total) {                                                                                           \
-            raw_store(st, pm, smem + SOFF_RAW + (s & 1) * RAW_BYTES, in & 1, tid);                                     \
-            nxt = in;                                                                                                  \
-        }                                                                                                              \
-        if (s + 4 < total) {                                                                                           \
-            in = stage_at(s + 4);                                                                                      \
-            raw_load(st, pm, T, in >> 1, in & 1);                                                                      \
-        }                                                                                                              \
-        PHASE_MARK(1);                                                                                                 \
-        __syncthreads();                                                                                               \
-        PHASE_MARK(3);                                                                                                 \
+    for (int s = 0; s < total; s += 2) {
+        PHASE_SELECT((stA & 1) ? 0 : 4);
+        prepare(setA, s, stA);
+        PHASE_MARK(2);
+        __syncthreads();
+        PHASE_MARK(3);
+        if (s + 1 < total) {
+            PHASE_SELECT((stB & 1) ? 0 : 4);
+            prepare(setB, s + 1, stB);
+            PHASE_MARK(2);
+            __syncthreads();
+            PHASE_MARK(3);
+        }
     }
-    for (int s2 = 0; s2 < total; s2 += 2) {
-        T2FW_SPLIT_ITERATION(s2, stA, inA)
-        if (s2 + 1 < total) T2FW_SPLIT_ITERATION(s2 + 1, stB, inB)
-    }
-#undef T2FW_SPLIT_ITERATION
     // Both workgroups of a row see all four gates' blocks and reach the same verdict, so either
     // order of their writes leaves the same flag.
     if (bad) p.row_flags[b] = 1;
@@ -370,39 +369,44 @@ __device__ __forceinline__ void split_matrix_waves(const ChunkBwdArgs &p, unsign
     float carry = 0.f;
     int s = 0;
     if (tid == 0) p.row_flags[b] = 0;
-    __syncthreads();      // raw inputs of the first stages are in LDS
-    __syncthreads();      // operand tiles of stage 0 are in LDS
     PHASE_BEGIN();
 
+    // every stage starts with the workgroup barrier that publishes its operand tiles
     for (int64_t chunk = NC - 1; chunk >= 0; --chunk) {
         const int nb = chunk == NC - 1 ? nb_last : NB;
         take_state(pf, S);
         if (chunk > 0) load_state(ckpt + (chunk - 1) * (CH_N * CH_N), pf);
-        // ---- R stages: block-start states, forward in time
+        // ---- R stages: block-start states, forward in time, two blocks per stage
 #pragma unroll
-        for (int i = 0; i < NB; ++i) {
-            if (i < nb) {
-                const unsigned char *stage = smem + (s & 1) * STAGE_BYTES;
-                const u16 *VOHc = reinterpret_cast<const u16 *>(stage + OFF_CM + CM_VOH * CM_TILE);
-                const u16 *VHc = reinterpret_cast<const u16 *>(stage + OFF_CM + CM_VH * CM_TILE);
-                const float *LX = reinterpret_cast<const float *>(stage + OFF_LX);
-                const float *LO = reinterpret_cast<const float *>(stage + OFF_LO);
-                {
-                    const uint2 a0 = pack4v<OPE>(S[0]), a1 = pack4v<OPE>(S[1]), a2 = pack4v<OPE>(S[2]), a3 = pack4v<OPE>(S[3]);
-                    sv[i][0] = cat(a0, a1);
-                    sv[i][1] = cat(a2, a3);
-                }
-                const float lo = LO[ch];
-                const uint2 vhc = ld2(VHc + ch * CC + 4 * g);
-#pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    const float4 lx = *reinterpret_cast<const float4 *>(LX + 16 * j + 4 * g);
-                    S[j][0] *= lo * lx.x; S[j][1] *= lo * lx.y; S[j][2] *= lo * lx.z; S[j][3] *= lo * lx.w;
-                    S[j] = OPE::mfma16(ld2(VOHc + (16 * j + r) * CC + 4 * g), vhc, S[j]);
-                }
-                PHASE_MARK(0);
+        for (int i2 = 0; i2 < NB; i2 += 2) {
+            if (i2 < nb) {
                 __syncthreads();
                 PHASE_MARK(3);
+                const unsigned char *stage = smem + (s & 1) * STAGE_BYTES;
+#pragma unroll
+                for (int jb = 0; jb < 2; ++jb) {
+                    const int i = i2 + jb;
+                    if (i < nb) {
+                        const u16 *VOHc = reinterpret_cast<const u16 *>(stage + OFF_CM + (2 * jb) * CM_TILE);
+                        const u16 *VHc = reinterpret_cast<const u16 *>(stage + OFF_CM + (2 * jb + 1) * CM_TILE);
+                        const float *LX = lv_vec(stage, jb, 0), *LO = lv_vec(stage, jb, 1);
+                        {
+                            const uint2 a0 = pack4v<OPE>(S[0]), a1 = pack4v<OPE>(S[1]), a2 = pack4v<OPE>(S[2]),
+                                        a3 = pack4v<OPE>(S[3]);
+                            sv[i][0] = cat(a0, a1);
+                            sv[i][1] = cat(a2, a3);
+                        }
+                        const float lo = LO[ch];
+                        const uint2 vhc = ld2(VHc + ch * CC + 4 * g);
+#pragma unroll
+                        for (int j = 0; j < 4; ++j) {
+                            const float4 lx = *reinterpret_cast<const float4 *>(LX + 16 * j + 4 * g);
+                            S[j][0] *= lo * lx.x; S[j][1] *= lo * lx.y; S[j][2] *= lo * lx.z; S[j][3] *= lo * lx.w;
+                            S[j] = OPE::mfma16(ld2(VOHc + (16 * j + r) * CC + 4 * g), vhc, S[j]);
+                        }
+                    }
+                }
+                PHASE_MARK(0);
                 ++s;
             }
         }
@@ -421,6 +425,8 @@ __device__ __forceinline__ void split_matrix_waves(const ChunkBwdArgs &p, unsign
 #pragma unroll
         for (int i = NB - 1; i >= 0; --i) {
             if (i < nb) {
+                __syncthreads();
+                PHASE_MARK(2);
                 const unsigned char *stage = smem + (s & 1) * STAGE_BYTES;
                 const u16 *AOS = reinterpret_cast<const u16 *>(stage + OFF_TM + TM_AOS * TM_TILE);
                 const u16 *VOT = reinterpret_cast<const u16 *>(stage + OFF_TM + TM_VOT * TM_TILE);
@@ -428,8 +434,7 @@ __device__ __forceinline__ void split_matrix_waves(const ChunkBwdArgs &p, unsign
                 const u16 *AOSc = reinterpret_cast<const u16 *>(stage + OFF_CM + CM_AOS * CM_TILE);
                 const u16 *ASc = reinterpret_cast<const u16 *>(stage + OFF_CM + CM_AS * CM_TILE);
                 const u16 *VTc = reinterpret_cast<const u16 *>(stage + OFF_CM + CM_VT * CM_TILE);
-                const float *LX = reinterpret_cast<const float *>(stage + OFF_LX);
-                const float *LO = reinterpret_cast<const float *>(stage + OFF_LO);
+                const float *LX = lv_vec(stage, 0, 0), *LO = lv_vec(stage, 0, 1);
                 const floatx4 zero = {0.f, 0.f, 0.f, 0.f};
                 // the 16x16 token-token product, in both orientations (full contraction over 64 channels)
                 const int ro = r * TS + 8 * g;
@@ -498,8 +503,6 @@ __device__ __forceinline__ void split_matrix_waves(const ChunkBwdArgs &p, unsign
                     }
                 }
                 PHASE_MARK(1);
-                __syncthreads();
-                PHASE_MARK(2);
                 ++s;
             }
         }
@@ -537,7 +540,8 @@ template <typename IOE, typename OPE, int NB> int launch(const ChunkBwdArgs &a, 
                        "hipFuncSetAttribute(split backward chunk kernel)");
     if (rc) return rc;
     if (a.B > 0x1fffffffLL) return fail(T2FW_ERR_UNSUPPORTED, "B=%lld is too large", (long long)a.B);
-    if (a.T >= CHUNK_SPLIT_MAX_T) return fail(T2FW_ERR_UNSUPPORTED, "T=%lld is too long for 32-bit row offsets", (long long)a.T);
+    if (a.T >= CHUNK_SPLIT_MAX_T || a.T % CH_L != 0)
+        return fail(T2FW_ERR_UNSUPPORTED, "the split backward kernel takes T %% 16 == 0, T < 2^24 (T=%lld)", (long long)a.T);
     const int rows_padded = (int)((a.B + 7) / 8 * 8);
     hipLaunchKernelGGL(kern, dim3(2u * (unsigned)rows_padded), dim3(SP_THREADS), SP_SMEM, stream, a, rows_padded);
     return check_hip(hipGetLastError(), "lfw_bwd_split_kernel launch");
