@@ -271,7 +271,7 @@ __device__ __forceinline__ void split_prep_waves(const ChunkBwdArgs &p, unsigned
     const int total = sched.total;
     u32 bad = 0;
 
-    auto issue = [&](RawSet &r, int st) {          // raw inputs of stage st (wave-uniform) -> registers
+    auto issue = [&](RawSet &r, int st, int c) {   // raw inputs of stage st (wave-uniform) -> registers
         const int tok = st >> 1;
         if (st & 1) {
             raw_issue(r, b_gate + (u32)tok * CH_N, b_val + (u32)tok * CH_N, h, c);
@@ -286,10 +286,18 @@ __device__ __forceinline__ void split_prep_waves(const ChunkBwdArgs &p, unsigned
     auto prepare = [&](RawSet &r, int s, int &st_io) {
         const int st = st_io;
         const RawF fr = raw_take<IOE>(r);
-        if (s + 2 < total) {
-            st_io = sched.at(s + 2);
-            issue(r, st_io);
-        }
+        // The loads that refill r must come after the conversions above, or they need registers
+        // (and a wait) of their own: tie their address to the converted values.
+        int cdep = c;
+        asm volatile("" : "+v"(cdep)
+                     : "v"(fr.gown[0]), "v"(fr.gown[1]), "v"(fr.gown[2]), "v"(fr.gown[3]), "v"(fr.gown[4]),
+                       "v"(fr.gown[5]), "v"(fr.gown[6]), "v"(fr.gown[7]), "v"(fr.val[0]), "v"(fr.val[1]), "v"(fr.val[2]),
+                       "v"(fr.val[3]), "v"(fr.val[4]), "v"(fr.val[5]), "v"(fr.val[6]), "v"(fr.val[7]), "v"(fr.goth_prod),
+                       "v"(fr.bad));
+        // unconditional (past the end: the last stage again), so that the number of loads in flight
+        // is the same on every path and the waits for them can be exact
+        st_io = sched.at(min(s + 2, total - 1));
+        issue(r, st_io, cdep);
         unsigned char *stage = smem + (s & 1) * STAGE_BYTES;
         if (st & 1)
             prep_b<OPE>(fr, stage, role, h, c, side == 1, bad);
@@ -297,24 +305,40 @@ __device__ __forceinline__ void split_prep_waves(const ChunkBwdArgs &p, unsigned
             prep_r<OPE>(fr, stage, rj, rown, h, c, bad);
     };
 
+    // Stages alternate between two register sets.  The loop below always does a whole pair (set A,
+    // then set B), with no exit in between, so that the order of the loads in flight is the same
+    // on every path into it; an odd stage count peels the first stage off.
     RawSet setA, setB;
-    int stA = sched.at(0), stB = total > 1 ? sched.at(1) : stA;
-    issue(setA, stA);
-    if (total > 1) issue(setB, stB);
+    int stA, stB, s = 0;
     PHASE_BEGIN();
-    for (int s = 0; s < total; s += 2) {
+    if (total & 1) {
+        stB = sched.at(0);
+        stA = sched.at(min(1, total - 1));
+        issue(setB, stB, c);
+        issue(setA, stA, c);
+        PHASE_SELECT((stB & 1) ? 0 : 4);
+        prepare(setB, 0, stB);
+        PHASE_MARK(2);
+        __syncthreads();
+        PHASE_MARK(3);
+        s = 1;
+    } else {
+        stA = sched.at(0);
+        stB = sched.at(1);
+        issue(setA, stA, c);
+        issue(setB, stB, c);
+    }
+    for (; s < total; s += 2) {
         PHASE_SELECT((stA & 1) ? 0 : 4);
         prepare(setA, s, stA);
         PHASE_MARK(2);
         __syncthreads();
         PHASE_MARK(3);
-        if (s + 1 < total) {
-            PHASE_SELECT((stB & 1) ? 0 : 4);
-            prepare(setB, s + 1, stB);
-            PHASE_MARK(2);
-            __syncthreads();
-            PHASE_MARK(3);
-        }
+        PHASE_SELECT((stB & 1) ? 0 : 4);
+        prepare(setB, s + 1, stB);
+        PHASE_MARK(2);
+        __syncthreads();
+        PHASE_MARK(3);
     }
     // Both workgroups of a row see all four gates' blocks and reach the same verdict, so either
     // order of their writes leaves the same flag.
