@@ -98,6 +98,30 @@ template <int NB> struct SplitSchedule {
     }
 };
 
+// The same schedule as a forward iterator (no divisions): cur() is SplitSchedule::at of the stage
+// it stands on; advancing past the last stage leaves it there.
+template <int NB> struct StageIter {
+    int chunk, local, nb, C, left;      // left: stages after the current one
+    __device__ StageIter(const SplitSchedule<NB> &sc) : chunk(sc.NC - 1), local(0), nb(sc.nb_last), C(sc.C), left(sc.total - 1) {}
+    __device__ void advance() {
+        if (left > 0) {
+            --left;
+            ++local;
+            if (local == (nb + 1) / 2 + nb) {
+                --chunk;
+                local = 0;
+                nb = NB;
+            }
+        }
+    }
+    __device__ int cur() const {
+        const int nr = (nb + 1) / 2;
+        const bool bmode = local >= nr;
+        const int block = bmode ? nb - 1 - (local - nr) : 2 * local;
+        return ((chunk * C + block * CH_L) << 1) | (bmode ? 1 : 0);
+    }
+};
+
 // ---- raw inputs --------------------------------------------------------------------------
 // A prep thread works on one channel and eight tokens; it needs the gate at those tokens, the
 // gate at the block's other eight tokens and one value (or adjoint) array at its own tokens:
@@ -107,14 +131,18 @@ struct RawSet {
     u16 gown[8], goth[8], val[8];
 };
 
-__device__ __forceinline__ void raw_issue(RawSet &r, const u16 *gate, const u16 *val, int h, int c) {
-    const u16 *go = gate + 8 * h * CH_N + c, *gx = gate + 8 * (1 - h) * CH_N + c, *va = val + 8 * h * CH_N + c;
+// gate, val: wave-uniform addresses of the block's first token; lane_bytes = 2 * channel
+__device__ __forceinline__ void raw_issue(RawSet &r, const u16 *gate, const u16 *val, int h, u32 lane_bytes) {
+    auto at = [&](const u16 *base, int tok) -> const u16 * {
+        return reinterpret_cast<const u16 *>(reinterpret_cast<const unsigned char *>(base + tok * CH_N) + lane_bytes);
+    };
+    const u16 *go = at(gate, 8 * h), *gx = at(gate, 8 * (1 - h)), *va = at(val, 8 * h);
 #pragma unroll
-    for (int t = 0; t < 8; ++t) {
-        r.gown[t] = go[t * CH_N];
-        r.goth[t] = gx[t * CH_N];
-        r.val[t] = va[t * CH_N];
-    }
+    for (int t = 0; t < 8; ++t) r.goth[t] = gx[t * CH_N];
+#pragma unroll
+    for (int t = 0; t < 8; ++t) r.gown[t] = go[t * CH_N];
+#pragma unroll
+    for (int t = 0; t < 8; ++t) r.val[t] = va[t * CH_N];
 }
 
 template <typename IOE> __device__ __forceinline__ u32 gate_check8(const u16 (&g)[8]) {
@@ -127,18 +155,30 @@ template <typename IOE> __device__ __forceinline__ u32 gate_check8(const u16 (&g
     return (mx >= IOE::ONE_BITS) ? 1u : 0u;
 }
 
-template <typename OPE>
-__device__ __forceinline__ void write_tm8(unsigned char *stage, int tile, int c, int t0, const float (&v)[8]) {
-    u16 *tm = reinterpret_cast<u16 *>(stage + OFF_TM + tile * TM_TILE) + t0 * TS + tm_pos(c);
+// eight tokens of one channel as four packed pairs
+struct Packed8 {
+    u32 p[4];
+};
+template <typename OPE> __device__ __forceinline__ Packed8 pack8(const float (&v)[8]) {
+    Packed8 r;
 #pragma unroll
-    for (int t = 0; t < 8; ++t) tm[t * TS] = cvt1<OPE>(v[t]);
+    for (int i = 0; i < 4; ++i) r.p[i] = OPE::pack2(v[2 * i], v[2 * i + 1]);
+    return r;
 }
 
-template <typename OPE>
-__device__ __forceinline__ void write_cm8(unsigned char *stage, int tile, int c, int t0, const float (&v)[8]) {
+__device__ __forceinline__ void write_tm8(unsigned char *stage, int tile, int c, int t0, const Packed8 &v) {
+    u16 *tm = reinterpret_cast<u16 *>(stage + OFF_TM + tile * TM_TILE) + t0 * TS + tm_pos(c);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        tm[(2 * i) * TS] = (u16)(v.p[i] & 0xffffu);
+        tm[(2 * i + 1) * TS] = (u16)(v.p[i] >> 16);
+    }
+}
+
+__device__ __forceinline__ void write_cm8(unsigned char *stage, int tile, int c, int t0, const Packed8 &v) {
     uint2 *cm = reinterpret_cast<uint2 *>(stage + OFF_CM + tile * CM_TILE + (c * CC + t0) * 2);
-    cm[0] = packq<OPE>(v[0], v[1], v[2], v[3]);
-    cm[1] = packq<OPE>(v[4], v[5], v[6], v[7]);
+    cm[0] = make_uint2(v.p[0], v.p[1]);
+    cm[1] = make_uint2(v.p[2], v.p[3]);
 }
 
 __device__ __forceinline__ void write_cf8(unsigned char *stage, int tile, int c, int t0, const float (&v)[8]) {
@@ -153,9 +193,11 @@ struct RawF {
     u32 bad;      // own gates outside (0, 1]
 };
 
-template <typename IOE> __device__ __forceinline__ RawF raw_take(const RawSet &r) {
+template <typename IOE> __device__ __forceinline__ RawF raw_take(const RawSet &r, bool check) {
     RawF f;
-    f.bad = gate_check8<IOE>(r.gown);
+    // the loads complete in order: one wait for the last of them covers the whole set
+    asm volatile("" ::"v"(r.val[7]));
+    f.bad = check ? gate_check8<IOE>(r.gown) : 0u;
     float po = 1.0f;
 #pragma unroll
     for (int t = 0; t < 8; ++t) {
@@ -208,14 +250,15 @@ __device__ __forceinline__ void prep_b(const RawF &f, unsigned char *stage, int 
             pre[t] = run;
             v[t] = f.val[t] * run;
         }
+        const Packed8 vp = pack8<OPE>(v);
         if (other) {
-            write_tm8<OPE>(stage, TM_AOS, c, t0, v);
-            write_cm8<OPE>(stage, CM_AOS, c, t0, v);
+            write_tm8(stage, TM_AOS, c, t0, vp);
+            write_cm8(stage, CM_AOS, c, t0, vp);
         } else {
             float rg[8];
 #pragma unroll
             for (int t = 0; t < 8; ++t) rg[t] = __builtin_amdgcn_rcpf(f.gown[t]);
-            write_cm8<OPE>(stage, CM_AS, c, t0, v);
+            write_cm8(stage, CM_AS, c, t0, vp);
             write_cf8(stage, F_RG, c, t0, rg);
             if (want_pp) write_cf8(stage, F_PP, c, t0, pre);
         }
@@ -223,13 +266,14 @@ __device__ __forceinline__ void prep_b(const RawF &f, unsigned char *stage, int 
         float hat[8], til[8], inv[8];
         const float tot = suffix_scale<OPE>(f, h, hat, til, inv, bad);
         if (h == 0) lv_vec(stage, 0, other ? 0 : 1)[c] = tot;
+        const Packed8 hp = pack8<OPE>(hat), tp = pack8<OPE>(til);
         if (other) {
-            write_cm8<OPE>(stage, CM_VOH, c, t0, hat);
-            write_tm8<OPE>(stage, TM_VOH, c, t0, hat);
-            write_tm8<OPE>(stage, TM_VOT, c, t0, til);
+            write_cm8(stage, CM_VOH, c, t0, hp);
+            write_tm8(stage, TM_VOH, c, t0, hp);
+            write_tm8(stage, TM_VOT, c, t0, tp);
         } else {
-            write_cm8<OPE>(stage, CM_VH, c, t0, hat);
-            write_cm8<OPE>(stage, CM_VT, c, t0, til);
+            write_cm8(stage, CM_VH, c, t0, hp);
+            write_cm8(stage, CM_VT, c, t0, tp);
             write_cf8(stage, F_IP, c, t0, inv);
         }
     }
@@ -242,7 +286,7 @@ __device__ __forceinline__ void prep_r(const RawF &f, unsigned char *stage, int 
     float hat[8], til[8], inv[8];
     const float tot = suffix_scale<OPE>(f, h, hat, til, inv, bad);
     if (h == 0) lv_vec(stage, j, own)[c] = tot;
-    write_cm8<OPE>(stage, 2 * j + own, c, 8 * h, hat);
+    write_cm8(stage, 2 * j + own, c, 8 * h, pack8<OPE>(hat));
 }
 
 template <typename IOE, typename OPE, int NB>
@@ -271,33 +315,35 @@ __device__ __forceinline__ void split_prep_waves(const ChunkBwdArgs &p, unsigned
     const int total = sched.total;
     u32 bad = 0;
 
-    auto issue = [&](RawSet &r, int st, int c) {   // raw inputs of stage st (wave-uniform) -> registers
+    const u32 lane_bytes = 2u * (u32)c;
+    auto issue = [&](RawSet &r, int st, u32 lb) {   // raw inputs of stage st (wave-uniform) -> registers
         const int tok = st >> 1;
         if (st & 1) {
-            raw_issue(r, b_gate + (u32)tok * CH_N, b_val + (u32)tok * CH_N, h, c);
+            raw_issue(r, b_gate + (u32)tok * CH_N, b_val + (u32)tok * CH_N, h, lb);
         } else {
             // the second block of the last pair may lie past the end: read the last block instead
             // (its tiles are never used)
             const int t2 = min(tok + rj * CH_L, T - CH_L);
-            raw_issue(r, r_gate + (u32)t2 * CH_N, r_val + (u32)t2 * CH_N, h, c);
+            raw_issue(r, r_gate + (u32)t2 * CH_N, r_val + (u32)t2 * CH_N, h, lb);
         }
     };
-    // builds the tiles of stage s (= st); r then takes stage s+2, and st that stage's descriptor
-    auto prepare = [&](RawSet &r, int s, int &st_io) {
-        const int st = st_io;
-        const RawF fr = raw_take<IOE>(r);
+    // builds the tiles of stage s, which r holds and it stands on; r and it then move on two stages
+    auto prepare = [&](RawSet &r, int s, StageIter<NB> &it) {
+        const int st = it.cur();
+        const RawF fr = raw_take<IOE>(r, !(st & 1) || (role & 1));
         // The loads that refill r must come after the conversions above, or they need registers
         // (and a wait) of their own: tie their address to the converted values.
-        int cdep = c;
-        asm volatile("" : "+v"(cdep)
+        u32 lb = lane_bytes;
+        asm volatile("" : "+v"(lb)
                      : "v"(fr.gown[0]), "v"(fr.gown[1]), "v"(fr.gown[2]), "v"(fr.gown[3]), "v"(fr.gown[4]),
                        "v"(fr.gown[5]), "v"(fr.gown[6]), "v"(fr.gown[7]), "v"(fr.val[0]), "v"(fr.val[1]), "v"(fr.val[2]),
                        "v"(fr.val[3]), "v"(fr.val[4]), "v"(fr.val[5]), "v"(fr.val[6]), "v"(fr.val[7]), "v"(fr.goth_prod),
                        "v"(fr.bad));
         // unconditional (past the end: the last stage again), so that the number of loads in flight
         // is the same on every path and the waits for them can be exact
-        st_io = sched.at(min(s + 2, total - 1));
-        issue(r, st_io, cdep);
+        it.advance();
+        it.advance();
+        issue(r, it.cur(), lb);
         unsigned char *stage = smem + (s & 1) * STAGE_BYTES;
         if (st & 1)
             prep_b<OPE>(fr, stage, role, h, c, side == 1, bad);
@@ -309,33 +355,32 @@ __device__ __forceinline__ void split_prep_waves(const ChunkBwdArgs &p, unsigned
     // then set B), with no exit in between, so that the order of the loads in flight is the same
     // on every path into it; an odd stage count peels the first stage off.
     RawSet setA, setB;
-    int stA, stB, s = 0;
+    StageIter<NB> itA(sched), itB(sched);
+    int s = 0;
     PHASE_BEGIN();
     if (total & 1) {
-        stB = sched.at(0);
-        stA = sched.at(min(1, total - 1));
-        issue(setB, stB, c);
-        issue(setA, stA, c);
-        PHASE_SELECT((stB & 1) ? 0 : 4);
-        prepare(setB, 0, stB);
+        itA.advance();                  // B: stage 0, A: stage 1
+        issue(setB, itB.cur(), lane_bytes);
+        issue(setA, itA.cur(), lane_bytes);
+        PHASE_SELECT((itB.cur() & 1) ? 0 : 4);
+        prepare(setB, 0, itB);
         PHASE_MARK(2);
         __syncthreads();
         PHASE_MARK(3);
         s = 1;
     } else {
-        stA = sched.at(0);
-        stB = sched.at(1);
-        issue(setA, stA, c);
-        issue(setB, stB, c);
+        itB.advance();                  // A: stage 0, B: stage 1
+        issue(setA, itA.cur(), lane_bytes);
+        issue(setB, itB.cur(), lane_bytes);
     }
     for (; s < total; s += 2) {
-        PHASE_SELECT((stA & 1) ? 0 : 4);
-        prepare(setA, s, stA);
+        PHASE_SELECT((itA.cur() & 1) ? 0 : 4);
+        prepare(setA, s, itA);
         PHASE_MARK(2);
         __syncthreads();
         PHASE_MARK(3);
-        PHASE_SELECT((stB & 1) ? 0 : 4);
-        prepare(setB, s + 1, stB);
+        PHASE_SELECT((itB.cur() & 1) ? 0 : 4);
+        prepare(setB, s + 1, itB);
         PHASE_MARK(2);
         __syncthreads();
         PHASE_MARK(3);
