@@ -396,8 +396,7 @@ __device__ __forceinline__ void split_matrix_waves(const ChunkBwdArgs &p, unsign
                                                    int side) {
     const int w = tid >> 6, l = tid & 63, r = l & 15, g = l >> 4;
     const int ch = 16 * w + r;       // this lane's own-side channel
-    const int T = (int)p.T;                              // the launcher admits T < 2^24 only
-    const int64_t NC = p.NC;
+    const int64_t NC = p.NC;                             // (the launcher admits T < 2^24, T % 16 == 0 only)
     const int C = p.C;
     const u16 *ckpt = reinterpret_cast<const u16 *>(p.ckpt) + b * NC * (CH_N * CH_N);
     const int nb_last = (int)((p.T - (NC - 1) * C + CH_L - 1) / CH_L);
@@ -486,9 +485,7 @@ __device__ __forceinline__ void split_matrix_waves(const ChunkBwdArgs &p, unsign
             for (int j = 0; j < 4; ++j)
 #pragma unroll
                 for (int i = 0; i < 4; ++i) us += G[j][i] * S[j][i];
-            us += __shfl_xor(us, 16, 64);
-            us += __shfl_xor(us, 32, 64);
-            carry = us;
+            carry = row_sums(us).all;
         }
         // ---- B stages: blocks last to first
 #pragma unroll
@@ -548,27 +545,25 @@ __device__ __forceinline__ void split_matrix_waves(const ChunkBwdArgs &p, unsign
                     unpack4<OPE>(vtc, vtv);
 #pragma unroll
                     for (int ii = 0; ii < 4; ++ii) du[ii] = oa[ii] * asv[ii] - va[ii] * vtv[ii];
-                    reverse_running_sum(du, carry, g, r);
+                    reverse_running_sum_swap(du, carry, g);
                     const float *cf = reinterpret_cast<const float *>(stage + OFF_CF) + ch * CC + 4 * g;
                     const float4 rg = *reinterpret_cast<const float4 *>(cf + F_RG * (CF_TILE / 4));
                     const float4 ip = *reinterpret_cast<const float4 *>(cf + F_IP * (CF_TILE / 4));
                     const float rgv[4] = {rg.x, rg.y, rg.z, rg.w}, ipv[4] = {ip.x, ip.y, ip.z, ip.w};
-                    // 16 lanes write 32 contiguous bytes of a token row; the four waves complete the row
-                    const int tg = (int)chunk * C + i * CH_L + 4 * g;         // this lane's first token
-                    const u32 go = (u32)tg * CH_N + (u32)ch;
+                    // 16 lanes write 32 contiguous bytes of a token row; the four waves complete the row.
+                    // T is a multiple of 16, so every token of the block exists.
+                    const u32 go = (u32)((int)chunk * C + i * CH_L + 4 * g) * CH_N + (u32)ch;
 #pragma unroll
                     for (int ii = 0; ii < 4; ++ii) {
-                        if (tg + ii < T) {
-                            d_val[go + ii * CH_N] = cvt1<IOE>(ipv[ii] * (va[ii] + asv[ii] * pd[ii]));
-                            d_gate[go + ii * CH_N] = cvt1<IOE>(du[ii] * rgv[ii]);
-                        }
+                        d_val[go + ii * CH_N] = cvt1<IOE>(ipv[ii] * (va[ii] + asv[ii] * pd[ii]));
+                        d_gate[go + ii * CH_N] = cvt1<IOE>(du[ii] * rgv[ii]);
                     }
                     if (side == 1) {
                         const float4 pp = *reinterpret_cast<const float4 *>(cf + F_PP * (CF_TILE / 4));
                         const float ppv[4] = {pp.x, pp.y, pp.z, pp.w};
 #pragma unroll
                         for (int ii = 0; ii < 4; ++ii)
-                            if (tg + ii < T) d_adj[go + ii * CH_N] = cvt1<IOE>(ppv[ii] * (oa[ii] + vtv[ii] * pd[ii]));
+                            d_adj[go + ii * CH_N] = cvt1<IOE>(ppv[ii] * (oa[ii] + vtv[ii] * pd[ii]));
                     }
                 }
                 PHASE_MARK(1);
