@@ -145,7 +145,7 @@ int t2fw_lfw_forward(const void *x, const void *f, const void *q, const void *k,
     a.C = ckpt ? C : 1;
     a.NC = ckpt ? t2fw_lfw_num_ckpt(T, C) : 1;
 
-    if (chunk_shape_ok(D, K, dtype, flags) && (ckpt == nullptr || C % 32 == 0) &&
+    if (chunk_shape_ok(D, K, dtype, flags) && (ckpt == nullptr || C % 32 == 0) && T < CHUNK_MAX_T &&
         aligned16({x, f, q, k, f_key, s0, out, next_state, ckpt})) {
         if (workspace == nullptr || workspace_bytes < row_flag_bytes(B))
             return fail(T2FW_ERR_WORKSPACE, "workspace of %zu bytes needed, %zu given", row_flag_bytes(B),
@@ -208,7 +208,7 @@ int t2fw_lfw_backward(const void *g_out, const void *g_state, const void *x, con
         c.row_flags = static_cast<int32_t *>(workspace);
         c.B = B; c.T = T; c.NC = a.NC; c.C = C;
         const int op = (dtype == T2FW_F16 && (flags & T2FW_FLAG_FP16_OPERANDS)) ? 1 : 0;
-        const bool split_ok = T < CHUNK_SPLIT_MAX_T && T % 16 == 0;
+        const bool split_ok = T < CHUNK_MAX_T && T % 16 == 0;
         bool split = (flags & T2FW_FLAG_BWD_SPLIT) != 0 && split_ok;
         if ((flags & (T2FW_FLAG_BWD_SPLIT | T2FW_FLAG_BWD_WHOLE_ROW)) == 0) {
             const int cus = compute_units();

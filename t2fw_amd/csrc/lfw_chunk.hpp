@@ -43,7 +43,7 @@ int chunk_forward(const ChunkFwdArgs &a, int dtype, int op, hipStream_t stream);
 int chunk_backward(const ChunkBwdArgs &a, int dtype, int op, hipStream_t stream);
 // same result from two workgroups per batch row (one per side of the state); for batches that leave CUs idle
 int chunk_backward_split(const ChunkBwdArgs &a, int dtype, int op, hipStream_t stream);
-constexpr int64_t CHUNK_SPLIT_MAX_T = 1 << 24;      // the split kernel addresses a batch row with 32-bit offsets
+constexpr int64_t CHUNK_MAX_T = 1 << 24;      // the forward and the split backward kernel address a batch row with 32-bit offsets
 
 #if defined(__HIPCC__)
 
@@ -116,6 +116,12 @@ constexpr int CH_N = 64;        // D = K = 64
 constexpr int TS = 72;          // token-major tiles [32 tokens][64 ch] of 16-bit: row stride
 constexpr int CS = 36;          // channel-major tiles [64 ch][32 tokens] of 16-bit / fp32: row stride
 constexpr int OS = 68;          // output tile [32 tokens][64 ch] of 16-bit: row stride
+
+// Position of channel c = 16j + 4g + e inside the row of a token-major tile whose rows are also
+// contracted against a wave's own accumulators: 16g + 4j + e.  The 16 values lane (r, g) pairs
+// with its accumulator elements (channels 16j + 4g + e, j = 0..3) are then contiguous (two
+// 16-byte reads).  Products between two such tiles are indifferent to the order.
+__device__ __forceinline__ int tm_pos(int c) { return 16 * ((c >> 2) & 3) + 4 * (c >> 4) + (c & 3); }
 
 #endif  // __HIPCC__
 

@@ -59,11 +59,6 @@ __device__ __forceinline__ const float *lv_vec(const unsigned char *stage, int j
     return reinterpret_cast<const float *>(stage + OFF_LV) + (2 * j + own) * CH_N;
 }
 
-// Position of channel c = 16j + 4g + e inside a token-major row: 16g + 4j + e.  The 16 values a
-// lane contracts against its own accumulators (channels 16j + 4g + e, j = 0..3) are then
-// contiguous.  Products between two token-major tiles are indifferent to the order.
-__device__ __forceinline__ int tm_pos(int c) { return 16 * ((c >> 2) & 3) + 4 * (c >> 4) + (c & 3); }
-
 // ---- stage schedule ----------------------------------------------------------------------
 // Chunks are visited from the last one down; a chunk with nb blocks takes ceil(nb/2) "R"
 // stages of two blocks each (forward in time), then nb "B" stages (blocks nb-1..0).
@@ -604,7 +599,7 @@ template <typename IOE, typename OPE, int NB> int launch(const ChunkBwdArgs &a, 
                        "hipFuncSetAttribute(split backward chunk kernel)");
     if (rc) return rc;
     if (a.B > 0x1fffffffLL) return fail(T2FW_ERR_UNSUPPORTED, "B=%lld is too large", (long long)a.B);
-    if (a.T >= CHUNK_SPLIT_MAX_T || a.T % CH_L != 0)
+    if (a.T >= CHUNK_MAX_T || a.T % CH_L != 0)
         return fail(T2FW_ERR_UNSUPPORTED, "the split backward kernel takes T %% 16 == 0, T < 2^24 (T=%lld)", (long long)a.T);
     const int rows_padded = (int)((a.B + 7) / 8 * 8);
     hipLaunchKernelGGL(kern, dim3(2u * (unsigned)rows_padded), dim3(SP_THREADS), SP_SMEM, stream, a, rows_padded);

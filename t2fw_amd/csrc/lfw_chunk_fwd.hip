@@ -1,9 +1,12 @@
 // Forward scan of the decay rule in chunked matrix-core form (see lfw_chunk.hpp for the
-// algebra).  One workgroup owns one batch row; matrix wave w keeps the 64 x 16
-// slab S[:, 16w:16w+16] of the state in fp32 accumulator registers for the whole
-// sequence.  Four more waves turn raw inputs into scaled 16-bit operand tiles in LDS, one
-// (channel, 16-token block) per thread and one 32-token step ahead of the MFMA phase;
-// raw inputs travel HBM -> registers (16-byte loads, two steps ahead) -> LDS -> per-channel columns.
+// algebra).  One workgroup of 12 waves owns one batch row.  Matrix wave w keeps the
+// 16 x 64 slab S[16w:16w+16, :] of the state in fp32 accumulator registers for the whole
+// sequence, runs the MFMA phase of a 32-token step and stores the outputs itself.  Eight
+// prep waves build the scaled 16-bit operand tiles of the next step in LDS: a wave takes
+// one side (key or value), one of the step's two 16-token blocks and eight of its tokens,
+// a lane one channel.  Raw inputs go from global memory straight to the prep waves'
+// registers (two-byte loads, coalesced over the wave's 64 channels), two steps ahead of
+// their use; one workgroup barrier per step hands the double-buffered tiles over.
 //
 // Replaces lfw_cuda_fwd_kernel + the output einsum of the reference
 // (t2fw/csrc/lfw_kernel.cu:18-59, t2fw/csrc/lfw.cpp:45); semantics t2fw/torch.py:21-31.
@@ -24,9 +27,11 @@
 namespace t2fw {
 namespace {
 
+constexpr int FWD_THREADS = 768;
+
 // ---- LDS layout of one operand buffer (bytes) -------------------------------------------
-constexpr int OFF_QT = 0;                                  // qs  token-major  [32][TS] u16
-constexpr int OFF_KT = OFF_QT + CH_STEP * TS * 2;          // kt  token-major  [32][TS] u16
+constexpr int OFF_QT = 0;                                  // qs  token-major  [32][TS] u16, channels at tm_pos
+constexpr int OFF_KT = OFF_QT + CH_STEP * TS * 2;          // kt  token-major  [32][TS] u16, channels at tm_pos
 constexpr int OFF_KH = OFF_KT + CH_STEP * TS * 2;          // kh  channel-major [64][CS] u16
 constexpr int OFF_XT = OFF_KH + CH_N * CS * 2;             // xt  channel-major
 constexpr int OFF_XH = OFF_XT + CH_N * CS * 2;             // xh  channel-major
@@ -34,117 +39,244 @@ constexpr int OFF_AS = OFF_XH + CH_N * CS * 2;             // a_t channel-major 
 constexpr int OFF_BL = OFF_AS + CH_N * CS * 4;             // b_L [2][64] f32
 constexpr int OFF_AL = OFF_BL + 2 * CH_N * 4;              // a_L [2][64] f32
 constexpr int OPS_BYTES = OFF_AL + 2 * CH_N * 4;
-constexpr int OUT_BYTES = CH_STEP * OS * 2;
-constexpr int OFF_OUT = 2 * OPS_BYTES;
-// raw inputs of one step as they lie in HBM: 5 arrays [32 tokens][64 ch] u16 (f_key,k,q,f,x)
-constexpr int RAW_ARRAY = CH_STEP * CH_N * 2;
-constexpr int RAW_BYTES = 5 * RAW_ARRAY;
-constexpr int OFF_RAW = OFF_OUT + 2 * OUT_BYTES;
-constexpr int FWD_SMEM = OFF_RAW + 2 * RAW_BYTES;
+constexpr int FWD_SMEM = 2 * OPS_BYTES;
+static_assert(OPS_BYTES % 16 == 0, "operand buffers must keep 16-byte alignment");
 
-struct Raw {
-    u16 g[CH_L];   // gate  (f_key or f)
-    u16 a[CH_L];   // k or x
-    u16 u[CH_L];   // q (key side only)
+// ---- raw inputs --------------------------------------------------------------------------
+// One prep lane: the gate at its eight tokens, the gate at the block's other eight tokens, and
+// NV value arrays (key side: k and q, value side: x) at its own tokens.
+template <int NV> struct RawSet {
+    u16 gown[8], goth[8], val[NV][8];
 };
 
-// One step of raw inputs in flight: thread (token = tid/8, piece = tid%8) carries the
-// 16-byte piece [token][8*piece .. 8*piece+8) of each of the five arrays.
-struct Stage {
-    uint4 v[5];
-};
-
-template <typename IOE>
-__device__ __forceinline__ void stage_load(Stage &st, const u16 *const (&src)[5], int64_t row_base, int64_t T,
-                                           int64_t step, int tid) {
-    const int tok = tid >> 3, piece = tid & 7;
-    const int64_t t = step * CH_STEP + tok;
-    if (t < T) {
-        const int64_t o = (row_base + t) * CH_N + 8 * piece;
+// gate, val0, val1 (NV = 2 only): wave-uniform addresses of token 0 of the batch row; tok_own / tok_oth: first of the
+// eight own / other tokens; lane_bytes = 2 * channel.  Tokens past the end of the sequence are
+// read from the last one (and replaced when the set is taken), with the same number of loads as
+// the fast path, so that the count of loads in flight does not depend on the path.
+template <int NV>
+__device__ __forceinline__ void raw_issue(RawSet<NV> &r, const u16 *gate, const u16 *val0, const u16 *val1, int tok_own,
+                                          int tok_oth, int T, u32 lane_bytes) {
+    const u16 *const val[2] = {val0, val1};
+    auto at = [&](const u16 *base, int tok) -> const u16 * {
+        return reinterpret_cast<const u16 *>(reinterpret_cast<const unsigned char *>(base + (u32)tok * CH_N) + lane_bytes);
+    };
+    if (max(tok_own, tok_oth) + 8 <= T) {
+        const u16 *go = at(gate, tok_own), *gx = at(gate, tok_oth);
 #pragma unroll
-        for (int a = 0; a < 5; ++a) st.v[a] = *reinterpret_cast<const uint4 *>(src[a] + o);
+        for (int t = 0; t < 8; ++t) r.goth[t] = gx[t * CH_N];
+#pragma unroll
+        for (int t = 0; t < 8; ++t) r.gown[t] = go[t * CH_N];
+#pragma unroll
+        for (int a = 0; a < NV; ++a) {
+            const u16 *va = at(val[a], tok_own);
+#pragma unroll
+            for (int t = 0; t < 8; ++t) r.val[a][t] = va[t * CH_N];
+        }
     } else {
-        // steps past the end act as identity: gates 1, everything else 0
-        const u32 one2 = (u32)IOE::ONE_BITS * 0x10001u;
 #pragma unroll
-        for (int a = 0; a < 5; ++a) st.v[a] = make_uint4(0, 0, 0, 0);
-        st.v[0] = make_uint4(one2, one2, one2, one2);
-        st.v[3] = make_uint4(one2, one2, one2, one2);
+        for (int t = 0; t < 8; ++t) r.goth[t] = *at(gate, min(tok_oth + t, T - 1));
+#pragma unroll
+        for (int t = 0; t < 8; ++t) r.gown[t] = *at(gate, min(tok_own + t, T - 1));
+#pragma unroll
+        for (int a = 0; a < NV; ++a)
+#pragma unroll
+            for (int t = 0; t < 8; ++t) r.val[a][t] = *at(val[a], min(tok_own + t, T - 1));
     }
 }
 
-__device__ __forceinline__ void stage_store(const Stage &st, unsigned char *raw, int tid) {
-#pragma unroll
-    for (int a = 0; a < 5; ++a) *reinterpret_cast<uint4 *>(raw + a * RAW_ARRAY + tid * 16) = st.v[a];
-}
+template <int NV> struct RawF {
+    float gown[8], goth_prod, val[NV][8];
+    u32 bad;      // own gates outside (0, 1]
+};
 
-// channel c, block h: this thread's column of the raw tiles
-__device__ __forceinline__ void raw_read(Raw &r, const unsigned char *raw, bool kside, int h, int c) {
-    const u16 *base = reinterpret_cast<const u16 *>(raw + (kside ? 0 : 3) * RAW_ARRAY) + (CH_L * h) * CH_N + c;
-#pragma unroll
-    for (int t = 0; t < CH_L; ++t) {
-        r.g[t] = base[t * CH_N];
-        r.a[t] = base[RAW_ARRAY / 2 + t * CH_N];
-        if (kside) r.u[t] = base[RAW_ARRAY + t * CH_N];
-    }
-}
-
-// One thread: channel c of one side, block h of the step -> operand tiles.
-template <typename IOE, typename OPE>
-__device__ __forceinline__ void prep_block(const Raw &r, bool kside, int h, int c, unsigned char *ops, u32 &bad) {
-    float gate[CH_L], pre[CH_L];
+// Registers -> floats; tokens past the end act as identity (gate 1, everything else 0).
+template <typename IOE, int NV>
+__device__ __forceinline__ RawF<NV> raw_take(const RawSet<NV> &r, int tok_own, int tok_oth, int T) {
+    RawF<NV> f;
+    // the loads complete in order: one wait for the last of them covers the whole set
+    asm volatile("" ::"v"(r.val[NV - 1][7]));
     u16 mx = 0;
+    float po = 1.0f;
 #pragma unroll
-    for (int t = 0; t < CH_L; ++t) {
-        gate[t] = IOE::to_f32(r.g[t]);
-        const u16 m1 = (u16)(r.g[t] - 1);     // gates must lie in (0, 1]: 0 < bits <= bits(1.0)
+    for (int t = 0; t < 8; ++t) {
+        const u16 m1 = (u16)(r.gown[t] - 1);      // gates must lie in (0, 1]: 0 < bits <= bits(1.0)
         mx = m1 > mx ? m1 : mx;
+        f.gown[t] = IOE::to_f32(r.gown[t]);
+        po *= IOE::to_f32(r.goth[t]);
+#pragma unroll
+        for (int a = 0; a < NV; ++a) f.val[a][t] = IOE::to_f32(r.val[a][t]);
     }
-    bad |= (mx >= IOE::ONE_BITS) ? 1u : 0u;
-    pre[0] = gate[0];
+    f.bad = (mx >= IOE::ONE_BITS) ? 1u : 0u;
+    f.goth_prod = po;
+    if (max(tok_own, tok_oth) + 8 > T) {          // wave-uniform, last step of the sequence only
+        po = 1.0f;
+        mx = 0;
 #pragma unroll
-    for (int t = 1; t < CH_L; ++t) pre[t] = pre[t - 1] * gate[t];
-    const float pL = pre[CH_L - 1];
-    bad |= (pL >= OPE::MIN_PRODUCT) ? 0u : 1u;
-    const float ipL = __builtin_amdgcn_rcpf(pL);
-    float hat[CH_L], til[CH_L];
-    float sfx = 1.0f;
+        for (int t = 0; t < 8; ++t) {
+            if (tok_oth + t < T) po *= IOE::to_f32(r.goth[t]);
+            if (tok_own + t < T) {
+                const u16 m1 = (u16)(r.gown[t] - 1);
+                mx = m1 > mx ? m1 : mx;
+            } else {
+                f.gown[t] = 1.0f;
 #pragma unroll
-    for (int t = CH_L - 1; t >= 0; --t) {
-        hat[t] = IOE::to_f32(r.a[t]) * sfx;      // scaled to the block end   (<= |a|)
-        til[t] = hat[t] * ipL;                   // scaled to the block start (a / prefix)
-        sfx *= gate[t];
-    }
-    const int tok0 = CH_L * h;
-    if (kside) {
-        u16 *QT = reinterpret_cast<u16 *>(ops + OFF_QT);
-        u16 *KT = reinterpret_cast<u16 *>(ops + OFF_KT);
-#pragma unroll
-        for (int t = 0; t < CH_L; ++t) {
-            QT[(tok0 + t) * TS + c] = cvt1<OPE>(IOE::to_f32(r.u[t]) * pre[t]);
-            KT[(tok0 + t) * TS + c] = cvt1<OPE>(til[t]);
+                for (int a = 0; a < NV; ++a) f.val[a][t] = 0.0f;
+            }
         }
-        uint2 *KH = reinterpret_cast<uint2 *>(ops + OFF_KH + (c * CS + tok0) * 2);
-#pragma unroll
-        for (int t = 0; t < CH_L; t += 4)
-            KH[t / 4] = make_uint2(OPE::pack2(hat[t], hat[t + 1]), OPE::pack2(hat[t + 2], hat[t + 3]));
-        reinterpret_cast<float *>(ops + OFF_BL)[h * CH_N + c] = pL;
-    } else {
-        uint2 *XT = reinterpret_cast<uint2 *>(ops + OFF_XT + (c * CS + tok0) * 2);
-        uint2 *XH = reinterpret_cast<uint2 *>(ops + OFF_XH + (c * CS + tok0) * 2);
-        float4 *AS = reinterpret_cast<float4 *>(ops + OFF_AS + (c * CS + tok0) * 4);
-#pragma unroll
-        for (int t = 0; t < CH_L; t += 4) {
-            XT[t / 4] = make_uint2(OPE::pack2(til[t], til[t + 1]), OPE::pack2(til[t + 2], til[t + 3]));
-            XH[t / 4] = make_uint2(OPE::pack2(hat[t], hat[t + 1]), OPE::pack2(hat[t + 2], hat[t + 3]));
-            AS[t / 4] = make_float4(pre[t], pre[t + 1], pre[t + 2], pre[t + 3]);
-        }
-        reinterpret_cast<float *>(ops + OFF_AL)[h * CH_N + c] = pL;
+        f.bad = (mx >= IOE::ONE_BITS) ? 1u : 0u;
+        f.goth_prod = po;
     }
+    return f;
 }
 
-template <typename E>
-__device__ __forceinline__ uint2 pack4(const floatx4 &v) {
+// eight tokens of one channel as four packed pairs
+struct Packed8 {
+    u32 p[4];
+};
+template <typename OPE> __device__ __forceinline__ Packed8 pack8(const float (&v)[8]) {
+    Packed8 r;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) r.p[i] = OPE::pack2(v[2 * i], v[2 * i + 1]);
+    return r;
+}
+// token-major: tile[(tok0 + t) * TS + tm_pos(c)]
+__device__ __forceinline__ void write_tm8(unsigned char *tile, int c, int tok0, const Packed8 &v) {
+    u16 *tm = reinterpret_cast<u16 *>(tile) + tok0 * TS + tm_pos(c);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        tm[(2 * i) * TS] = (u16)(v.p[i] & 0xffffu);
+        tm[(2 * i + 1) * TS] = (u16)(v.p[i] >> 16);
+    }
+}
+// channel-major: tile[c * CS + tok0 + t]
+__device__ __forceinline__ void write_cm8(unsigned char *tile, int c, int tok0, const Packed8 &v) {
+    uint2 *cm = reinterpret_cast<uint2 *>(tile + (c * CS + tok0) * 2);
+    cm[0] = make_uint2(v.p[0], v.p[1]);
+    cm[1] = make_uint2(v.p[2], v.p[3]);
+}
+
+// Prefix and suffix scalings of one half block (h = 0: tokens 0..7, h = 1: tokens 8..15):
+//   pre[t] = prod_{r<=t} gate_r from the block start, hat = v * prod_{r>t} gate_r, til = hat / total.
+template <typename OPE, int NV>
+__device__ __forceinline__ float scale_half(const RawF<NV> &f, int h, float (&pre)[8], float (&hat)[8], float (&til)[8],
+                                            u32 &bad) {
+    float run = h ? f.goth_prod : 1.0f;
+#pragma unroll
+    for (int t = 0; t < 8; ++t) {
+        run *= f.gown[t];
+        pre[t] = run;
+    }
+    const float tot = h ? run : run * f.goth_prod;
+    bad |= f.bad | ((tot >= OPE::MIN_PRODUCT) ? 0u : 1u);
+    const float itot = __builtin_amdgcn_rcpf(tot);
+    float sfx = h ? 1.0f : f.goth_prod;
+#pragma unroll
+    for (int t = 7; t >= 0; --t) {
+        hat[t] = f.val[0][t] * sfx;      // scaled to the block end   (<= |v|)
+        til[t] = hat[t] * itot;          // scaled to the block start (v / prefix)
+        sfx *= f.gown[t];
+    }
+    return tot;
+}
+
+// One side of the prep work for the whole sequence: KEY = true builds qs, kt (token-major), kh
+// (channel-major) and b_L from f_key, k, q; KEY = false builds xt, xh, a_t and a_L from f, x.
+template <typename IOE, typename OPE, bool KEY>
+__device__ __forceinline__ void fwd_prep_side(const ChunkFwdArgs &p, unsigned char *smem, int tid, int64_t b, int hh,
+                                              int h) {
+    constexpr int NV = KEY ? 2 : 1;
+    const int c = tid & 63;
+    const int T = (int)p.T;                                // the launcher admits T < 2^24 only
+    const int64_t row_off = b * p.T * CH_N;
+    const u16 *const gate = reinterpret_cast<const u16 *>(KEY ? p.f_key : p.f) + row_off;
+    const u16 *const val0 = reinterpret_cast<const u16 *>(KEY ? p.k : p.x) + row_off;
+    const u16 *const val1 = reinterpret_cast<const u16 *>(p.q) + row_off;      // key side only
+    const int nsteps = (T + CH_STEP - 1) / CH_STEP;
+    const int off_own = CH_L * hh + 8 * h, off_oth = CH_L * hh + 8 * (1 - h);   // inside a step
+    const u32 lane_bytes = 2u * (u32)c;
+    u32 bad = 0;
+
+    auto issue = [&](RawSet<NV> &r, int step, u32 lb) {
+        const int st = min(step, nsteps - 1);      // past the end: the last step again (never used)
+        raw_issue<NV>(r, gate, val0, val1, st * CH_STEP + off_own, st * CH_STEP + off_oth, T, lb);
+    };
+    // builds this wave's share of the tiles of step n, which r holds; r then takes step n + 2
+    auto prepare = [&](RawSet<NV> &r, int n) {
+        const RawF<NV> f = raw_take<IOE, NV>(r, n * CH_STEP + off_own, n * CH_STEP + off_oth, T);
+        // The loads that refill r must come after the conversions above, or they need registers
+        // (and a wait) of their own: tie their address to the converted values.
+        u32 lb = lane_bytes;
+        if constexpr (KEY) {
+            asm volatile("" : "+v"(lb)
+                         : "v"(f.gown[0]), "v"(f.gown[1]), "v"(f.gown[2]), "v"(f.gown[3]), "v"(f.gown[4]), "v"(f.gown[5]),
+                           "v"(f.gown[6]), "v"(f.gown[7]), "v"(f.val[0][0]), "v"(f.val[0][1]), "v"(f.val[0][2]),
+                           "v"(f.val[0][3]), "v"(f.val[0][4]), "v"(f.val[0][5]), "v"(f.val[0][6]), "v"(f.val[0][7]),
+                           "v"(f.val[NV - 1][0]), "v"(f.val[NV - 1][1]), "v"(f.val[NV - 1][2]), "v"(f.val[NV - 1][3]),
+                           "v"(f.val[NV - 1][4]), "v"(f.val[NV - 1][5]), "v"(f.val[NV - 1][6]), "v"(f.val[NV - 1][7]),
+                           "v"(f.goth_prod), "v"(f.bad));
+        } else {
+            asm volatile("" : "+v"(lb)
+                         : "v"(f.gown[0]), "v"(f.gown[1]), "v"(f.gown[2]), "v"(f.gown[3]), "v"(f.gown[4]), "v"(f.gown[5]),
+                           "v"(f.gown[6]), "v"(f.gown[7]), "v"(f.val[0][0]), "v"(f.val[0][1]), "v"(f.val[0][2]),
+                           "v"(f.val[0][3]), "v"(f.val[0][4]), "v"(f.val[0][5]), "v"(f.val[0][6]), "v"(f.val[0][7]),
+                           "v"(f.goth_prod), "v"(f.bad));
+        }
+        issue(r, n + 2, lb);
+        unsigned char *ops = smem + (n & 1) * OPS_BYTES;
+        float pre[8], hat[8], til[8];
+        const float tot = scale_half<OPE, NV>(f, h, pre, hat, til, bad);
+        const int tok0 = CH_L * hh + 8 * h;
+        if constexpr (KEY) {
+            float qs[8];
+#pragma unroll
+            for (int t = 0; t < 8; ++t) qs[t] = f.val[1][t] * pre[t];
+            write_tm8(ops + OFF_QT, c, tok0, pack8<OPE>(qs));
+            write_tm8(ops + OFF_KT, c, tok0, pack8<OPE>(til));
+            write_cm8(ops + OFF_KH, c, tok0, pack8<OPE>(hat));
+            if (h == 0) reinterpret_cast<float *>(ops + OFF_BL)[hh * CH_N + c] = tot;
+        } else {
+            write_cm8(ops + OFF_XT, c, tok0, pack8<OPE>(til));
+            write_cm8(ops + OFF_XH, c, tok0, pack8<OPE>(hat));
+            float4 *AS = reinterpret_cast<float4 *>(ops + OFF_AS + (c * CS + tok0) * 4);
+            AS[0] = make_float4(pre[0], pre[1], pre[2], pre[3]);
+            AS[1] = make_float4(pre[4], pre[5], pre[6], pre[7]);
+            if (h == 0) reinterpret_cast<float *>(ops + OFF_AL)[hh * CH_N + c] = tot;
+        }
+    };
+
+    // Steps alternate between two register sets.  The loop always does a whole pair (set A, then
+    // set B) with no exit in between, so that the order of the loads in flight is the same on
+    // every path into it; an odd step count peels the first step off.
+    RawSet<NV> setA, setB;
+    int n = 0;
+    PHASE_BEGIN();
+    if (nsteps & 1) {
+        issue(setB, 0, lane_bytes);
+        issue(setA, 1, lane_bytes);
+        prepare(setB, 0);
+        PHASE_MARK(0);
+        __syncthreads();
+        PHASE_MARK(3);
+        n = 1;
+    } else {
+        issue(setA, 0, lane_bytes);
+        issue(setB, 1, lane_bytes);
+    }
+    for (; n < nsteps; n += 2) {
+        prepare(setA, n);
+        PHASE_MARK(0);
+        __syncthreads();
+        PHASE_MARK(3);
+        prepare(setB, n + 1);
+        PHASE_MARK(0);
+        __syncthreads();
+        PHASE_MARK(3);
+    }
+    if (bad) p.row_flags[b] = 1;
+    PHASE_END(4 + (tid >> 6));
+}
+
+template <typename E> __device__ __forceinline__ uint2 pack4(const floatx4 &v) {
     return make_uint2(E::pack2(v[0], v[1]), E::pack2(v[2], v[3]));
 }
 
@@ -156,78 +288,14 @@ __device__ __forceinline__ void store_state(const floatx4 (&S)[4], u16 *dst, int
         *reinterpret_cast<uint2 *>(dst + d * CH_N + 16 * j + 4 * g) = pack4<IOE>(S[j]);
 }
 
-// Workgroup = 8 waves.  Waves 0-3 ("matrix waves") own the state slabs and run the MFMA
-// phase of step n; waves 4-7 ("prep waves") build the operand tiles of step n+1, prefetch
-// raw inputs and write the previous step's outputs.  One barrier per step hands the
-// double-buffered tiles over.
-constexpr int FWD_THREADS = 512;
-
-template <typename IOE, typename OPE>
-__device__ __forceinline__ void fwd_prep_waves(const ChunkFwdArgs &p, unsigned char *smem, int tid, int64_t b) {
-    const int h = tid >> 7, c = tid & 63;      // block of the step, channel
-    const bool kside = ((tid >> 6) & 1) == 0;
-    const int64_t T = p.T;
-    const int64_t row_base = b * T;
-    const u16 *const src[5] = {reinterpret_cast<const u16 *>(p.f_key), reinterpret_cast<const u16 *>(p.k),
-                               reinterpret_cast<const u16 *>(p.q), reinterpret_cast<const u16 *>(p.f),
-                               reinterpret_cast<const u16 *>(p.x)};
-    u16 *out = reinterpret_cast<u16 *>(p.out);
-    const int64_t nsteps = (T + CH_STEP - 1) / CH_STEP;
-    u32 bad = 0;
-    if (tid == 0) p.row_flags[b] = 0;
-
-    // step m of the raw inputs lives in RAW[m & 1]; `st` carries the next step to be written
-    Stage st;
-    stage_load<IOE>(st, src, row_base, T, 0, tid);
-    stage_store(st, smem + OFF_RAW, tid);
-    if (nsteps > 1) {
-        stage_load<IOE>(st, src, row_base, T, 1, tid);
-        stage_store(st, smem + OFF_RAW + RAW_BYTES, tid);
-    }
-    if (nsteps > 2) stage_load<IOE>(st, src, row_base, T, 2, tid);
-    __syncthreads();
-    {
-        Raw r;
-        raw_read(r, smem + OFF_RAW, kside, h, c);
-        prep_block<IOE, OPE>(r, kside, h, c, smem, bad);
-    }
-    __syncthreads();
-
-    auto store_out = [&](int64_t step) {      // outputs of `step`: LDS tile -> global, 16 B per thread
-        const u16 *OUTP = reinterpret_cast<const u16 *>(smem + OFF_OUT + (step & 1) * OUT_BYTES);
-        const int tok = tid >> 3, piece = tid & 7;
-        const int64_t t = step * CH_STEP + tok;
-        if (t < T) {
-            const uint2 lo = *reinterpret_cast<const uint2 *>(OUTP + tok * OS + 8 * piece);
-            const uint2 hi = *reinterpret_cast<const uint2 *>(OUTP + tok * OS + 8 * piece + 4);
-            *reinterpret_cast<uint4 *>(out + (row_base + t) * CH_N + 8 * piece) = make_uint4(lo.x, lo.y, hi.x, hi.y);
-        }
-    };
-    PHASE_BEGIN();
-    for (int64_t n = 0; n < nsteps; ++n) {
-        Raw r;
-        if (n + 1 < nsteps) raw_read(r, smem + OFF_RAW + ((n + 1) & 1) * RAW_BYTES, kside, h, c);
-        if (n > 0) store_out(n - 1);
-        PHASE_MARK(2);
-        if (n + 2 < nsteps) stage_store(st, smem + OFF_RAW + (n & 1) * RAW_BYTES, tid);   // step n+2
-        if (n + 3 < nsteps) stage_load<IOE>(st, src, row_base, T, n + 3, tid);
-        PHASE_MARK(1);
-        if (n + 1 < nsteps) prep_block<IOE, OPE>(r, kside, h, c, smem + ((n + 1) & 1) * OPS_BYTES, bad);
-        PHASE_MARK(0);
-        __syncthreads();
-        PHASE_MARK(3);
-    }
-    store_out(nsteps - 1);
-    if (bad) p.row_flags[b] = 1;
-    PHASE_END(4 + (tid >> 6));
-}
-
 template <typename IOE, typename OPE>
 __device__ __forceinline__ void fwd_matrix_waves(const ChunkFwdArgs &p, unsigned char *smem, int tid, int64_t b) {
     const int w = tid >> 6, l = tid & 63, r = l & 15, g = l >> 4;
-    const int d = 16 * w + r;                  // this lane's state column
-    const int64_t T = p.T;
+    const int d = 16 * w + r;                  // this lane's state row (value channel)
+    const int T = (int)p.T;
     u16 *ckpt = reinterpret_cast<u16 *>(p.ckpt);
+    u16 *const out = reinterpret_cast<u16 *>(p.out) + b * p.T * CH_N;
+    // S[j][i]: value channel d, key channel 16j + 4g + i
     floatx4 S[4];
     {
         const u16 *s0 = reinterpret_cast<const u16 *>(p.s0) + b * (CH_N * CH_N);
@@ -240,15 +308,15 @@ __device__ __forceinline__ void fwd_matrix_waves(const ChunkFwdArgs &p, unsigned
             S[j][3] = IOE::to_f32((u16)(v.y >> 16));
         }
     }
-    const int64_t nsteps = (T + CH_STEP - 1) / CH_STEP;
+    const int nsteps = (T + CH_STEP - 1) / CH_STEP;
     int until_ckpt = 0;
     int64_t chunk = 0;
-    __syncthreads();      // raw inputs of the first steps are in LDS
-    __syncthreads();      // operand tiles of step 0 are in LDS
+    if (tid == 0) p.row_flags[b] = 0;
     PHASE_BEGIN();
-    for (int64_t n = 0; n < nsteps; ++n) {
+    for (int n = 0; n < nsteps; ++n) {
+        __syncthreads();        // the operand tiles of step n are in LDS
+        PHASE_MARK(3);
         const unsigned char *ops = smem + (n & 1) * OPS_BYTES;
-        u16 *OUT = reinterpret_cast<u16 *>(smem + OFF_OUT + (n & 1) * OUT_BYTES);
         const u16 *QT = reinterpret_cast<const u16 *>(ops + OFF_QT);
         const u16 *KT = reinterpret_cast<const u16 *>(ops + OFF_KT);
         const u16 *KH = reinterpret_cast<const u16 *>(ops + OFF_KH);
@@ -278,22 +346,26 @@ __device__ __forceinline__ void fwd_matrix_waves(const ChunkFwdArgs &p, unsigned
             for (int i = 0; i < 4; ++i) pt[i] = (4 * g + i <= r) ? pt[i] : 0.f;
             const uint2 pa = pack4<OPE>(pt);
             // o[t,d] = a_t[d] * ( sum_k qs_t[k] S0[d,k] + sum_{s<=t} P[t,s] xt_s[d] )
-            const u16 *qperm = QT + (tok0 + r) * TS + 4 * g;
-            const uint2 q0 = *reinterpret_cast<const uint2 *>(qperm);
-            const uint2 q1 = *reinterpret_cast<const uint2 *>(qperm + 16);
-            const uint2 q2 = *reinterpret_cast<const uint2 *>(qperm + 32);
-            const uint2 q3 = *reinterpret_cast<const uint2 *>(qperm + 48);
+            const u16 *qperm = QT + (tok0 + r) * TS + 16 * g;     // channels 16j + 4g + e, j = 0..3, contiguous
             const uint2 s0p = pack4<OPE>(S[0]), s1p = pack4<OPE>(S[1]), s2p = pack4<OPE>(S[2]), s3p = pack4<OPE>(S[3]);
             floatx4 o = {0.f, 0.f, 0.f, 0.f};
-            o = OPE::mfma32(make_uint4(q0.x, q0.y, q1.x, q1.y), make_uint4(s0p.x, s0p.y, s1p.x, s1p.y), o);
-            o = OPE::mfma32(make_uint4(q2.x, q2.y, q3.x, q3.y), make_uint4(s2p.x, s2p.y, s3p.x, s3p.y), o);
+            o = OPE::mfma32(*reinterpret_cast<const uint4 *>(qperm), make_uint4(s0p.x, s0p.y, s1p.x, s1p.y), o);
+            o = OPE::mfma32(*reinterpret_cast<const uint4 *>(qperm + 8), make_uint4(s2p.x, s2p.y, s3p.x, s3p.y), o);
             const floatx4 zero = {0.f, 0.f, 0.f, 0.f};
             const floatx4 oi = OPE::mfma16(pa, *reinterpret_cast<const uint2 *>(XT + d * CS + tok0 + 4 * g), zero);
             const float4 as = *reinterpret_cast<const float4 *>(AS + d * CS + tok0 + 4 * g);
-            OUT[(tok0 + 4 * g + 0) * OS + d] = cvt1<IOE>((o[0] + oi[0]) * as.x);
-            OUT[(tok0 + 4 * g + 1) * OS + d] = cvt1<IOE>((o[1] + oi[1]) * as.y);
-            OUT[(tok0 + 4 * g + 2) * OS + d] = cvt1<IOE>((o[2] + oi[2]) * as.z);
-            OUT[(tok0 + 4 * g + 3) * OS + d] = cvt1<IOE>((o[3] + oi[3]) * as.w);
+            const float asv[4] = {as.x, as.y, as.z, as.w};
+            // 16 lanes write 32 contiguous bytes of a token row; the four waves complete the row
+            const int tg = n * CH_STEP + tok0 + 4 * g;
+            const u32 go = (u32)tg * CH_N + (u32)d;
+            if ((n + 1) * CH_STEP <= T) {
+#pragma unroll
+                for (int i = 0; i < 4; ++i) out[go + i * CH_N] = cvt1<IOE>((o[i] + oi[i]) * asv[i]);
+            } else {
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                    if (tg + i < T) out[go + i * CH_N] = cvt1<IOE>((o[i] + oi[i]) * asv[i]);
+            }
             // S_L = (a_L (x) b_L) * S0 + sum_s xh_s (x) kh_s
             const float aL = AL[hh * CH_N + d];
             const uint2 xh = *reinterpret_cast<const uint2 *>(XH + d * CS + tok0 + 4 * g);
@@ -308,8 +380,6 @@ __device__ __forceinline__ void fwd_matrix_waves(const ChunkFwdArgs &p, unsigned
             }
             PHASE_MARK(hh);
         }
-        __syncthreads();
-        PHASE_MARK(3);
     }
     store_state<IOE>(S, reinterpret_cast<u16 *>(p.next_state) + b * (CH_N * CH_N), d, g);
     PHASE_END(tid >> 6);
@@ -320,11 +390,18 @@ __global__ __launch_bounds__(FWD_THREADS) void lfw_fwd_chunk_kernel(ChunkFwdArgs
     extern __shared__ __align__(16) unsigned char smem[];
     const int tid = threadIdx.x;
     const int64_t b = blockIdx.x;
-    // both branches execute exactly 2 + nsteps workgroup barriers
-    if (tid < 256)
+    // every wave executes exactly (number of steps) workgroup barriers
+    if (tid < 256) {
         fwd_matrix_waves<IOE, OPE>(p, smem, tid, b);
-    else
-        fwd_prep_waves<IOE, OPE>(p, smem, tid - 256, b);
+    } else {
+        // prep wave pw: (side, block of the step, token half); each SIMD gets one wave of each side
+        const int pw = __builtin_amdgcn_readfirstlane((tid - 256) >> 6);
+        const int hh = (pw >> 1) & 1, h = pw >> 2;
+        if (((pw ^ h) & 1) == 0)
+            fwd_prep_side<IOE, OPE, true>(p, smem, tid - 256, b, hh, h);
+        else
+            fwd_prep_side<IOE, OPE, false>(p, smem, tid - 256, b, hh, h);
+    }
 }
 
 template <typename IOE, typename OPE> int launch(const ChunkFwdArgs &a, hipStream_t stream) {
@@ -335,6 +412,7 @@ template <typename IOE, typename OPE> int launch(const ChunkFwdArgs &a, hipStrea
                        "hipFuncSetAttribute(forward chunk kernel)");
     if (rc) return rc;
     if (a.B > 0x7fffffffLL) return fail(T2FW_ERR_UNSUPPORTED, "B=%lld is too large", (long long)a.B);
+    if (a.T >= CHUNK_MAX_T) return fail(T2FW_ERR_UNSUPPORTED, "T=%lld is too long for 32-bit row offsets", (long long)a.T);
     hipLaunchKernelGGL(kern, dim3((unsigned)a.B), dim3(FWD_THREADS), FWD_SMEM, stream, a);
     return check_hip(hipGetLastError(), "lfw_fwd_chunk_kernel launch");
 }
