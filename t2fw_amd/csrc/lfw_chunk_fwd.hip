@@ -49,38 +49,44 @@ template <int NV> struct RawSet {
     u16 gown[8], goth[8], val[NV][8];
 };
 
-// gate, val0, val1 (NV = 2 only): wave-uniform addresses of token 0 of the batch row; tok_own / tok_oth: first of the
-// eight own / other tokens; lane_bytes = 2 * channel.  Tokens past the end of the sequence are
-// read from the last one (and replaced when the set is taken), with the same number of loads as
-// the fast path, so that the count of loads in flight does not depend on the path.
+// gate, val0, val1 (NV = 2 only): wave-uniform addresses of token 0 of the batch row; tok_own / tok_oth:
+// first of the eight own / other tokens; lane_bytes = 2 * channel.  All sixteen tokens must exist.
 template <int NV>
 __device__ __forceinline__ void raw_issue(RawSet<NV> &r, const u16 *gate, const u16 *val0, const u16 *val1, int tok_own,
-                                          int tok_oth, int T, u32 lane_bytes) {
+                                          int tok_oth, u32 lane_bytes) {
     const u16 *const val[2] = {val0, val1};
     auto at = [&](const u16 *base, int tok) -> const u16 * {
         return reinterpret_cast<const u16 *>(reinterpret_cast<const unsigned char *>(base + (u32)tok * CH_N) + lane_bytes);
     };
-    if (max(tok_own, tok_oth) + 8 <= T) {
-        const u16 *go = at(gate, tok_own), *gx = at(gate, tok_oth);
+    const u16 *go = at(gate, tok_own), *gx = at(gate, tok_oth);
 #pragma unroll
-        for (int t = 0; t < 8; ++t) r.goth[t] = gx[t * CH_N];
+    for (int t = 0; t < 8; ++t) r.goth[t] = gx[t * CH_N];
 #pragma unroll
-        for (int t = 0; t < 8; ++t) r.gown[t] = go[t * CH_N];
+    for (int t = 0; t < 8; ++t) r.gown[t] = go[t * CH_N];
 #pragma unroll
-        for (int a = 0; a < NV; ++a) {
-            const u16 *va = at(val[a], tok_own);
+    for (int a = 0; a < NV; ++a) {
+        const u16 *va = at(val[a], tok_own);
 #pragma unroll
-            for (int t = 0; t < 8; ++t) r.val[a][t] = va[t * CH_N];
-        }
-    } else {
+        for (int t = 0; t < 8; ++t) r.val[a][t] = va[t * CH_N];
+    }
+}
+
+// The same for the last, partial step of a sequence: tokens past the end are read from the last
+// one (and replaced by raw_take_tail).
+template <int NV>
+__device__ __forceinline__ void raw_issue_tail(RawSet<NV> &r, const u16 *gate, const u16 *val0, const u16 *val1,
+                                               int tok_own, int tok_oth, int T, u32 lane_bytes) {
+    const u16 *const val[2] = {val0, val1};
+    auto at = [&](const u16 *base, int tok) -> const u16 * {
+        return reinterpret_cast<const u16 *>(reinterpret_cast<const unsigned char *>(base + (u32)min(tok, T - 1) * CH_N) +
+                                             lane_bytes);
+    };
 #pragma unroll
-        for (int t = 0; t < 8; ++t) r.goth[t] = *at(gate, min(tok_oth + t, T - 1));
+    for (int t = 0; t < 8; ++t) {
+        r.goth[t] = *at(gate, tok_oth + t);
+        r.gown[t] = *at(gate, tok_own + t);
 #pragma unroll
-        for (int t = 0; t < 8; ++t) r.gown[t] = *at(gate, min(tok_own + t, T - 1));
-#pragma unroll
-        for (int a = 0; a < NV; ++a)
-#pragma unroll
-            for (int t = 0; t < 8; ++t) r.val[a][t] = *at(val[a], min(tok_own + t, T - 1));
+        for (int a = 0; a < NV; ++a) r.val[a][t] = *at(val[a], tok_own + t);
     }
 }
 
@@ -89,9 +95,8 @@ template <int NV> struct RawF {
     u32 bad;      // own gates outside (0, 1]
 };
 
-// Registers -> floats; tokens past the end act as identity (gate 1, everything else 0).
-template <typename IOE, int NV>
-__device__ __forceinline__ RawF<NV> raw_take(const RawSet<NV> &r, int tok_own, int tok_oth, int T) {
+// Registers -> floats.
+template <typename IOE, int NV> __device__ __forceinline__ RawF<NV> raw_take(const RawSet<NV> &r) {
     RawF<NV> f;
     // the loads complete in order: one wait for the last of them covers the whole set
     asm volatile("" ::"v"(r.val[NV - 1][7]));
@@ -108,24 +113,27 @@ __device__ __forceinline__ RawF<NV> raw_take(const RawSet<NV> &r, int tok_own, i
     }
     f.bad = (mx >= IOE::ONE_BITS) ? 1u : 0u;
     f.goth_prod = po;
-    if (max(tok_own, tok_oth) + 8 > T) {          // wave-uniform, last step of the sequence only
-        po = 1.0f;
-        mx = 0;
+    return f;
+}
+
+// Partial step: tokens past the end act as identity (gate 1, everything else 0).
+template <typename IOE, int NV>
+__device__ __forceinline__ RawF<NV> raw_take_tail(const RawSet<NV> &r, int tok_own, int tok_oth, int T) {
+    RawF<NV> f;
+    u16 mx = 0;
+    float po = 1.0f;
 #pragma unroll
-        for (int t = 0; t < 8; ++t) {
-            if (tok_oth + t < T) po *= IOE::to_f32(r.goth[t]);
-            if (tok_own + t < T) {
-                const u16 m1 = (u16)(r.gown[t] - 1);
-                mx = m1 > mx ? m1 : mx;
-            } else {
-                f.gown[t] = 1.0f;
+    for (int t = 0; t < 8; ++t) {
+        if (tok_oth + t < T) po *= IOE::to_f32(r.goth[t]);
+        const bool own = tok_own + t < T;
+        const u16 m1 = own ? (u16)(r.gown[t] - 1) : (u16)0;
+        mx = m1 > mx ? m1 : mx;
+        f.gown[t] = own ? IOE::to_f32(r.gown[t]) : 1.0f;
 #pragma unroll
-                for (int a = 0; a < NV; ++a) f.val[a][t] = 0.0f;
-            }
-        }
-        f.bad = (mx >= IOE::ONE_BITS) ? 1u : 0u;
-        f.goth_prod = po;
+        for (int a = 0; a < NV; ++a) f.val[a][t] = own ? IOE::to_f32(r.val[a][t]) : 0.0f;
     }
+    f.bad = (mx >= IOE::ONE_BITS) ? 1u : 0u;
+    f.goth_prod = po;
     return f;
 }
 
@@ -191,37 +199,13 @@ __device__ __forceinline__ void fwd_prep_side(const ChunkFwdArgs &p, unsigned ch
     const u16 *const gate = reinterpret_cast<const u16 *>(KEY ? p.f_key : p.f) + row_off;
     const u16 *const val0 = reinterpret_cast<const u16 *>(KEY ? p.k : p.x) + row_off;
     const u16 *const val1 = reinterpret_cast<const u16 *>(p.q) + row_off;      // key side only
-    const int nsteps = (T + CH_STEP - 1) / CH_STEP;
+    const int nfull = T / CH_STEP;                         // full 32-token steps; a partial one may follow
     const int off_own = CH_L * hh + 8 * h, off_oth = CH_L * hh + 8 * (1 - h);   // inside a step
     const u32 lane_bytes = 2u * (u32)c;
     u32 bad = 0;
 
-    auto issue = [&](RawSet<NV> &r, int step, u32 lb) {
-        const int st = min(step, nsteps - 1);      // past the end: the last step again (never used)
-        raw_issue<NV>(r, gate, val0, val1, st * CH_STEP + off_own, st * CH_STEP + off_oth, T, lb);
-    };
-    // builds this wave's share of the tiles of step n, which r holds; r then takes step n + 2
-    auto prepare = [&](RawSet<NV> &r, int n) {
-        const RawF<NV> f = raw_take<IOE, NV>(r, n * CH_STEP + off_own, n * CH_STEP + off_oth, T);
-        // The loads that refill r must come after the conversions above, or they need registers
-        // (and a wait) of their own: tie their address to the converted values.
-        u32 lb = lane_bytes;
-        if constexpr (KEY) {
-            asm volatile("" : "+v"(lb)
-                         : "v"(f.gown[0]), "v"(f.gown[1]), "v"(f.gown[2]), "v"(f.gown[3]), "v"(f.gown[4]), "v"(f.gown[5]),
-                           "v"(f.gown[6]), "v"(f.gown[7]), "v"(f.val[0][0]), "v"(f.val[0][1]), "v"(f.val[0][2]),
-                           "v"(f.val[0][3]), "v"(f.val[0][4]), "v"(f.val[0][5]), "v"(f.val[0][6]), "v"(f.val[0][7]),
-                           "v"(f.val[NV - 1][0]), "v"(f.val[NV - 1][1]), "v"(f.val[NV - 1][2]), "v"(f.val[NV - 1][3]),
-                           "v"(f.val[NV - 1][4]), "v"(f.val[NV - 1][5]), "v"(f.val[NV - 1][6]), "v"(f.val[NV - 1][7]),
-                           "v"(f.goth_prod), "v"(f.bad));
-        } else {
-            asm volatile("" : "+v"(lb)
-                         : "v"(f.gown[0]), "v"(f.gown[1]), "v"(f.gown[2]), "v"(f.gown[3]), "v"(f.gown[4]), "v"(f.gown[5]),
-                           "v"(f.gown[6]), "v"(f.gown[7]), "v"(f.val[0][0]), "v"(f.val[0][1]), "v"(f.val[0][2]),
-                           "v"(f.val[0][3]), "v"(f.val[0][4]), "v"(f.val[0][5]), "v"(f.val[0][6]), "v"(f.val[0][7]),
-                           "v"(f.goth_prod), "v"(f.bad));
-        }
-        issue(r, n + 2, lb);
+    // this wave's share of the operand tiles of step n
+    auto build = [&](const RawF<NV> &f, int n) {
         unsigned char *ops = smem + (n & 1) * OPS_BYTES;
         float pre[8], hat[8], til[8];
         const float tot = scale_half<OPE, NV>(f, h, pre, hat, til, bad);
@@ -243,34 +227,71 @@ __device__ __forceinline__ void fwd_prep_side(const ChunkFwdArgs &p, unsigned ch
             if (h == 0) reinterpret_cast<float *>(ops + OFF_AL)[hh * CH_N + c] = tot;
         }
     };
+    auto issue = [&](RawSet<NV> &r, int step, u32 lb) {
+        const int st = min(step, nfull - 1);       // past the last full step: that step again (never used)
+        raw_issue<NV>(r, gate, val0, val1, st * CH_STEP + off_own, st * CH_STEP + off_oth, lb);
+    };
+    // builds the tiles of full step n, which r holds; r then takes step n + 2
+    auto prepare = [&](RawSet<NV> &r, int n) {
+        const RawF<NV> f = raw_take<IOE, NV>(r);
+        // The loads that refill r must come after the conversions above, or they need registers
+        // (and a wait) of their own: tie their address to the converted values.
+        u32 lb = lane_bytes;
+        if constexpr (KEY) {
+            asm volatile("" : "+v"(lb)
+                         : "v"(f.gown[0]), "v"(f.gown[1]), "v"(f.gown[2]), "v"(f.gown[3]), "v"(f.gown[4]), "v"(f.gown[5]),
+                           "v"(f.gown[6]), "v"(f.gown[7]), "v"(f.val[0][0]), "v"(f.val[0][1]), "v"(f.val[0][2]),
+                           "v"(f.val[0][3]), "v"(f.val[0][4]), "v"(f.val[0][5]), "v"(f.val[0][6]), "v"(f.val[0][7]),
+                           "v"(f.val[NV - 1][0]), "v"(f.val[NV - 1][1]), "v"(f.val[NV - 1][2]), "v"(f.val[NV - 1][3]),
+                           "v"(f.val[NV - 1][4]), "v"(f.val[NV - 1][5]), "v"(f.val[NV - 1][6]), "v"(f.val[NV - 1][7]),
+                           "v"(f.goth_prod), "v"(f.bad));
+        } else {
+            asm volatile("" : "+v"(lb)
+                         : "v"(f.gown[0]), "v"(f.gown[1]), "v"(f.gown[2]), "v"(f.gown[3]), "v"(f.gown[4]), "v"(f.gown[5]),
+                           "v"(f.gown[6]), "v"(f.gown[7]), "v"(f.val[0][0]), "v"(f.val[0][1]), "v"(f.val[0][2]),
+                           "v"(f.val[0][3]), "v"(f.val[0][4]), "v"(f.val[0][5]), "v"(f.val[0][6]), "v"(f.val[0][7]),
+                           "v"(f.goth_prod), "v"(f.bad));
+        }
+        issue(r, n + 2, lb);
+        build(f, n);
+    };
 
-    // Steps alternate between two register sets.  The loop always does a whole pair (set A, then
-    // set B) with no exit in between, so that the order of the loads in flight is the same on
-    // every path into it; an odd step count peels the first step off.
-    RawSet<NV> setA, setB;
-    int n = 0;
+    // Full steps alternate between two register sets.  The loop always does a whole pair (set A,
+    // then set B) with no exit in between, so that the order of the loads in flight is the same on
+    // every path into it; an odd count peels the first step off.
     PHASE_BEGIN();
-    if (nsteps & 1) {
-        issue(setB, 0, lane_bytes);
-        issue(setA, 1, lane_bytes);
-        prepare(setB, 0);
-        PHASE_MARK(0);
-        __syncthreads();
-        PHASE_MARK(3);
-        n = 1;
-    } else {
-        issue(setA, 0, lane_bytes);
-        issue(setB, 1, lane_bytes);
+    if (nfull > 0) {
+        RawSet<NV> setA, setB;
+        int n = 0;
+        if (nfull & 1) {
+            issue(setB, 0, lane_bytes);
+            issue(setA, 1, lane_bytes);
+            prepare(setB, 0);
+            PHASE_MARK(0);
+            __syncthreads();
+            PHASE_MARK(3);
+            n = 1;
+        } else {
+            issue(setA, 0, lane_bytes);
+            issue(setB, 1, lane_bytes);
+        }
+        for (; n < nfull; n += 2) {
+            prepare(setA, n);
+            PHASE_MARK(0);
+            __syncthreads();
+            PHASE_MARK(3);
+            prepare(setB, n + 1);
+            PHASE_MARK(0);
+            __syncthreads();
+            PHASE_MARK(3);
+        }
     }
-    for (; n < nsteps; n += 2) {
-        prepare(setA, n);
-        PHASE_MARK(0);
+    if (nfull * CH_STEP < T) {      // the partial step at the end
+        RawSet<NV> r;
+        const int t_own = nfull * CH_STEP + off_own, t_oth = nfull * CH_STEP + off_oth;
+        raw_issue_tail<NV>(r, gate, val0, val1, t_own, t_oth, T, lane_bytes);
+        build(raw_take_tail<IOE, NV>(r, t_own, t_oth, T), nfull);
         __syncthreads();
-        PHASE_MARK(3);
-        prepare(setB, n + 1);
-        PHASE_MARK(0);
-        __syncthreads();
-        PHASE_MARK(3);
     }
     if (bad) p.row_flags[b] = 1;
     PHASE_END(4 + (tid >> 6));
