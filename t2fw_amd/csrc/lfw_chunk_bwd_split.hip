@@ -325,7 +325,7 @@ __device__ __forceinline__ void split_prep_waves(const ChunkBwdArgs &p, unsigned
     // builds the tiles of stage s, which r holds and it stands on; r and it then move on two stages
     auto prepare = [&](RawSet &r, int s, StageIter<NB> &it) {
         const int st = it.cur();
-        const RawF fr = raw_take<IOE>(r, !(st & 1) || (role & 1));
+        const RawF fr = raw_take<IOE>(r, (st & 1) && (role & 1));     // every block's gates are checked in its B stage
         // The loads that refill r must come after the conversions above, or they need registers
         // (and a wait) of their own: tie their address to the converted values.
         u32 lb = lane_bytes;

@@ -134,7 +134,7 @@ __global__ __launch_bounds__(SCAN_THREADS) void lfw_fwd_scan_kernel(ScanFwdArgs 
 template <int KPL> struct SegLen { static constexpr int value = (32 / KPL) < 1 ? 1 : (KPL <= 4 ? 8 : 32 / KPL); };
 
 template <typename IO, int KPL, int SIDE>
-__global__ __launch_bounds__(SCAN_THREADS) void lfw_bwd_scan_kernel(ScanBwdArgs p) {
+__device__ __forceinline__ void bwd_scan_body(const ScanBwdArgs &p) {
     using Acc = typename AccOf<IO>::type;
     constexpr int SEG = SegLen<KPL>::value;
     extern __shared__ __align__(16) unsigned char smem_raw[];
@@ -301,6 +301,22 @@ __global__ __launch_bounds__(SCAN_THREADS) void lfw_bwd_scan_kernel(ScanBwdArgs 
     }
 }
 
+template <typename IO, int KPL, int SIDE>
+__global__ __launch_bounds__(SCAN_THREADS) void lfw_bwd_scan_kernel(ScanBwdArgs p) {
+    bwd_scan_body<IO, KPL, SIDE>(p);
+}
+
+// Both sides in one launch (blockIdx.y = side) for square states, where the two sides share
+// their geometry.  Used when the kernel only redoes the rows another kernel has flagged:
+// then most workgroups exit at once and a launch costs more than it computes.
+template <typename IO, int KPL>
+__global__ __launch_bounds__(SCAN_THREADS) void lfw_bwd_scan_both_kernel(ScanBwdArgs p) {
+    if (blockIdx.y == 0)
+        bwd_scan_body<IO, KPL, 0>(p);
+    else
+        bwd_scan_body<IO, KPL, 1>(p);
+}
+
 // ------------------------------------------------------------------------------------
 // host dispatch
 // ------------------------------------------------------------------------------------
@@ -331,8 +347,13 @@ int launch_bwd(ScanBwdArgs a, const ScanGeom &g, hipStream_t stream) {
     a.ntiles = (int)((nrows + g.rows - 1) / g.rows);
     const int64_t nblocks = a.B * a.ntiles;
     if (nblocks > 0x7fffffffLL) return fail(T2FW_ERR_UNSUPPORTED, "grid of %lld workgroups is too large", (long long)nblocks);
+    if (SIDE == 2) {
+        hipLaunchKernelGGL((lfw_bwd_scan_both_kernel<IO, KPL>), dim3((unsigned)nblocks, 2, 1), dim3(SCAN_THREADS), smem,
+                           stream, a);
+        return check_hip(hipGetLastError(), "lfw_bwd_scan_both_kernel launch");
+    }
     dim3 grid((unsigned)nblocks, 1, 1);
-    hipLaunchKernelGGL((lfw_bwd_scan_kernel<IO, KPL, SIDE>), grid, dim3(SCAN_THREADS), smem, stream, a);
+    hipLaunchKernelGGL((lfw_bwd_scan_kernel<IO, KPL, (SIDE == 2 ? 0 : SIDE)>), grid, dim3(SCAN_THREADS), smem, stream, a);
     return check_hip(hipGetLastError(), "lfw_bwd_scan_kernel launch");
 }
 
@@ -374,6 +395,8 @@ template <typename IO, int SIDE> int bwd_by_kpl(const ScanBwdArgs &a, hipStream_
 }
 
 template <typename IO> int bwd_both(const ScanBwdArgs &a, hipStream_t stream) {
+    // SIDE 2 = both sides in one launch (square states, fix-up mode only)
+    if (a.row_select != nullptr && a.D == a.K) return bwd_by_kpl<IO, 2>(a, stream);
     int rc = bwd_by_kpl<IO, 0>(a, stream);
     if (rc != T2FW_OK) return rc;
     return bwd_by_kpl<IO, 1>(a, stream);
