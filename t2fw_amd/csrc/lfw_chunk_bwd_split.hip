@@ -93,51 +93,69 @@ template <int NB> struct SplitSchedule {
     }
 };
 
-// The same schedule as a forward iterator (no divisions): cur() is SplitSchedule::at of the stage
-// it stands on; advancing past the last stage leaves it there.
+// The same schedule as a forward iterator: cur() is SplitSchedule::at of the stage it stands on;
+// advancing past the last stage leaves it there.  The stages of a chunk are one byte each in a
+// 64-bit table, (block << 1) | (1 for a B stage), so that a step costs a few scalar instructions.
 template <int NB> struct StageIter {
-    int chunk, local, nb, C, left;      // left: stages after the current one
-    __device__ StageIter(const SplitSchedule<NB> &sc) : chunk(sc.NC - 1), local(0), nb(sc.nb_last), C(sc.C), left(sc.total - 1) {}
+    static __host__ __device__ constexpr uint64_t table_of(int nb) {
+        uint64_t t = 0;
+        const int nr = (nb + 1) / 2;
+        for (int l = 0; l < nr + nb; ++l) {
+            const uint64_t e = l < nr ? (uint64_t)(2 * l) << 1 : ((uint64_t)(nb - 1 - (l - nr)) << 1) | 1u;
+            t |= e << (8 * l);
+        }
+        return t;
+    }
+    uint64_t table;     // of the chunk it stands in
+    int base2;          // (first token of that chunk) * 2
+    int local, count;   // stage inside the chunk, stages of the chunk
+    int C2, left;       // 2 * C; stages after the current one
+    __device__ StageIter(const SplitSchedule<NB> &sc)
+        : base2((sc.NC - 1) * sc.C * 2), local(0), count(sc.st_last), C2(2 * sc.C), left(sc.total - 1) {
+        table = sc.nb_last == 1 ? table_of(1) : sc.nb_last == 2 ? table_of(2) : sc.nb_last == 3 ? table_of(3) : table_of(4);
+    }
     __device__ void advance() {
         if (left > 0) {
             --left;
             ++local;
-            if (local == (nb + 1) / 2 + nb) {
-                --chunk;
+            if (local == count) {
+                base2 -= C2;
                 local = 0;
-                nb = NB;
+                count = (int)SplitSchedule<NB>::PER_CHUNK;
+                table = table_of(NB);
             }
         }
     }
     __device__ int cur() const {
-        const int nr = (nb + 1) / 2;
-        const bool bmode = local >= nr;
-        const int block = bmode ? nb - 1 - (local - nr) : 2 * local;
-        return ((chunk * C + block * CH_L) << 1) | (bmode ? 1 : 0);
+        const int e = (int)(table >> (8 * local)) & 0xff;       // (block << 1) | bmode
+        return base2 + (e >> 1) * (2 * CH_L) + (e & 1);
     }
 };
+static_assert(SplitSchedule<4>::PER_CHUNK <= 8, "a chunk's stages must fit the 64-bit table");
 
 // ---- raw inputs --------------------------------------------------------------------------
 // A prep thread works on one channel and eight tokens; it needs the gate at those tokens, the
 // gate at the block's other eight tokens and one value (or adjoint) array at its own tokens:
 // 24 two-byte loads, coalesced over the wave's 64 channels.  They go straight to registers,
-// two stages ahead of their use, from a wave-uniform base with immediate token offsets.
+// two stages ahead of their use: the block's first token of an array is a scalar base, the
+// lane's channel and token half a constant vector offset, the token inside the half an
+// immediate one.
 struct RawSet {
     u16 gown[8], goth[8], val[8];
 };
 
-// gate, val: wave-uniform addresses of the block's first token; lane_bytes = 2 * channel
-__device__ __forceinline__ void raw_issue(RawSet &r, const u16 *gate, const u16 *val, int h, u32 lane_bytes) {
-    auto at = [&](const u16 *base, int tok) -> const u16 * {
-        return reinterpret_cast<const u16 *>(reinterpret_cast<const unsigned char *>(base + tok * CH_N) + lane_bytes);
+// gate, val: wave-uniform addresses of the block's first token; voff_own / voff_oth: byte offsets of
+// (own / other token half, channel) inside a block
+__device__ __forceinline__ void raw_issue(RawSet &r, const u16 *gate, const u16 *val, u32 voff_own, u32 voff_oth) {
+    auto at = [&](const u16 *base, u32 voff, int t) -> u16 {
+        return *reinterpret_cast<const u16 *>(reinterpret_cast<const unsigned char *>(base + t * CH_N) + voff);
     };
-    const u16 *go = at(gate, 8 * h), *gx = at(gate, 8 * (1 - h)), *va = at(val, 8 * h);
 #pragma unroll
-    for (int t = 0; t < 8; ++t) r.goth[t] = gx[t * CH_N];
+    for (int t = 0; t < 8; ++t) r.goth[t] = at(gate, voff_oth, t);
 #pragma unroll
-    for (int t = 0; t < 8; ++t) r.gown[t] = go[t * CH_N];
+    for (int t = 0; t < 8; ++t) r.gown[t] = at(gate, voff_own, t);
 #pragma unroll
-    for (int t = 0; t < 8; ++t) r.val[t] = va[t * CH_N];
+    for (int t = 0; t < 8; ++t) r.val[t] = at(val, voff_own, t);
 }
 
 template <typename IOE> __device__ __forceinline__ u32 gate_check8(const u16 (&g)[8]) {
@@ -182,46 +200,30 @@ __device__ __forceinline__ void write_cf8(unsigned char *stage, int tile, int c,
     cf[1] = make_float4(v[4], v[5], v[6], v[7]);
 }
 
-// Raw inputs as floats: the registers of the RawSet are free again after this.
-struct RawF {
-    float gown[8], goth_prod, val[8];
-    u32 bad;      // own gates outside (0, 1]
-};
-
-template <typename IOE> __device__ __forceinline__ RawF raw_take(const RawSet &r, bool check) {
-    RawF f;
-    // the loads complete in order: one wait for the last of them covers the whole set
-    asm volatile("" ::"v"(r.val[7]));
-    f.bad = check ? gate_check8<IOE>(r.gown) : 0u;
-    float po = 1.0f;
+template <typename IOE> __device__ __forceinline__ float product8(const u16 (&g)[8]) {
+    float p = IOE::mul2(g[0], g[1]);
 #pragma unroll
-    for (int t = 0; t < 8; ++t) {
-        f.gown[t] = IOE::to_f32(r.gown[t]);
-        f.val[t] = IOE::to_f32(r.val[t]);
-        po *= IOE::to_f32(r.goth[t]);
-    }
-    f.goth_prod = po;
-    return f;
+    for (int t = 2; t < 8; ++t) p = IOE::mul(g[t], p);
+    return p;
 }
 
 // Gate-suffix scalings of one half block: hat = v * prod_{r>t} gate_r, til = hat / total,
 // inv = 1 / prod_{r<=t} gate_r; returns the 16-step product.
-template <typename OPE>
-__device__ __forceinline__ float suffix_scale(const RawF &f, int h, float (&hat)[8], float (&til)[8], float (&inv)[8],
-                                              u32 &bad) {
-    float pown = 1.0f;
-#pragma unroll
-    for (int t = 0; t < 8; ++t) pown *= f.gown[t];
-    const float tot = pown * f.goth_prod;
-    bad |= f.bad | ((tot >= OPE::MIN_PRODUCT) ? 0u : 1u);
+template <typename IOE, typename OPE>
+__device__ __forceinline__ float suffix_scale(const RawSet &r, int h, bool check, float (&hat)[8], float (&til)[8],
+                                              float (&inv)[8], u32 &bad) {
+    const float poth = product8<IOE>(r.goth);
+    const float tot = product8<IOE>(r.gown) * poth;
+    if (check) bad |= gate_check8<IOE>(r.gown);
+    bad |= (tot >= OPE::MIN_PRODUCT) ? 0u : 1u;
     const float itot = __builtin_amdgcn_rcpf(tot);
-    float sfx = h ? 1.0f : f.goth_prod;
+    float sfx = h ? 1.0f : poth;
 #pragma unroll
     for (int t = 7; t >= 0; --t) {
         inv[t] = sfx * itot;
-        hat[t] = f.val[t] * sfx;
+        hat[t] = IOE::mul(r.val[t], sfx);
         til[t] = hat[t] * itot;
-        sfx *= f.gown[t];
+        sfx = IOE::mul(r.gown[t], sfx);
     }
     return tot;
 }
@@ -231,35 +233,42 @@ __device__ __forceinline__ float suffix_scale(const RawF &f, int h, float (&hat)
 //   role 1: other gate suffix -> VOH (both layouts), VOT (token-major), L_other
 //   role 2: own gate prefix   -> AS, 1/gate, prefix (side 1)
 //   role 3: own gate suffix   -> VH, VT, 1/prefix, L_own
-template <typename OPE>
-__device__ __forceinline__ void prep_b(const RawF &f, unsigned char *stage, int role, int h, int c, bool want_pp,
+template <typename IOE, typename OPE>
+__device__ __forceinline__ void prep_b(const RawSet &r, unsigned char *stage, int role, int h, int c, bool want_pp,
                                        u32 &bad) {
     const bool other = role < 2;
     const int t0 = 8 * h;
     if ((role & 1) == 0) {
-        float run = h ? f.goth_prod : 1.0f;
+        const float base = h ? product8<IOE>(r.goth) : 1.0f;
+        float run = base;
         float pre[8], v[8];
 #pragma unroll
         for (int t = 0; t < 8; ++t) {
-            run *= f.gown[t];
+            run = IOE::mul(r.gown[t], run);
             pre[t] = run;
-            v[t] = f.val[t] * run;
+            v[t] = IOE::mul(r.val[t], run);
         }
         const Packed8 vp = pack8<OPE>(v);
         if (other) {
             write_tm8(stage, TM_AOS, c, t0, vp);
             write_cm8(stage, CM_AOS, c, t0, vp);
         } else {
+            // 1/gate_t = prefix_{t-1} / prefix_t from one reciprocal and the running products
+            float ipre = __builtin_amdgcn_rcpf(pre[7]);
             float rg[8];
 #pragma unroll
-            for (int t = 0; t < 8; ++t) rg[t] = __builtin_amdgcn_rcpf(f.gown[t]);
+            for (int t = 7; t >= 1; --t) {
+                rg[t] = pre[t - 1] * ipre;
+                ipre = IOE::mul(r.gown[t], ipre);
+            }
+            rg[0] = base * ipre;
             write_cm8(stage, CM_AS, c, t0, vp);
             write_cf8(stage, F_RG, c, t0, rg);
             if (want_pp) write_cf8(stage, F_PP, c, t0, pre);
         }
     } else {
         float hat[8], til[8], inv[8];
-        const float tot = suffix_scale<OPE>(f, h, hat, til, inv, bad);
+        const float tot = suffix_scale<IOE, OPE>(r, h, true, hat, til, inv, bad);
         if (h == 0) lv_vec(stage, 0, other ? 0 : 1)[c] = tot;
         const Packed8 hp = pack8<OPE>(hat), tp = pack8<OPE>(til);
         if (other) {
@@ -275,11 +284,12 @@ __device__ __forceinline__ void prep_b(const RawF &f, unsigned char *stage, int 
 }
 
 // R stage, one prep wave: block j of the pair, own or other side, tokens 8h..8h+7, channel c:
-// the suffix-scaled values (channel-major) and the 16-step gate product.
-template <typename OPE>
-__device__ __forceinline__ void prep_r(const RawF &f, unsigned char *stage, int j, int own, int h, int c, u32 &bad) {
+// the suffix-scaled values (channel-major) and the 16-step gate product.  (Every block's gates
+// are range-checked in its B stage.)
+template <typename IOE, typename OPE>
+__device__ __forceinline__ void prep_r(const RawSet &r, unsigned char *stage, int j, int own, int h, int c, u32 &bad) {
     float hat[8], til[8], inv[8];
-    const float tot = suffix_scale<OPE>(f, h, hat, til, inv, bad);
+    const float tot = suffix_scale<IOE, OPE>(r, h, false, hat, til, inv, bad);
     if (h == 0) lv_vec(stage, j, own)[c] = tot;
     write_cm8(stage, 2 * j + own, c, 8 * h, pack8<OPE>(hat));
 }
@@ -310,75 +320,68 @@ __device__ __forceinline__ void split_prep_waves(const ChunkBwdArgs &p, unsigned
     const int total = sched.total;
     u32 bad = 0;
 
-    const u32 lane_bytes = 2u * (u32)c;
-    auto issue = [&](RawSet &r, int st, u32 lb) {   // raw inputs of stage st (wave-uniform) -> registers
-        const int tok = st >> 1;
-        if (st & 1) {
-            raw_issue(r, b_gate + (u32)tok * CH_N, b_val + (u32)tok * CH_N, h, lb);
-        } else {
-            // the second block of the last pair may lie past the end: read the last block instead
-            // (its tiles are never used)
-            const int t2 = min(tok + rj * CH_L, T - CH_L);
-            raw_issue(r, r_gate + (u32)t2 * CH_N, r_val + (u32)t2 * CH_N, h, lb);
-        }
+    const u32 voff_own = (u32)(8 * h * CH_N + c) * 2u, voff_oth = (u32)(8 * (1 - h) * CH_N + c) * 2u;
+    auto issue = [&](RawSet &r, int st) {          // raw inputs of stage st (wave-uniform) -> registers
+        const bool bmode = st & 1;
+        // R stages: the second block of the last pair may lie past the end; read the last block
+        // instead (its tiles are never used)
+        const u32 tok = (u32)(bmode ? st >> 1 : min((st >> 1) + rj * CH_L, T - CH_L));
+        raw_issue(r, (bmode ? b_gate : r_gate) + tok * CH_N, (bmode ? b_val : r_val) + tok * CH_N, voff_own, voff_oth);
     };
-    // builds the tiles of stage s, which r holds and it stands on; r and it then move on two stages
-    auto prepare = [&](RawSet &r, int s, StageIter<NB> &it) {
-        const int st = it.cur();
-        const RawF fr = raw_take<IOE>(r, (st & 1) && (role & 1));     // every block's gates are checked in its B stage
-        // The loads that refill r must come after the conversions above, or they need registers
-        // (and a wait) of their own: tie their address to the converted values.
-        u32 lb = lane_bytes;
-        asm volatile("" : "+v"(lb)
-                     : "v"(fr.gown[0]), "v"(fr.gown[1]), "v"(fr.gown[2]), "v"(fr.gown[3]), "v"(fr.gown[4]),
-                       "v"(fr.gown[5]), "v"(fr.gown[6]), "v"(fr.gown[7]), "v"(fr.val[0]), "v"(fr.val[1]), "v"(fr.val[2]),
-                       "v"(fr.val[3]), "v"(fr.val[4]), "v"(fr.val[5]), "v"(fr.val[6]), "v"(fr.val[7]), "v"(fr.goth_prod),
-                       "v"(fr.bad));
-        // unconditional (past the end: the last stage again), so that the number of loads in flight
-        // is the same on every path and the waits for them can be exact
-        it.advance();
-        it.advance();
-        issue(r, it.cur(), lb);
+    // Three register sets rotate: the tiles of stage s are built from `cur`, which was loaded two
+    // stages ago, while `refill` (used up in the stage before) takes the raw inputs of stage s + 2.
+    // The loads are unconditional (past the end: the last stage again), so that the number of loads
+    // in flight is the same on every path and the waits for them can be exact.
+    StageIter<NB> it_load(sched);
+    int st_cur = 0, st_next = 0;                   // descriptors of stages s and s + 1
+    auto prepare = [&](const RawSet &cur, RawSet &refill, int s) {
+        const int st = st_cur;
+        it_load.advance();
+        const int st_new = it_load.cur();
+        issue(refill, st_new);
+        st_cur = st_next;
+        st_next = st_new;
+        // the loads complete in order: one wait for the last of `cur` covers the whole set
+        asm volatile("" ::"v"(cur.val[7]));
         unsigned char *stage = smem + (s & 1) * STAGE_BYTES;
         if (st & 1)
-            prep_b<OPE>(fr, stage, role, h, c, side == 1, bad);
+            prep_b<IOE, OPE>(cur, stage, role, h, c, side == 1, bad);
         else
-            prep_r<OPE>(fr, stage, rj, rown, h, c, bad);
+            prep_r<IOE, OPE>(cur, stage, rj, rown, h, c, bad);
+        PHASE_MARK(2);
+        __syncthreads();
+        PHASE_MARK(3);
     };
 
-    // Stages alternate between two register sets.  The loop below always does a whole pair (set A,
-    // then set B), with no exit in between, so that the order of the loads in flight is the same
-    // on every path into it; an odd stage count peels the first stage off.
-    RawSet setA, setB;
-    StageIter<NB> itA(sched), itB(sched);
+    // The loop does whole triples (sets A, B, C in turn) with no exit in between, so that the order
+    // of the loads in flight is the same on every path into it; the first total % 3 stages are
+    // peeled off, with the sets assigned so that the loop starts on A.
+    RawSet setA, setB, setC;
     int s = 0;
     PHASE_BEGIN();
-    if (total & 1) {
-        itA.advance();                  // B: stage 0, A: stage 1
-        issue(setB, itB.cur(), lane_bytes);
-        issue(setA, itA.cur(), lane_bytes);
-        PHASE_SELECT((itB.cur() & 1) ? 0 : 4);
-        prepare(setB, 0, itB);
-        PHASE_MARK(2);
-        __syncthreads();
-        PHASE_MARK(3);
+    const int rem = total % 3;
+    st_cur = it_load.cur();
+    it_load.advance();
+    st_next = it_load.cur();
+    if (rem == 0) {
+        issue(setA, st_cur);
+        issue(setB, st_next);
+    } else if (rem == 1) {
+        issue(setC, st_cur);
+        issue(setA, st_next);
+        prepare(setC, setB, 0);
         s = 1;
     } else {
-        itB.advance();                  // A: stage 0, B: stage 1
-        issue(setA, itA.cur(), lane_bytes);
-        issue(setB, itB.cur(), lane_bytes);
+        issue(setB, st_cur);
+        issue(setC, st_next);
+        prepare(setB, setA, 0);
+        prepare(setC, setB, 1);
+        s = 2;
     }
-    for (; s < total; s += 2) {
-        PHASE_SELECT((itA.cur() & 1) ? 0 : 4);
-        prepare(setA, s, itA);
-        PHASE_MARK(2);
-        __syncthreads();
-        PHASE_MARK(3);
-        PHASE_SELECT((itB.cur() & 1) ? 0 : 4);
-        prepare(setB, s + 1, itB);
-        PHASE_MARK(2);
-        __syncthreads();
-        PHASE_MARK(3);
+    for (; s < total; s += 3) {
+        prepare(setA, setC, s);
+        prepare(setB, setA, s + 1);
+        prepare(setC, setB, s + 2);
     }
     // Both workgroups of a row see all four gates' blocks and reach the same verdict, so either
     // order of their writes leaves the same flag.

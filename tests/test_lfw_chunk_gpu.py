@@ -69,6 +69,34 @@ def test_config_like_inputs(dtype, gate_mean, state_std, B, T, C):
     check_against_oracle((x, f, q, k, fk, s), go, gs, C, dtype, expect_flagged=0)
 
 
+@pytest.mark.parametrize("flags", [4, 8], ids=["whole_row", "split_by_side"])
+@pytest.mark.parametrize("dtype,B,T,C", [(torch.float16, 4, 1024, 64), (torch.bfloat16, 3, 112, 64),
+                                         (torch.float16, 2, 48, 32), (torch.float16, 3, 16, 64),
+                                         (torch.bfloat16, 2, 80, 64), (torch.float16, 2, 77, 32)])
+def test_both_backward_kernels(flags, dtype, B, T, C):
+    """The backward has two matrix-core kernels (one workgroup per batch row, or one per side of the
+    state); the library picks by batch size, the flags force either.  T = 77 is not a multiple of 16,
+    which the split kernel does not take: the call must still succeed (whole-row kernel)."""
+    x, f, q, k, fk, s, go, gs = make_config_inputs(B, T, 64, 64, dtype, seed=100 + T, gate_mean=2.5, state_std=0.3)
+    check_against_oracle((x, f, q, k, fk, s), go, gs, C, dtype, flags=flags, expect_flagged=0)
+
+
+@pytest.mark.parametrize("flags", [4, 8], ids=["whole_row", "split_by_side"])
+def test_both_backward_kernels_flag_the_same_rows(flags):
+    B, T = 3, 96
+    x, f, q, k, fk, s, go, gs = make_config_inputs(B, T, 64, 64, torch.float16, seed=11, state_std=0.3)
+    f, fk = f.clone(), fk.clone()
+    f[0, 40, 9] = 0.0
+    fk[2, 90, 63] = 2.0
+    out, nxt, ckpt, grads, flagged = run_abi((x, f, q, k, fk, s), go, gs, 32, flags=flags)
+    assert flagged == (2, 2), flagged
+    r_grads = c_oracle.lfw_backward(go, gs, x, f, q, k, fk, s)
+    for n, g, r in zip(NAMES, grads, r_grads):
+        assert_close(g[0:1], r[0:1], torch.float16, n + "[flagged row 0]")
+        assert_close(g[2:3], r[2:3], torch.float16, n + "[flagged row 2]")
+        assert_close(g, r, torch.float16, n, tol=TOL_CHUNK_GATE if n in ("d_f", "d_f_key") else TOL_CHUNK)
+
+
 def test_wide_gate_distribution_stays_on_the_chunked_path():
     # gates = sigmoid(N(0,1)): 16-step products down to ~1e-10, far below what fp16 operands could carry
     x, f, q, k, fk, s, go, gs = make_config_inputs(3, 256, 64, 64, torch.float16, seed=5, gate_mean=0.0,
