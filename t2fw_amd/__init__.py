@@ -2,5 +2,6 @@
 ``LFWFunction`` / ``DFWFunction`` autograd functions)."""
 from .functional_lfw import LFWFunction, lfw_step, DEFAULT_CKPT_INTERVAL  # noqa: F401
 from .functional_dfw import DFWFunction  # noqa: F401
+from .state_cache import FastWeightState  # noqa: F401
 
-__all__ = ["LFWFunction", "DFWFunction", "lfw_step", "DEFAULT_CKPT_INTERVAL"]
+__all__ = ["LFWFunction", "DFWFunction", "FastWeightState", "lfw_step", "DEFAULT_CKPT_INTERVAL"]
