@@ -24,6 +24,8 @@
 //
 // Replaces lfw_cuda_bwd_kernel and the six einsums of the reference
 // (t2fw/csrc/lfw_kernel.cu:61-102, t2fw/csrc/lfw.cpp:84-93).
+#include <type_traits>
+
 #include "lfw_chunk_bwd_dev.hpp"
 
 namespace t2fw {
@@ -317,7 +319,6 @@ __device__ __forceinline__ void split_prep_waves(const ChunkBwdArgs &p, unsigned
     const u16 *const r_gate = rown ? GW : GO;
     const u16 *const r_val = rown ? VW : VO;
     const SplitSchedule<NB> sched(p.T, p.NC, p.C);
-    const int total = sched.total;
     u32 bad = 0;
 
     const u32 voff_own = (u32)(8 * h * CH_N + c) * 2u, voff_oth = (u32)(8 * (1 - h) * CH_N + c) * 2u;
@@ -353,13 +354,15 @@ __device__ __forceinline__ void split_prep_waves(const ChunkBwdArgs &p, unsigned
         PHASE_MARK(3);
     };
 
-    // The loop does whole triples (sets A, B, C in turn) with no exit in between, so that the order
-    // of the loads in flight is the same on every path into it; the first total % 3 stages are
-    // peeled off, with the sets assigned so that the loop starts on A.
+    // Stages are done in triples (sets A, B, C in turn) with no exit inside a triple, so that the
+    // order of the loads in flight is the same on every path.  First the stages of the last chunk of
+    // the sequence (it may be short), with the general iterator; its first (count % 3) stages are
+    // peeled off, with the sets assigned so that the triples start on A.
     RawSet setA, setB, setC;
     int s = 0;
     PHASE_BEGIN();
-    const int rem = total % 3;
+    const int n_last = sched.st_last;
+    const int rem = n_last % 3;
     st_cur = it_load.cur();
     it_load.advance();
     st_next = it_load.cur();
@@ -378,10 +381,58 @@ __device__ __forceinline__ void split_prep_waves(const ChunkBwdArgs &p, unsigned
         prepare(setC, setB, 1);
         s = 2;
     }
-    for (; s < total; s += 3) {
+    for (; s < n_last; s += 3) {
         prepare(setA, setC, s);
         prepare(setB, setA, s + 1);
         prepare(setC, setB, s + 2);
+    }
+
+    // Then the full chunks, last to first.  Inside a chunk the kind of every stage and its block are
+    // compile-time constants (position POS of PER), which leaves a pointer bump per stage for the
+    // scalar unit; PER is a multiple of three, so every chunk starts on set A.  The refill of
+    // position POS + 2 reaches into the chunk below for the last two positions (below the first
+    // chunk: that chunk again, never used).
+    constexpr int PER = (int)SplitSchedule<NB>::PER_CHUNK, NR = NB / 2;
+    static_assert(PER % 3 == 0, "a chunk must take a whole number of register-set triples");
+    const u16 *const r_gate_w = r_gate + rj * CH_L * CH_N, *const r_val_w = r_val + rj * CH_L * CH_N;
+    auto issue_at = [&](RawSet &r, int chunk_tok, auto pos_c) {
+        constexpr int POS = decltype(pos_c)::value;
+        if constexpr (POS < NR) {
+            const u32 e = (u32)(chunk_tok + 2 * POS * CH_L) * CH_N;
+            raw_issue(r, r_gate_w + e, r_val_w + e, voff_own, voff_oth);
+        } else {
+            const u32 e = (u32)(chunk_tok + (NB - 1 - (POS - NR)) * CH_L) * CH_N;
+            raw_issue(r, b_gate + e, b_val + e, voff_own, voff_oth);
+        }
+    };
+    auto prepare_at = [&](const RawSet &cur, RawSet &refill, int chunk_tok, int below_tok, auto pos_c) {
+        constexpr int POS = decltype(pos_c)::value;
+        if constexpr (POS + 2 < PER)
+            issue_at(refill, chunk_tok, std::integral_constant<int, (POS + 2) % PER>{});
+        else
+            issue_at(refill, below_tok, std::integral_constant<int, (POS + 2) % PER>{});
+        // the loads complete in order: one wait for the last of `cur` covers the whole set
+        asm volatile("" ::"v"(cur.val[7]));
+        unsigned char *stage = smem + (s & 1) * STAGE_BYTES;
+        if constexpr (POS >= NR)
+            prep_b<IOE, OPE>(cur, stage, role, h, c, side == 1, bad);
+        else
+            prep_r<IOE, OPE>(cur, stage, rj, rown, h, c, bad);
+        ++s;
+        PHASE_MARK(2);
+        __syncthreads();
+        PHASE_MARK(3);
+    };
+    for (int chunk_tok = (sched.NC - 2) * p.C; chunk_tok >= 0; chunk_tok -= p.C) {
+        const int below_tok = max(chunk_tok - p.C, 0);
+        prepare_at(setA, setC, chunk_tok, below_tok, std::integral_constant<int, 0>{});
+        prepare_at(setB, setA, chunk_tok, below_tok, std::integral_constant<int, 1>{});
+        prepare_at(setC, setB, chunk_tok, below_tok, std::integral_constant<int, 2>{});
+        if constexpr (PER == 6) {
+            prepare_at(setA, setC, chunk_tok, below_tok, std::integral_constant<int, 3>{});
+            prepare_at(setB, setA, chunk_tok, below_tok, std::integral_constant<int, 4>{});
+            prepare_at(setC, setB, chunk_tok, below_tok, std::integral_constant<int, 5>{});
+        }
     }
     // Both workgroups of a row see all four gates' blocks and reach the same verdict, so either
     // order of their writes leaves the same flag.
