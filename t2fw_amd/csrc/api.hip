@@ -73,7 +73,8 @@ int compute_units() {
     return n;
 }
 
-size_t row_flag_bytes(int64_t B) { return (size_t)((B * 4 + 255) / 256 * 256); }
+// two flag slots per batch row (kernels that split a row over two workgroups use both)
+size_t row_flag_bytes(int64_t B) { return (size_t)((2 * chunk_rows_padded(B) * 4 + 255) / 256 * 256); }
 
 int check_dims(int64_t B, int64_t T, int64_t D, int64_t K) {
     if (B < 0 || T < 0) return fail(T2FW_ERR_BAD_SHAPE, "B=%lld and T=%lld must be non-negative", (long long)B, (long long)T);
@@ -141,6 +142,7 @@ int t2fw_lfw_forward(const void *x, const void *f, const void *q, const void *k,
     a.x = x; a.f = f; a.q = q; a.k = k; a.f_key = f_key; a.s0 = s0;
     a.out = out; a.next_state = next_state; a.ckpt = ckpt;
     a.row_select = nullptr;
+    a.row_select2 = nullptr;
     a.B = B; a.T = T; a.D = D; a.K = K;
     a.C = ckpt ? C : 1;
     a.NC = ckpt ? t2fw_lfw_num_ckpt(T, C) : 1;
@@ -156,8 +158,13 @@ int t2fw_lfw_forward(const void *x, const void *f, const void *q, const void *k,
         c.row_flags = static_cast<int32_t *>(workspace);
         c.B = B; c.T = T; c.NC = a.NC; c.C = a.C;
         const int op = (dtype == T2FW_F16 && (flags & T2FW_FLAG_FP16_OPERANDS)) ? 1 : 0;
-        if ((rc = chunk_forward(c, dtype, op, st))) return rc;
+        // two workgroups per batch row while that still fits the device in one wave of workgroups
+        const int cus = compute_units();
+        if (cus < 0) return fail(T2FW_ERR_HIP, "could not read the device's compute-unit count");
+        const bool split = 2 * chunk_rows_padded(B) <= cus;
+        if ((rc = chunk_forward(c, dtype, op, split, st))) return rc;
         a.row_select = c.row_flags;      // rows the chunked form could not take
+        a.row_select2 = split ? c.row_flags + chunk_rows_padded(B) : nullptr;
     }
     return scan_forward(a, dtype, st);
 }
@@ -213,7 +220,7 @@ int t2fw_lfw_backward(const void *g_out, const void *g_state, const void *x, con
         if ((flags & (T2FW_FLAG_BWD_SPLIT | T2FW_FLAG_BWD_WHOLE_ROW)) == 0) {
             const int cus = compute_units();
             if (cus < 0) return fail(T2FW_ERR_HIP, "could not read the device's compute-unit count");
-            split = 2 * ((B + 7) / 8 * 8) <= cus && split_ok;
+            split = 2 * chunk_rows_padded(B) <= cus && split_ok;
         }
         if ((rc = split ? chunk_backward_split(c, dtype, op, st) : chunk_backward(c, dtype, op, st))) return rc;
         a.row_select = c.row_flags;      // rows the chunked form could not take

@@ -25,7 +25,7 @@ namespace t2fw {
 struct ChunkFwdArgs {
     const void *x, *f, *q, *k, *f_key, *s0;
     void *out, *next_state, *ckpt;     // ckpt may be null
-    int32_t *row_flags;                // [B]: set to 1 for rows the exact kernels must redo
+    int32_t *row_flags;                // [2 * chunk_rows_padded(B)]: set to 1 for rows the exact kernels must redo
     int64_t B, T, NC;
     int32_t C;                         // checkpoint interval, multiple of 32
 };
@@ -38,8 +38,12 @@ struct ChunkBwdArgs {
     int32_t C;
 };
 
-// op: 0 = bf16 operands, 1 = fp16 operands (fp16 I/O only)
-int chunk_forward(const ChunkFwdArgs &a, int dtype, int op, hipStream_t stream);
+// Kernels that split a batch row over two workgroups index them as half * chunk_rows_padded(B) + row
+// and use two flag slots per row, row_flags[row] and row_flags[chunk_rows_padded(B) + row].
+inline int64_t chunk_rows_padded(int64_t B) { return (B + 7) / 8 * 8; }
+
+// op: 0 = bf16 operands, 1 = fp16 operands (fp16 I/O only); split: two workgroups per batch row
+int chunk_forward(const ChunkFwdArgs &a, int dtype, int op, bool split, hipStream_t stream);
 int chunk_backward(const ChunkBwdArgs &a, int dtype, int op, hipStream_t stream);
 // same result from two workgroups per batch row (one per side of the state); for batches that leave CUs idle
 int chunk_backward_split(const ChunkBwdArgs &a, int dtype, int op, hipStream_t stream);

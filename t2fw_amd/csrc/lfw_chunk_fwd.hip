@@ -8,6 +8,11 @@
 // registers (two-byte loads, coalesced over the wave's 64 channels), two steps ahead of
 // their use; one workgroup barrier per step hands the double-buffered tiles over.
 //
+// The rows S[d, :] of the state never interact, so a batch row can also be split over two
+// workgroups by value channel (d < 32 / d >= 32): each then runs two matrix waves, the whole
+// key-side preparation (duplicated) and half of the value-side one.  The launcher does this
+// when twice the batch still fits the CUs of the device.
+//
 // Replaces lfw_cuda_fwd_kernel + the output einsum of the reference
 // (t2fw/csrc/lfw_kernel.cu:18-59, t2fw/csrc/lfw.cpp:45); semantics t2fw/torch.py:21-31.
 #include "lfw_chunk.hpp"
@@ -27,7 +32,8 @@
 namespace t2fw {
 namespace {
 
-constexpr int FWD_THREADS = 768;
+constexpr int FWD_THREADS = 768;          // one workgroup per batch row: 4 matrix + 8 prep waves
+constexpr int FWD_THREADS_HALF = 512;     // two per batch row: 2 matrix + 4 key-side + 2 value-side prep waves
 
 // ---- LDS layout of one operand buffer (bytes) -------------------------------------------
 constexpr int OFF_QT = 0;                                  // qs  token-major  [32][TS] u16, channels at tm_pos
@@ -189,11 +195,13 @@ __device__ __forceinline__ float scale_half(const RawF<NV> &f, int h, float (&pr
 
 // One side of the prep work for the whole sequence: KEY = true builds qs, kt (token-major), kh
 // (channel-major) and b_L from f_key, k, q; KEY = false builds xt, xh, a_t and a_L from f, x.
+// c: this lane's channel; hh: block of the step (wave-uniform); h: token half (wave-uniform, or
+// per lane when a wave covers both halves of 32 channels); flag_slot: where this workgroup
+// reports rows the chunked form cannot take.
 template <typename IOE, typename OPE, bool KEY>
-__device__ __forceinline__ void fwd_prep_side(const ChunkFwdArgs &p, unsigned char *smem, int tid, int64_t b, int hh,
-                                              int h) {
+__device__ __forceinline__ void fwd_prep_side(const ChunkFwdArgs &p, unsigned char *smem, int tid, int64_t b, int c,
+                                              int hh, int h, int64_t flag_slot) {
     constexpr int NV = KEY ? 2 : 1;
-    const int c = tid & 63;
     const int T = (int)p.T;                                // the launcher admits T < 2^24 only
     const int64_t row_off = b * p.T * CH_N;
     const u16 *const gate = reinterpret_cast<const u16 *>(KEY ? p.f_key : p.f) + row_off;
@@ -293,7 +301,7 @@ __device__ __forceinline__ void fwd_prep_side(const ChunkFwdArgs &p, unsigned ch
         build(raw_take_tail<IOE, NV>(r, t_own, t_oth, T), nfull);
         __syncthreads();
     }
-    if (bad) p.row_flags[b] = 1;
+    if (bad) p.row_flags[flag_slot] = 1;
     PHASE_END(4 + (tid >> 6));
 }
 
@@ -310,9 +318,10 @@ __device__ __forceinline__ void store_state(const floatx4 (&S)[4], u16 *dst, int
 }
 
 template <typename IOE, typename OPE>
-__device__ __forceinline__ void fwd_matrix_waves(const ChunkFwdArgs &p, unsigned char *smem, int tid, int64_t b) {
+__device__ __forceinline__ void fwd_matrix_waves(const ChunkFwdArgs &p, unsigned char *smem, int tid, int64_t b,
+                                                 int dbase, int64_t flag_slot) {
     const int w = tid >> 6, l = tid & 63, r = l & 15, g = l >> 4;
-    const int d = 16 * w + r;                  // this lane's state row (value channel)
+    const int d = dbase + 16 * w + r;          // this lane's state row (value channel)
     const int T = (int)p.T;
     u16 *ckpt = reinterpret_cast<u16 *>(p.ckpt);
     u16 *const out = reinterpret_cast<u16 *>(p.out) + b * p.T * CH_N;
@@ -332,7 +341,7 @@ __device__ __forceinline__ void fwd_matrix_waves(const ChunkFwdArgs &p, unsigned
     const int nsteps = (T + CH_STEP - 1) / CH_STEP;
     int until_ckpt = 0;
     int64_t chunk = 0;
-    if (tid == 0) p.row_flags[b] = 0;
+    if (tid == 0) p.row_flags[flag_slot] = 0;
     PHASE_BEGIN();
     for (int n = 0; n < nsteps; ++n) {
         __syncthreads();        // the operand tiles of step n are in LDS
@@ -413,36 +422,71 @@ __global__ __launch_bounds__(FWD_THREADS) void lfw_fwd_chunk_kernel(ChunkFwdArgs
     const int64_t b = blockIdx.x;
     // every wave executes exactly (number of steps) workgroup barriers
     if (tid < 256) {
-        fwd_matrix_waves<IOE, OPE>(p, smem, tid, b);
+        fwd_matrix_waves<IOE, OPE>(p, smem, tid, b, 0, b);
     } else {
         // prep wave pw: (side, block of the step, token half); each SIMD gets one wave of each side
         const int pw = __builtin_amdgcn_readfirstlane((tid - 256) >> 6);
         const int hh = (pw >> 1) & 1, h = pw >> 2;
         if (((pw ^ h) & 1) == 0)
-            fwd_prep_side<IOE, OPE, true>(p, smem, tid - 256, b, hh, h);
+            fwd_prep_side<IOE, OPE, true>(p, smem, tid - 256, b, tid & 63, hh, h, b);
         else
-            fwd_prep_side<IOE, OPE, false>(p, smem, tid - 256, b, hh, h);
+            fwd_prep_side<IOE, OPE, false>(p, smem, tid - 256, b, tid & 63, hh, h, b);
     }
 }
 
-template <typename IOE, typename OPE> int launch(const ChunkFwdArgs &a, hipStream_t stream) {
-    auto kern = lfw_fwd_chunk_kernel<IOE, OPE>;
+// Two workgroups per batch row: blockIdx = half * rows_padded + row with rows_padded a multiple of
+// 8, so that the two halves of a row land on the same XCD and share its L2 for the key-side
+// inputs both of them read.  Each half reports flagged rows in a slot of its own (the value-side
+// gates it checks are its own 32 channels): row_flags[row] and row_flags[rows_padded + row].
+template <typename IOE, typename OPE>
+__global__ __launch_bounds__(FWD_THREADS_HALF) void lfw_fwd_chunk_half_kernel(ChunkFwdArgs p, int rows_padded) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    const int tid = threadIdx.x;
+    const int half = (int)blockIdx.x >= rows_padded ? 1 : 0;
+    const int64_t b = (int)blockIdx.x - half * rows_padded;
+    if (b >= p.B) return;
+    const int64_t slot = (int64_t)half * rows_padded + b;
+    // waves: 0, 1 matrix; 2..5 key side (block, token half); 6, 7 value side (block; a lane takes
+    // one of the half's 32 channels and one token half).  SIMD i runs waves i and i + 4.
+    if (tid < 128) {
+        fwd_matrix_waves<IOE, OPE>(p, smem, tid, b, 32 * half, slot);
+    } else if (tid < 384) {
+        const int pw = __builtin_amdgcn_readfirstlane((tid - 128) >> 6);
+        fwd_prep_side<IOE, OPE, true>(p, smem, tid - 128, b, tid & 63, pw & 1, pw >> 1, slot);
+    } else {
+        const int pw = __builtin_amdgcn_readfirstlane((tid - 384) >> 6);
+        fwd_prep_side<IOE, OPE, false>(p, smem, tid - 128, b, 32 * half + (tid & 31), pw, (tid >> 5) & 1, slot);
+    }
+}
+
+template <typename IOE, typename OPE> int launch(const ChunkFwdArgs &a, bool split, hipStream_t stream) {
+    if (a.B > 0x1fffffffLL) return fail(T2FW_ERR_UNSUPPORTED, "B=%lld is too large", (long long)a.B);
+    if (a.T >= CHUNK_MAX_T) return fail(T2FW_ERR_UNSUPPORTED, "T=%lld is too long for 32-bit row offsets", (long long)a.T);
     // more than 64 KB of dynamic LDS has to be enabled per function (and per device)
+    if (split) {
+        auto kern = lfw_fwd_chunk_half_kernel<IOE, OPE>;
+        int rc = check_hip(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, FWD_SMEM),
+                           "hipFuncSetAttribute(forward chunk kernel, two workgroups per row)");
+        if (rc) return rc;
+        const int rows_padded = (int)chunk_rows_padded(a.B);
+        hipLaunchKernelGGL(kern, dim3(2u * (unsigned)rows_padded), dim3(FWD_THREADS_HALF), FWD_SMEM, stream, a, rows_padded);
+        return check_hip(hipGetLastError(), "lfw_fwd_chunk_half_kernel launch");
+    }
+    auto kern = lfw_fwd_chunk_kernel<IOE, OPE>;
     int rc = check_hip(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, FWD_SMEM),
                        "hipFuncSetAttribute(forward chunk kernel)");
     if (rc) return rc;
-    if (a.B > 0x7fffffffLL) return fail(T2FW_ERR_UNSUPPORTED, "B=%lld is too large", (long long)a.B);
-    if (a.T >= CHUNK_MAX_T) return fail(T2FW_ERR_UNSUPPORTED, "T=%lld is too long for 32-bit row offsets", (long long)a.T);
     hipLaunchKernelGGL(kern, dim3((unsigned)a.B), dim3(FWD_THREADS), FWD_SMEM, stream, a);
     return check_hip(hipGetLastError(), "lfw_fwd_chunk_kernel launch");
 }
 
 }  // namespace
 
-int chunk_forward(const ChunkFwdArgs &a, int dtype, int op, hipStream_t stream) {
-    if (dtype == T2FW_F16) return op == 1 ? launch<Fp16, Fp16>(a, stream) : launch<Fp16, Bf16>(a, stream);
-    if (dtype == T2FW_BF16) return launch<Bf16, Bf16>(a, stream);
+int chunk_forward(const ChunkFwdArgs &a, int dtype, int op, bool split, hipStream_t stream) {
+    if (dtype == T2FW_F16) return op == 1 ? launch<Fp16, Fp16>(a, split, stream) : launch<Fp16, Bf16>(a, split, stream);
+    if (dtype == T2FW_BF16) return launch<Bf16, Bf16>(a, split, stream);
     return fail(T2FW_ERR_UNSUPPORTED, "the chunked kernels take fp16 or bf16 tensors");
 }
 

@@ -38,7 +38,7 @@ __global__ __launch_bounds__(SCAN_THREADS) void lfw_fwd_scan_kernel(ScanFwdArgs 
     Acc *outL = rowL + (size_t)tb * 2 * g.rows;          // [tb][rows]
 
     const int64_t b = blockIdx.x / p.ntiles;
-    if (p.row_select && p.row_select[b] == 0) return;     // uniform per workgroup
+    if (p.row_select && p.row_select[b] == 0 && !(p.row_select2 && p.row_select2[b] != 0)) return;     // uniform per workgroup
     const int64_t T = p.T, D = p.D, K = p.K;
     const int64_t d0 = (int64_t)(blockIdx.x % p.ntiles) * g.rows;
     const int64_t d = d0 + g.r;

@@ -8,7 +8,8 @@ namespace t2fw {
 struct ScanFwdArgs {
     const void *x, *f, *q, *k, *f_key, *s0;
     void *out, *next_state, *ckpt;      // ckpt may be null
-    const int32_t *row_select;          // null, or per batch row: 0 = skip the row
+    const int32_t *row_select;          // null, or per batch row: 0 = skip the row ...
+    const int32_t *row_select2;         // ... unless this second per-row array (may be null) is nonzero there
     int64_t B, T, D, K, NC;
     int32_t C, kg, tb, ntiles;
 };

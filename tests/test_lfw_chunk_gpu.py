@@ -13,6 +13,14 @@ pytestmark = pytest.mark.gpu
 NAMES = ("d_x", "d_f", "d_q", "d_k", "d_f_key", "d_state")
 
 
+def flagged_rows(ws, B):
+    """rows the matrix-core kernels handed to the exact kernels: two flag slots per row (kernels that
+    split a row over two workgroups report per workgroup), the second at the batch padded to 8"""
+    f = ws.view(torch.int32)
+    pad = (B + 7) // 8 * 8
+    return int(((f[:B] != 0) | (f[pad:pad + B] != 0)).sum())
+
+
 def run_abi(inputs, go, gs, C, flags=0, with_backward=True):
     """forward (+ backward) through the C ABI; returns out, next_state, ckpt, grads, flagged rows"""
     from t2fw_amd import _lib
@@ -31,7 +39,7 @@ def run_abi(inputs, go, gs, C, flags=0, with_backward=True):
     _lib.check(lib.t2fw_lfw_forward(*[_lib.ptr(t) for t in ins], _lib.ptr(out), _lib.ptr(nxt), _lib.ptr(ckpt),
                                     B, T, D, K, C, code, flags, _lib.ptr(ws), wsb, st))
     torch.cuda.synchronize()
-    flagged_fwd = int(ws[:4 * B].view(torch.int32).sum()) if wsb else 0
+    flagged_fwd = flagged_rows(ws, B) if wsb else 0
     grads, flagged_bwd = None, 0
     if with_backward:
         grads = [torch.empty_like(t) for t in ins]
@@ -40,7 +48,7 @@ def run_abi(inputs, go, gs, C, flags=0, with_backward=True):
                                          _lib.ptr(ckpt), *[_lib.ptr(t) for t in grads], B, T, D, K, C, code, flags,
                                          _lib.ptr(ws), wsb, st))
         torch.cuda.synchronize()
-        flagged_bwd = int(ws[:4 * B].view(torch.int32).sum()) if wsb else 0
+        flagged_bwd = flagged_rows(ws, B) if wsb else 0
     return out, nxt, ckpt, grads, (flagged_fwd, flagged_bwd)
 
 
@@ -112,13 +120,16 @@ def test_reference_test_gates_stay_on_the_chunked_path():
                          gate_tol=(2e-1, 4e-2))
 
 
-@pytest.mark.parametrize("kind", ["zero_gate", "gate_above_one", "negative_gate", "tiny_product", "nan_free_inf_gate"])
+@pytest.mark.parametrize("kind", ["zero_gate", "zero_gate_upper_channels", "gate_above_one", "negative_gate",
+                                  "tiny_product", "nan_free_inf_gate"])
 def test_rows_outside_the_gate_range_fall_back_to_the_exact_kernels(kind):
     B, T = 4, 160
     x, f, q, k, fk, s, go, gs = make_config_inputs(B, T, 64, 64, torch.float16, seed=3, state_std=0.3)
     f, fk = f.clone(), fk.clone()
     if kind == "zero_gate":
         f[1, 70, 5] = 0.0
+    elif kind == "zero_gate_upper_channels":
+        f[1, 70, 40] = 0.0              # seen only by the workgroup that owns value channels 32..63
     elif kind == "gate_above_one":
         fk[1, 3, 60] = 1.5
     elif kind == "negative_gate":
