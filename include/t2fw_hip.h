@@ -76,7 +76,14 @@ extern "C" {
 #define T2FW_FLAG_BWD_WHOLE_ROW 4 /* backward, matrix-core path: one workgroup per batch row  */
 #define T2FW_FLAG_BWD_SPLIT 8     /* backward, matrix-core path: two workgroups per batch row
                                      (value side / key side).  With neither bit the library
-                                     splits when twice the batch fits the device's CUs.      */
+                                     splits when twice the batch fits the device's CUs
+                                     (and T % 16 == 0, which the split kernel needs).        */
+#define T2FW_FLAG_NO_FIXUP 16     /* matrix-core path: do not launch the exact kernels for the
+                                     rows it flagged; the caller reads the flags from the
+                                     workspace (int32 [2][B rounded up to 8], nonzero in either
+                                     slot = that row's results are not valid) and redoes those
+                                     rows with T2FW_FLAG_FORCE_SCAN, or knows its gates are in
+                                     range.  Saves one launch per call.                         */
 
 int t2fw_abi_version(void);
 const char *t2fw_last_error(void);

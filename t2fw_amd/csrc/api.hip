@@ -165,6 +165,7 @@ int t2fw_lfw_forward(const void *x, const void *f, const void *q, const void *k,
         if ((rc = chunk_forward(c, dtype, op, split, st))) return rc;
         a.row_select = c.row_flags;      // rows the chunked form could not take
         a.row_select2 = split ? c.row_flags + chunk_rows_padded(B) : nullptr;
+        if (flags & T2FW_FLAG_NO_FIXUP) return T2FW_OK;
     }
     return scan_forward(a, dtype, st);
 }
@@ -224,6 +225,7 @@ int t2fw_lfw_backward(const void *g_out, const void *g_state, const void *x, con
         }
         if ((rc = split ? chunk_backward_split(c, dtype, op, st) : chunk_backward(c, dtype, op, st))) return rc;
         a.row_select = c.row_flags;      // rows the chunked form could not take
+        if (flags & T2FW_FLAG_NO_FIXUP) return T2FW_OK;
     }
     return scan_backward(a, dtype, st);
 }

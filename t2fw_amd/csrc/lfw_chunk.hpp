@@ -33,14 +33,14 @@ struct ChunkFwdArgs {
 struct ChunkBwdArgs {
     const void *g_out, *g_state, *x, *f, *q, *k, *f_key, *ckpt;
     void *d_x, *d_f, *d_q, *d_k, *d_f_key, *d_s0;
-    int32_t *row_flags;
+    int32_t *row_flags;                // as for the forward
     int64_t B, T, NC;
     int32_t C;
 };
 
 // Kernels that split a batch row over two workgroups index them as half * chunk_rows_padded(B) + row
 // and use two flag slots per row, row_flags[row] and row_flags[chunk_rows_padded(B) + row].
-inline int64_t chunk_rows_padded(int64_t B) { return (B + 7) / 8 * 8; }
+__host__ __device__ inline int64_t chunk_rows_padded(int64_t B) { return (B + 7) / 8 * 8; }
 
 // op: 0 = bf16 operands, 1 = fp16 operands (fp16 I/O only); split: two workgroups per batch row
 int chunk_forward(const ChunkFwdArgs &a, int dtype, int op, bool split, hipStream_t stream);

@@ -195,7 +195,10 @@ __device__ __forceinline__ void bwd_prep_waves(const ChunkBwdArgs &p, unsigned c
     const Schedule<NB> sched(T, p.NC, p.C);
     const int total = sched.total;
     u32 bad = 0;
-    if (tid == 0) p.row_flags[b] = 0;
+    if (tid == 0) {      // both flag slots of the row (the backward kernels report in the first)
+        p.row_flags[b] = 0;
+        p.row_flags[chunk_rows_padded(p.B) + b] = 0;
+    }
     auto tok0_of = [&](const StageInfo &si) -> int64_t { return (int64_t)si.chunk * p.C + si.block * CH_L; };
 
     PieceMap pm;

@@ -485,7 +485,10 @@ __device__ __forceinline__ void split_matrix_waves(const ChunkBwdArgs &p, unsign
     load_state(ckpt + (NC - 1) * (CH_N * CH_N), pf);
     float carry = 0.f;
     int s = 0;
-    if (tid == 0) p.row_flags[b] = 0;
+    if (tid == 0) {      // both flag slots of the row (the backward kernels report in the first)
+        p.row_flags[b] = 0;
+        p.row_flags[chunk_rows_padded(p.B) + b] = 0;
+    }
     PHASE_BEGIN();
 
     // every stage starts with the workgroup barrier that publishes its operand tiles

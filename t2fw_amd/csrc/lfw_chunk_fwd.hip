@@ -319,7 +319,7 @@ __device__ __forceinline__ void store_state(const floatx4 (&S)[4], u16 *dst, int
 
 template <typename IOE, typename OPE>
 __device__ __forceinline__ void fwd_matrix_waves(const ChunkFwdArgs &p, unsigned char *smem, int tid, int64_t b,
-                                                 int dbase, int64_t flag_slot) {
+                                                 int dbase, int64_t flag_slot, bool clear_other_slot) {
     const int w = tid >> 6, l = tid & 63, r = l & 15, g = l >> 4;
     const int d = dbase + 16 * w + r;          // this lane's state row (value channel)
     const int T = (int)p.T;
@@ -341,7 +341,10 @@ __device__ __forceinline__ void fwd_matrix_waves(const ChunkFwdArgs &p, unsigned
     const int nsteps = (T + CH_STEP - 1) / CH_STEP;
     int until_ckpt = 0;
     int64_t chunk = 0;
-    if (tid == 0) p.row_flags[flag_slot] = 0;
+    if (tid == 0) {
+        p.row_flags[flag_slot] = 0;
+        if (clear_other_slot) p.row_flags[chunk_rows_padded(p.B) + b] = 0;
+    }
     PHASE_BEGIN();
     for (int n = 0; n < nsteps; ++n) {
         __syncthreads();        // the operand tiles of step n are in LDS
@@ -422,7 +425,7 @@ __global__ __launch_bounds__(FWD_THREADS) void lfw_fwd_chunk_kernel(ChunkFwdArgs
     const int64_t b = blockIdx.x;
     // every wave executes exactly (number of steps) workgroup barriers
     if (tid < 256) {
-        fwd_matrix_waves<IOE, OPE>(p, smem, tid, b, 0, b);
+        fwd_matrix_waves<IOE, OPE>(p, smem, tid, b, 0, b, true);
     } else {
         // prep wave pw: (side, block of the step, token half); each SIMD gets one wave of each side
         const int pw = __builtin_amdgcn_readfirstlane((tid - 256) >> 6);
@@ -449,7 +452,7 @@ __global__ __launch_bounds__(FWD_THREADS_HALF) void lfw_fwd_chunk_half_kernel(Ch
     // waves: 0, 1 matrix; 2..5 key side (block, token half); 6, 7 value side (block; a lane takes
     // one of the half's 32 channels and one token half).  SIMD i runs waves i and i + 4.
     if (tid < 128) {
-        fwd_matrix_waves<IOE, OPE>(p, smem, tid, b, 32 * half, slot);
+        fwd_matrix_waves<IOE, OPE>(p, smem, tid, b, 32 * half, slot, false);
     } else if (tid < 384) {
         const int pw = __builtin_amdgcn_readfirstlane((tid - 128) >> 6);
         fwd_prep_side<IOE, OPE, true>(p, smem, tid - 128, b, tid & 63, pw & 1, pw >> 1, slot);
