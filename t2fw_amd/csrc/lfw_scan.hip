@@ -27,8 +27,9 @@ using namespace scan;
 // ------------------------------------------------------------------------------------
 // forward
 // ------------------------------------------------------------------------------------
+// batch row b, tile of g.rows value channels
 template <typename IO, int KPL>
-__global__ __launch_bounds__(SCAN_THREADS) void lfw_fwd_scan_kernel(ScanFwdArgs p) {
+__device__ __forceinline__ void fwd_scan_body(const ScanFwdArgs &p, int64_t b, int tile) {
     using Acc = typename AccOf<IO>::type;
     extern __shared__ __align__(16) unsigned char smem_raw[];
     const Tile g(p.kg, KPL);
@@ -37,10 +38,8 @@ __global__ __launch_bounds__(SCAN_THREADS) void lfw_fwd_scan_kernel(ScanFwdArgs 
     Acc *rowL = colL + (size_t)tb * 3 * g.KP;            // [tb][2][rows] x, f
     Acc *outL = rowL + (size_t)tb * 2 * g.rows;          // [tb][rows]
 
-    const int64_t b = blockIdx.x / p.ntiles;
-    if (p.row_select && p.row_select[b] == 0 && !(p.row_select2 && p.row_select2[b] != 0)) return;     // uniform per workgroup
     const int64_t T = p.T, D = p.D, K = p.K;
-    const int64_t d0 = (int64_t)(blockIdx.x % p.ntiles) * g.rows;
+    const int64_t d0 = (int64_t)tile * g.rows;
     const int64_t d = d0 + g.r;
     const bool row_ok = d < D;
 
@@ -118,6 +117,23 @@ __global__ __launch_bounds__(SCAN_THREADS) void lfw_fwd_scan_kernel(ScanFwdArgs 
     }
 }
 
+// Normal mode: one workgroup per (batch row, tile).  Fix-up mode (row_select given): one
+// workgroup per batch row that walks the tiles itself, so that the launch, in which nearly all
+// workgroups leave at once, dispatches as few of them as possible.
+template <typename IO, int KPL>
+__global__ __launch_bounds__(SCAN_THREADS) void lfw_fwd_scan_kernel(ScanFwdArgs p) {
+    if (p.row_select == nullptr) {
+        fwd_scan_body<IO, KPL>(p, blockIdx.x / p.ntiles, (int)(blockIdx.x % p.ntiles));
+        return;
+    }
+    const int64_t b = blockIdx.x;
+    if (p.row_select[b] == 0 && !(p.row_select2 && p.row_select2[b] != 0)) return;     // uniform per workgroup
+    for (int tile = 0; tile < p.ntiles; ++tile) {
+        if (tile) __syncthreads();
+        fwd_scan_body<IO, KPL>(p, b, tile);
+    }
+}
+
 // ------------------------------------------------------------------------------------
 // backward, one side.  "rows" are the dimension this launch keeps per lane-group,
 // "cols" the dimension it reduces over:
@@ -134,7 +150,7 @@ __global__ __launch_bounds__(SCAN_THREADS) void lfw_fwd_scan_kernel(ScanFwdArgs 
 template <int KPL> struct SegLen { static constexpr int value = (32 / KPL) < 1 ? 1 : (KPL <= 4 ? 8 : 32 / KPL); };
 
 template <typename IO, int KPL, int SIDE>
-__device__ __forceinline__ void bwd_scan_body(const ScanBwdArgs &p) {
+__device__ __forceinline__ void bwd_scan_body(const ScanBwdArgs &p, int64_t b, int tile) {
     using Acc = typename AccOf<IO>::type;
     constexpr int SEG = SegLen<KPL>::value;
     extern __shared__ __align__(16) unsigned char smem_raw[];
@@ -144,11 +160,9 @@ __device__ __forceinline__ void bwd_scan_body(const ScanBwdArgs &p) {
     Acc *outL = rowL + (size_t)SEG * 3 * g.rows;         // [SEG][3][rows] d_a, d_gate, d_u
     Acc *subL = outL + (size_t)SEG * 3 * g.rows;         // [nseg_max][KPL][SCAN_THREADS]
 
-    const int64_t b = blockIdx.x / p.ntiles;
-    if (p.row_select && p.row_select[b] == 0) return;
     const int64_t T = p.T;
     const int64_t nrows = SIDE == 0 ? p.D : p.K, ncols = SIDE == 0 ? p.K : p.D;
-    const int64_t row0 = (int64_t)(blockIdx.x % p.ntiles) * g.rows;
+    const int64_t row0 = (int64_t)tile * g.rows;
     const int64_t row = row0 + g.r;
     const bool row_ok = row < nrows;
     const int64_t DK = p.D * p.K;
@@ -301,9 +315,23 @@ __device__ __forceinline__ void bwd_scan_body(const ScanBwdArgs &p) {
     }
 }
 
+// workgroup -> (batch row, tiles): as for the forward kernel
+template <typename IO, int KPL, int SIDE> __device__ __forceinline__ void bwd_scan_rows(const ScanBwdArgs &p) {
+    if (p.row_select == nullptr) {
+        bwd_scan_body<IO, KPL, SIDE>(p, blockIdx.x / p.ntiles, (int)(blockIdx.x % p.ntiles));
+        return;
+    }
+    const int64_t b = blockIdx.x;
+    if (p.row_select[b] == 0) return;
+    for (int tile = 0; tile < p.ntiles; ++tile) {
+        if (tile) __syncthreads();
+        bwd_scan_body<IO, KPL, SIDE>(p, b, tile);
+    }
+}
+
 template <typename IO, int KPL, int SIDE>
 __global__ __launch_bounds__(SCAN_THREADS) void lfw_bwd_scan_kernel(ScanBwdArgs p) {
-    bwd_scan_body<IO, KPL, SIDE>(p);
+    bwd_scan_rows<IO, KPL, SIDE>(p);
 }
 
 // Both sides in one launch (blockIdx.y = side) for square states, where the two sides share
@@ -312,9 +340,9 @@ __global__ __launch_bounds__(SCAN_THREADS) void lfw_bwd_scan_kernel(ScanBwdArgs 
 template <typename IO, int KPL>
 __global__ __launch_bounds__(SCAN_THREADS) void lfw_bwd_scan_both_kernel(ScanBwdArgs p) {
     if (blockIdx.y == 0)
-        bwd_scan_body<IO, KPL, 0>(p);
+        bwd_scan_rows<IO, KPL, 0>(p);
     else
-        bwd_scan_body<IO, KPL, 1>(p);
+        bwd_scan_rows<IO, KPL, 1>(p);
 }
 
 // ------------------------------------------------------------------------------------
@@ -326,7 +354,7 @@ int launch_fwd(const ScanFwdArgs &a, const ScanGeom &g, hipStream_t stream) {
     const size_t smem = ((size_t)a.tb * 3 * g.kg * g.kpl + (size_t)a.tb * 3 * g.rows) * sizeof(Acc);
     ScanFwdArgs a2 = a;
     a2.ntiles = (int)((a.D + g.rows - 1) / g.rows);
-    const int64_t nblocks = a.B * a2.ntiles;
+    const int64_t nblocks = a.row_select != nullptr ? a.B : a.B * a2.ntiles;
     if (nblocks > 0x7fffffffLL) return fail(T2FW_ERR_UNSUPPORTED, "grid of %lld workgroups is too large", (long long)nblocks);
     dim3 grid((unsigned)nblocks, 1, 1);
     hipLaunchKernelGGL((lfw_fwd_scan_kernel<IO, KPL>), grid, dim3(SCAN_THREADS), smem, stream, a2);
@@ -345,7 +373,7 @@ int launch_bwd(ScanBwdArgs a, const ScanGeom &g, hipStream_t stream) {
     const size_t smem = base + (a.use_sub ? sub : 0);
     a.kg = g.kg;
     a.ntiles = (int)((nrows + g.rows - 1) / g.rows);
-    const int64_t nblocks = a.B * a.ntiles;
+    const int64_t nblocks = a.row_select != nullptr ? a.B : a.B * a.ntiles;
     if (nblocks > 0x7fffffffLL) return fail(T2FW_ERR_UNSUPPORTED, "grid of %lld workgroups is too large", (long long)nblocks);
     if (SIDE == 2) {
         hipLaunchKernelGGL((lfw_bwd_scan_both_kernel<IO, KPL>), dim3((unsigned)nblocks, 2, 1), dim3(SCAN_THREADS), smem,
