@@ -73,12 +73,7 @@ extern "C" {
 #define T2FW_FLAG_FP16_OPERANDS 2 /* fp16 tensors: fp16 (not bf16) matrix-core operands;
                                      more mantissa, but rows whose 16-step gate products
                                      fall below 2^-8 take the exact scan path          */
-#define T2FW_FLAG_BWD_WHOLE_ROW 4 /* backward, matrix-core path: one workgroup per batch row  */
-#define T2FW_FLAG_BWD_SPLIT 8     /* backward, matrix-core path: two workgroups per batch row
-                                     (value side / key side).  With neither bit the library
-                                     splits when twice the batch fits the device's CUs
-                                     (and T % 16 == 0, which the split kernel needs).        */
-#define T2FW_FLAG_NO_FIXUP 16     /* matrix-core path: do not launch the exact kernels for the
+#define T2FW_FLAG_NO_FIXUP 4      /* matrix-core path: do not launch the exact kernels for the
                                      rows it flagged; the caller reads the flags from the
                                      workspace (int32 [2][B rounded up to 8], nonzero in either
                                      slot = that row's results are not valid) and redoes those

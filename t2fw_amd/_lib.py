@@ -20,9 +20,7 @@ DTYPE_CODE = {torch.float32: F32, torch.float16: F16, torch.bfloat16: BF16, torc
 FLAG_AUTO = 0
 FLAG_FORCE_SCAN = 1
 FLAG_FP16_OPERANDS = 2
-FLAG_BWD_WHOLE_ROW = 4
-FLAG_BWD_SPLIT = 8
-FLAG_NO_FIXUP = 16
+FLAG_NO_FIXUP = 4
 
 _vp, _i64, _i32, _sz = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int32, ctypes.c_size_t
 

@@ -205,7 +205,7 @@ int t2fw_lfw_backward(const void *g_out, const void *g_state, const void *x, con
     a.B = B; a.T = T; a.D = D; a.K = K; a.C = C;
     a.NC = t2fw_lfw_num_ckpt(T, C);
 
-    if (chunk_shape_ok(D, K, dtype, flags) && (C == 32 || C == 64) &&
+    if (chunk_shape_ok(D, K, dtype, flags) && (C == 32 || C == 64) && T < CHUNK_MAX_T &&
         aligned16({g_out, g_state, x, f, q, k, f_key, ckpt, d_x, d_f, d_q, d_k, d_f_key, d_s0})) {
         if (workspace == nullptr || workspace_bytes < row_flag_bytes(B))
             return fail(T2FW_ERR_WORKSPACE, "workspace of %zu bytes needed, %zu given", row_flag_bytes(B),
@@ -216,14 +216,7 @@ int t2fw_lfw_backward(const void *g_out, const void *g_state, const void *x, con
         c.row_flags = static_cast<int32_t *>(workspace);
         c.B = B; c.T = T; c.NC = a.NC; c.C = C;
         const int op = (dtype == T2FW_F16 && (flags & T2FW_FLAG_FP16_OPERANDS)) ? 1 : 0;
-        const bool split_ok = T < CHUNK_MAX_T && T % 16 == 0;
-        bool split = (flags & T2FW_FLAG_BWD_SPLIT) != 0 && split_ok;
-        if ((flags & (T2FW_FLAG_BWD_SPLIT | T2FW_FLAG_BWD_WHOLE_ROW)) == 0) {
-            const int cus = compute_units();
-            if (cus < 0) return fail(T2FW_ERR_HIP, "could not read the device's compute-unit count");
-            split = 2 * chunk_rows_padded(B) <= cus && split_ok;
-        }
-        if ((rc = split ? chunk_backward_split(c, dtype, op, st) : chunk_backward(c, dtype, op, st))) return rc;
+        if ((rc = chunk_backward(c, dtype, op, st))) return rc;
         a.row_select = c.row_flags;      // rows the chunked form could not take
         if (flags & T2FW_FLAG_NO_FIXUP) return T2FW_OK;
     }

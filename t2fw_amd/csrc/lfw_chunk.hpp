@@ -44,9 +44,8 @@ __host__ __device__ inline int64_t chunk_rows_padded(int64_t B) { return (B + 7)
 
 // op: 0 = bf16 operands, 1 = fp16 operands (fp16 I/O only); split: two workgroups per batch row
 int chunk_forward(const ChunkFwdArgs &a, int dtype, int op, bool split, hipStream_t stream);
+// two workgroups per batch row (one per side of the state)
 int chunk_backward(const ChunkBwdArgs &a, int dtype, int op, hipStream_t stream);
-// same result from two workgroups per batch row (one per side of the state); for batches that leave CUs idle
-int chunk_backward_split(const ChunkBwdArgs &a, int dtype, int op, hipStream_t stream);
 constexpr int64_t CHUNK_MAX_T = 1 << 24;      // the forward and the split backward kernel address a batch row with 32-bit offsets
 
 #if defined(__HIPCC__)

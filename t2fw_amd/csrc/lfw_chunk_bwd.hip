@@ -1,8 +1,9 @@
-// Backward pass of the decay rule in chunked matrix-core form (algebra: lfw_chunk.hpp).
+// Backward pass of the decay rule in chunked matrix-core form (block algebra: lfw_chunk.hpp),
+// two workgroups per batch row.
 //
-// With G = dL/dS flowing backwards in time, Gb the adjoint entering a 16-step block from
-// the future, S0 the state at the block start and the block-local scalings of
-// lfw_chunk.hpp (qs, kt, kh, xt, xh, gs = g*a_t):
+// With G = dL/dS flowing backwards in time, Gb the adjoint entering a 16-step block from the
+// future, S0 the state at the block start and the block-local scalings of lfw_chunk.hpp
+// (qs, kt, kh, xt, xh, gs = g*a_t):
 //   P[t,s] = qs_t.kt_s      W[t,s] = gs_t.xt_s
 //   o'_t  = a_t  * ( S0 qs_t            + sum_{s<t} P[t,s] xt_s )       (output without its own write)
 //   dq'_t = b_t  * ( S0^T gs_t          + sum_{s<t} W[t,s] kt_s )
@@ -15,17 +16,34 @@
 // u and v are re-anchored at every checkpoint boundary from the states themselves
 // (u = rowsum(Gb*S_end), v = colsum(Gb*S_end)), so rounding does not accumulate over T.
 //
-// One workgroup (8 waves) per batch row.  Matrix wave w holds, in fp32 accumulators, the
-// slabs S[16w.., :] / Gb[16w.., :] ("D copy", indexed [k][d]) and S[:, 16w..] / Gb[:, 16w..]
-// ("K copy", indexed [d][k]) so that every contraction is local to a wave.  Chunks are
-// visited last to first; inside a chunk a forward sweep ("R" stages) recomputes the
-// block-start states from the checkpoint and keeps them as 16-bit operands in registers,
-// then the blocks are visited last to first ("B" stages).  Four prep waves build the
-// operand tiles of the next stage, prefetch raw inputs and write the previous stage's
-// gradients; one barrier per stage.
+// The recurrence is symmetric under (x, f, g_out, D) <-> (k, f_key, q, K) with the state
+// transposed, so the two sides get a workgroup (and a CU) each and nothing is exchanged:
+//   side 0 ("value side"): own = (x, f, g_out), other = (k, f_key, q); writes d_x, d_f, d_s0
+//   side 1 ("key side")  : own = (k, f_key, q), other = (x, f, g_out); writes d_k, d_f_key, d_q
+// In the names below V = own value (x | k), A = own adjoint (g_out | q), VO / AO the other
+// side's, a suffix S / T / H = scaled by the gate prefix / divided by it / scaled by the
+// gate suffix (qs, kt, kh ... above).  With own channel c, other channel e:
+//   P[t,s]  = AOS_t . VOT_s                                         (contraction over e)
+//   o'_t[c] = sum_e S0[c,e] AOS_t[e] + sum_{s<t} P[t,s] VT_s[c]
+//   v'_t[c] = sum_e (L_own[c] Gb[c,e]) VOH_t[e] + sum_{r>t} P[r,t] AS_r[c]
+//   d_own_gate_t = RG_t * (carry + sum_{r>=t} o'_r AS_r - v'_r VT_r)
+//   d_V_t = IP_t * (v'_t + AS_t P[t,t])        d_A_t = PP_t * (o'_t + VT_t P[t,t])   (side 1 only)
+//   Gb <- L_own[c] L_other[e] Gb[c,e] + sum_t AS_t[c] AOS_t[e]
+//
+// A workgroup has 12 waves.  Matrix wave w (of 4) holds, in fp32 accumulators, the slab of S and
+// of Gb for own channels 16w..16w+15 (all other channels), so that every contraction is local to
+// a wave.  Chunks are visited last to first; inside a chunk a forward sweep ("R" stages, two
+// blocks per stage) recomputes the block-start states from the checkpoint and keeps them as
+// 16-bit MFMA operands in registers, then the blocks are visited last to first ("B" stages).
+// Eight prep waves (B stages: 4 roles x 2 token halves; R stages: 2 blocks x 2 sides x 2 token
+// halves) build the operand tiles of the next stage in double-buffered LDS; one barrier per
+// stage.  Raw inputs go from global memory straight to the prep waves' registers two stages
+// ahead, and the matrix waves store the gradients themselves.
 //
 // Replaces lfw_cuda_bwd_kernel and the six einsums of the reference
 // (t2fw/csrc/lfw_kernel.cu:61-102, t2fw/csrc/lfw.cpp:84-93).
+#include <type_traits>
+
 #include "lfw_chunk_bwd_dev.hpp"
 
 namespace t2fw {
@@ -33,519 +51,673 @@ namespace {
 
 using namespace bwd;
 
-constexpr int BWD_THREADS = 512;
+constexpr int SP_THREADS = 768;
 constexpr int CC = 20;   // channel-major 16-token tiles: row stride in elements
 
 // ---- LDS layout of one stage buffer (bytes) ----------------------------------------------
-constexpr int TM_TILE = CH_L * TS * 2;       // token-major 16-bit tile [16][TS]
+constexpr int TM_TILE = CH_L * TS * 2;       // token-major 16-bit tile [16][TS], channels permuted (tm_pos)
 constexpr int CM_TILE = CH_N * CC * 2;       // channel-major 16-bit tile [64][CC]
 constexpr int CF_TILE = CH_N * CC * 4;       // channel-major fp32 tile [64][CC]
-enum { T_QT = 0, T_KT, T_GT, T_XT, T_KH, T_XH, T_NUM };   // same order in both layouts
+enum { TM_AOS = 0, TM_VOT, TM_VOH, TM_NUM };
+// B stages use the named tiles; an R stage covers two blocks j = 0, 1 and uses tiles 2j (VOH) and 2j+1 (VH)
+enum { CM_AOS = 0, CM_VOH, CM_AS, CM_VT, CM_VH, CM_NUM };
+enum { F_RG = 0, F_IP, F_PP, F_NUM };        // 1/own gate, 1/own prefix, own prefix
 constexpr int OFF_TM = 0;
-constexpr int OFF_CM = OFF_TM + T_NUM * TM_TILE;
-enum { F_BT = 0, F_RFK, F_IA, F_RF, F_NUM };              // b_t, 1/fk_t, 1/a_t, 1/f_t
-constexpr int OFF_CF = OFF_CM + T_NUM * CM_TILE;
-constexpr int OFF_BLV = OFF_CF + F_NUM * CF_TILE;          // b_L [64] f32
-constexpr int OFF_ALV = OFF_BLV + CH_N * 4;                // a_L [64] f32
-constexpr int STAGE_BYTES = OFF_ALV + CH_N * 4;
-constexpr int BOUT_TILE = CH_L * OS * 2;                   // one gradient tile [16][OS] u16
-enum { O_DX = 0, O_DF, O_DQ, O_DK, O_DFK, O_NUM };
-constexpr int BOUT_BYTES = O_NUM * BOUT_TILE;
-constexpr int BRAW_ARRAY = CH_L * CH_N * 2;                // [16][64] u16
-enum { R_FK = 0, R_K, R_F, R_X, R_Q, R_G, R_NUM };         // R stages need the first four only
-constexpr int BRAW_BYTES = R_NUM * BRAW_ARRAY;
-constexpr int BOFF_OUT = 2 * STAGE_BYTES;
-constexpr int BOFF_RAW = BOFF_OUT + 2 * BOUT_BYTES;
-constexpr int BWD_SMEM = BOFF_RAW + 2 * BRAW_BYTES;
-static_assert(BWD_SMEM <= 160 * 1024, "backward stage buffers exceed the LDS of one CU");
+constexpr int OFF_CM = OFF_TM + TM_NUM * TM_TILE;
+constexpr int OFF_CF = OFF_CM + CM_NUM * CM_TILE;
+// 16-step gate products, [block j of an R stage][other side, own side][64] f32 (B stages: j = 0)
+constexpr int OFF_LV = OFF_CF + F_NUM * CF_TILE;
+constexpr int STAGE_BYTES = OFF_LV + 4 * CH_N * 4;
+constexpr int SP_SMEM = 2 * STAGE_BYTES;
+static_assert(SP_SMEM <= 160 * 1024, "backward stage buffers exceed the LDS of one CU");
+static_assert(STAGE_BYTES % 16 == 0, "stage buffers must keep 16-byte alignment");
 
-// ---- raw staging -------------------------------------------------------------------------
-// A stage's raw inputs are R_NUM arrays of [16 tokens][64 channels]: 768 pieces of 16 bytes,
-// three per prep thread.  Everything that does not depend on the stage is worked out once per
-// thread (PieceMap), so that issuing a stage's loads costs a handful of instructions.
-struct BStage {
-    uint4 v[3];
+__device__ __forceinline__ float *lv_vec(unsigned char *stage, int j, int own) {
+    return reinterpret_cast<float *>(stage + OFF_LV) + (2 * j + own) * CH_N;
+}
+__device__ __forceinline__ const float *lv_vec(const unsigned char *stage, int j, int own) {
+    return reinterpret_cast<const float *>(stage + OFF_LV) + (2 * j + own) * CH_N;
+}
+
+// ---- stage schedule ----------------------------------------------------------------------
+// Chunks are visited from the last one down; a chunk with nb blocks takes ceil(nb/2) "R"
+// stages of two blocks each (forward in time), then nb "B" stages (blocks nb-1..0).
+// A stage is one int: (first token of its first block) * 2 + (1 for a B stage).
+template <int NB> struct SplitSchedule {
+    static constexpr unsigned PER_CHUNK = NB / 2 + NB;
+    int NC, C, total, nb_last, st_last;
+    __device__ SplitSchedule(int64_t T, int64_t NC_, int C_) {
+        NC = (int)NC_;
+        C = C_;
+        const int len_last = (int)(T - (NC_ - 1) * C_);
+        nb_last = (len_last + CH_L - 1) / CH_L;
+        st_last = (nb_last + 1) / 2 + nb_last;
+        total = st_last + (NC - 1) * (int)PER_CHUNK;
+    }
+    __device__ int at(int s) const {
+        int chunk, local, nb;
+        if (s < st_last) {
+            chunk = NC - 1;
+            local = s;
+            nb = nb_last;
+        } else {
+            const unsigned s2 = (unsigned)(s - st_last);
+            chunk = NC - 2 - (int)(s2 / PER_CHUNK);
+            local = (int)(s2 % PER_CHUNK);
+            nb = NB;
+        }
+        const int nr = (nb + 1) / 2;
+        const bool bmode = local >= nr;
+        const int block = bmode ? nb - 1 - (local - nr) : 2 * local;
+        return ((chunk * C + block * CH_L) << 1) | (bmode ? 1 : 0);
+    }
 };
 
-struct PieceMap {
-    const u16 *ld[3];     // source of raw piece m at token offset 0 of this batch row
-    u16 *st[3];           // destination of gradient piece m at token offset 0 (null: no such piece)
-    int arr[3];           // raw array index of piece m
-    int tok[3];           // token inside the block
-    u32 fill[3];          // identity fill for steps past the end of the sequence
-    int out_off[3];       // byte offset of gradient piece m inside one OUT buffer
+// The same schedule as a forward iterator: cur() is SplitSchedule::at of the stage it stands on;
+// advancing past the last stage leaves it there.  The stages of a chunk are one byte each in a
+// 64-bit table, (block << 1) | (1 for a B stage), so that a step costs a few scalar instructions.
+template <int NB> struct StageIter {
+    static __host__ __device__ constexpr uint64_t table_of(int nb) {
+        uint64_t t = 0;
+        const int nr = (nb + 1) / 2;
+        for (int l = 0; l < nr + nb; ++l) {
+            const uint64_t e = l < nr ? (uint64_t)(2 * l) << 1 : ((uint64_t)(nb - 1 - (l - nr)) << 1) | 1u;
+            t |= e << (8 * l);
+        }
+        return t;
+    }
+    uint64_t table;     // of the chunk it stands in
+    int base2;          // (first token of that chunk) * 2
+    int local, count;   // stage inside the chunk, stages of the chunk
+    int C2, left;       // 2 * C; stages after the current one
+    __device__ StageIter(const SplitSchedule<NB> &sc)
+        : base2((sc.NC - 1) * sc.C * 2), local(0), count(sc.st_last), C2(2 * sc.C), left(sc.total - 1) {
+        table = sc.nb_last == 1 ? table_of(1) : sc.nb_last == 2 ? table_of(2) : sc.nb_last == 3 ? table_of(3) : table_of(4);
+    }
+    __device__ void advance() {
+        if (left > 0) {
+            --left;
+            ++local;
+            if (local == count) {
+                base2 -= C2;
+                local = 0;
+                count = (int)SplitSchedule<NB>::PER_CHUNK;
+                table = table_of(NB);
+            }
+        }
+    }
+    __device__ int cur() const {
+        const int e = (int)(table >> (8 * local)) & 0xff;       // (block << 1) | bmode
+        return base2 + (e >> 1) * (2 * CH_L) + (e & 1);
+    }
+};
+static_assert(SplitSchedule<4>::PER_CHUNK <= 8, "a chunk's stages must fit the 64-bit table");
+
+// ---- raw inputs --------------------------------------------------------------------------
+// A prep thread works on one channel and eight tokens; it needs the gate at those tokens, the
+// gate at the block's other eight tokens and one value (or adjoint) array at its own tokens:
+// 24 two-byte loads, coalesced over the wave's 64 channels.  They go straight to registers,
+// two stages ahead of their use: the block's first token of an array is a scalar base, the
+// lane's channel and token half a constant vector offset, the token inside the half an
+// immediate one.
+struct RawSet {
+    u16 gown[8], goth[8], val[8];
 };
 
-__device__ __forceinline__ void bstage_load(BStage &st, const PieceMap &pm, int64_t T, int64_t t0, bool bmode) {
-    const int narr = bmode ? R_NUM : 4;
+// gate, val: wave-uniform addresses of the block's first token; voff_own / voff_oth: byte offsets of
+// (own / other token half, channel) inside a block
+__device__ __forceinline__ void raw_issue(RawSet &r, const u16 *gate, const u16 *val, u32 voff_own, u32 voff_oth) {
+    auto at = [&](const u16 *base, u32 voff, int t) -> u16 {
+        return *reinterpret_cast<const u16 *>(reinterpret_cast<const unsigned char *>(base + t * CH_N) + voff);
+    };
 #pragma unroll
-    for (int m = 0; m < 3; ++m) {
-        if (pm.arr[m] < narr) {
-            if (t0 + pm.tok[m] < T)
-                st.v[m] = *reinterpret_cast<const uint4 *>(pm.ld[m] + t0 * CH_N);
-            else
-                st.v[m] = make_uint4(pm.fill[m], pm.fill[m], pm.fill[m], pm.fill[m]);
+    for (int t = 0; t < 8; ++t) r.goth[t] = at(gate, voff_oth, t);
+#pragma unroll
+    for (int t = 0; t < 8; ++t) r.gown[t] = at(gate, voff_own, t);
+#pragma unroll
+    for (int t = 0; t < 8; ++t) r.val[t] = at(val, voff_own, t);
+}
+
+// The same for a block that reaches past the end of the sequence (T % 16 != 0, last chunk only):
+// tokens past the end are read from the last one, with the same number of loads, and replaced by
+// raw_patch_tail when the set is taken.  row_gate, row_val: token 0 of the batch row.
+__device__ __forceinline__ void raw_issue_tail(RawSet &r, const u16 *row_gate, const u16 *row_val, int tok_own,
+                                               int tok_oth, int T, int c) {
+    auto at = [&](const u16 *base, int tok) -> u16 { return base[(u32)min(tok, T - 1) * CH_N + c]; };
+#pragma unroll
+    for (int t = 0; t < 8; ++t) r.goth[t] = at(row_gate, tok_oth + t);
+#pragma unroll
+    for (int t = 0; t < 8; ++t) r.gown[t] = at(row_gate, tok_own + t);
+#pragma unroll
+    for (int t = 0; t < 8; ++t) r.val[t] = at(row_val, tok_own + t);
+}
+
+// tokens past the end act as identity: gate 1, everything else 0
+template <typename IOE> __device__ __forceinline__ void raw_patch_tail(RawSet &r, int tok_own, int tok_oth, int T) {
+#pragma unroll
+    for (int t = 0; t < 8; ++t) {
+        if (tok_oth + t >= T) r.goth[t] = IOE::ONE_BITS;
+        if (tok_own + t >= T) {
+            r.gown[t] = IOE::ONE_BITS;
+            r.val[t] = 0;
         }
     }
 }
 
-__device__ __forceinline__ void bstage_store(const BStage &st, const PieceMap &pm, unsigned char *raw, bool bmode,
-                                             int tid) {
-    const int narr = bmode ? R_NUM : 4;
+template <typename IOE> __device__ __forceinline__ u32 gate_check8(const u16 (&g)[8]) {
+    u16 mx = 0;
 #pragma unroll
-    for (int m = 0; m < 3; ++m)
-        if (pm.arr[m] < narr) *reinterpret_cast<uint4 *>(raw + (tid + 256 * m) * 16) = st.v[m];
+    for (int t = 0; t < 8; ++t) {
+        const u16 m1 = (u16)(g[t] - 1);      // gates must lie in (0, 1]: 0 < bits <= bits(1.0)
+        mx = m1 > mx ? m1 : mx;
+    }
+    return (mx >= IOE::ONE_BITS) ? 1u : 0u;
 }
 
-// column of one raw array for channel c
-__device__ __forceinline__ void raw_col(u16 (&dst)[CH_L], const unsigned char *raw, int array, int c) {
-    const u16 *base = reinterpret_cast<const u16 *>(raw + array * BRAW_ARRAY) + c;
+// eight tokens of one channel as four packed pairs
+struct Packed8 {
+    u32 p[4];
+};
+template <typename OPE> __device__ __forceinline__ Packed8 pack8(const float (&v)[8]) {
+    Packed8 r;
 #pragma unroll
-    for (int t = 0; t < CH_L; ++t) dst[t] = base[t * CH_N];
+    for (int i = 0; i < 4; ++i) r.p[i] = OPE::pack2(v[2 * i], v[2 * i + 1]);
+    return r;
 }
 
-template <typename OPE>
-__device__ __forceinline__ void write_tm(unsigned char *stage, int tile, int c, const float (&v)[CH_L]) {
-    u16 *tm = reinterpret_cast<u16 *>(stage + OFF_TM + tile * TM_TILE);
+__device__ __forceinline__ void write_tm8(unsigned char *stage, int tile, int c, int t0, const Packed8 &v) {
+    u16 *tm = reinterpret_cast<u16 *>(stage + OFF_TM + tile * TM_TILE) + t0 * TS + tm_pos(c);
 #pragma unroll
-    for (int t = 0; t < CH_L; ++t) tm[t * TS + c] = cvt1<OPE>(v[t]);
+    for (int i = 0; i < 4; ++i) {
+        tm[(2 * i) * TS] = (u16)(v.p[i] & 0xffffu);
+        tm[(2 * i + 1) * TS] = (u16)(v.p[i] >> 16);
+    }
 }
 
-template <typename OPE>
-__device__ __forceinline__ void write_cm(unsigned char *stage, int tile, int c, const float (&v)[CH_L]) {
-    uint2 *cm = reinterpret_cast<uint2 *>(stage + OFF_CM + tile * CM_TILE + c * CC * 2);
-#pragma unroll
-    for (int t = 0; t < CH_L; t += 4) cm[t / 4] = packq<OPE>(v[t], v[t + 1], v[t + 2], v[t + 3]);
+__device__ __forceinline__ void write_cm8(unsigned char *stage, int tile, int c, int t0, const Packed8 &v) {
+    uint2 *cm = reinterpret_cast<uint2 *>(stage + OFF_CM + tile * CM_TILE + (c * CC + t0) * 2);
+    cm[0] = make_uint2(v.p[0], v.p[1]);
+    cm[1] = make_uint2(v.p[2], v.p[3]);
 }
 
-__device__ __forceinline__ void write_cf(unsigned char *stage, int tile, int c, const float (&v)[CH_L]) {
-    float4 *cf = reinterpret_cast<float4 *>(stage + OFF_CF + tile * CF_TILE + c * CC * 4);
-#pragma unroll
-    for (int t = 0; t < CH_L; t += 4) cf[t / 4] = make_float4(v[t], v[t + 1], v[t + 2], v[t + 3]);
+__device__ __forceinline__ void write_cf8(unsigned char *stage, int tile, int c, int t0, const float (&v)[8]) {
+    float4 *cf = reinterpret_cast<float4 *>(stage + OFF_CF + tile * CF_TILE + (c * CC + t0) * 4);
+    cf[0] = make_float4(v[0], v[1], v[2], v[3]);
+    cf[1] = make_float4(v[4], v[5], v[6], v[7]);
 }
 
-// One prep wave, one role (role = prep wave index 0..3), channel c:
-//   role 0: key gate prefix -> qs tiles, b_t, 1/fk_t            role 1: key gate suffix -> kh, kt tiles, b_L
-//   role 2: value gate prefix -> gs tiles, 1/f_t                role 3: value gate suffix -> xh, xt tiles, 1/a_t, a_L
-// In R stages only roles 1 and 3 work and only the channel-major kh / xh tiles and a_L, b_L are made.
+template <typename IOE> __device__ __forceinline__ float product8(const u16 (&g)[8]) {
+    float p = IOE::mul2(g[0], g[1]);
+#pragma unroll
+    for (int t = 2; t < 8; ++t) p = IOE::mul(g[t], p);
+    return p;
+}
+
+// Gate-suffix scalings of one half block: hat = v * prod_{r>t} gate_r, til = hat / total,
+// inv = 1 / prod_{r<=t} gate_r; returns the 16-step product.
 template <typename IOE, typename OPE>
-__device__ __forceinline__ void bwd_prep(const unsigned char *raw, unsigned char *stage, int role, int c, bool bmode,
-                                         u32 &bad) {
-    const bool kside = role < 2;
-    const bool prefix_role = (role & 1) == 0;
-    if (!bmode && prefix_role) return;
-    u16 gr[CH_L], ar[CH_L];
-    raw_col(gr, raw, kside ? R_FK : R_F, c);
-    raw_col(ar, raw, prefix_role ? (kside ? R_Q : R_G) : (kside ? R_K : R_X), c);
-    float gate[CH_L];
+__device__ __forceinline__ float suffix_scale(const RawSet &r, int h, bool check, float (&hat)[8], float (&til)[8],
+                                              float (&inv)[8], u32 &bad) {
+    const float poth = product8<IOE>(r.goth);
+    const float tot = product8<IOE>(r.gown) * poth;
+    if (check) bad |= gate_check8<IOE>(r.gown);
+    bad |= (tot >= OPE::MIN_PRODUCT) ? 0u : 1u;
+    const float itot = __builtin_amdgcn_rcpf(tot);
+    float sfx = h ? 1.0f : poth;
 #pragma unroll
-    for (int t = 0; t < CH_L; ++t) gate[t] = IOE::to_f32(gr[t]);
-    if (prefix_role) {
-        float pre[CH_L], v[CH_L], rg[CH_L];
-        pre[0] = gate[0];
+    for (int t = 7; t >= 0; --t) {
+        inv[t] = sfx * itot;
+        hat[t] = IOE::mul(r.val[t], sfx);
+        til[t] = hat[t] * itot;
+        sfx = IOE::mul(r.gown[t], sfx);
+    }
+    return tot;
+}
+
+// B stage, one prep wave: one role, tokens 8h..8h+7 of the block, channel c.
+//   role 0: other gate prefix -> AOS (token- and channel-major)
+//   role 1: other gate suffix -> VOH (both layouts), VOT (token-major), L_other
+//   role 2: own gate prefix   -> AS, 1/gate, prefix (side 1)
+//   role 3: own gate suffix   -> VH, VT, 1/prefix, L_own
+template <typename IOE, typename OPE>
+__device__ __forceinline__ void prep_b(const RawSet &r, unsigned char *stage, int role, int h, int c, bool want_pp,
+                                       u32 &bad) {
+    const bool other = role < 2;
+    const int t0 = 8 * h;
+    if ((role & 1) == 0) {
+        const float base = h ? product8<IOE>(r.goth) : 1.0f;
+        float run = base;
+        float pre[8], v[8];
 #pragma unroll
-        for (int t = 1; t < CH_L; ++t) pre[t] = pre[t - 1] * gate[t];
-#pragma unroll
-        for (int t = 0; t < CH_L; ++t) {
-            v[t] = IOE::to_f32(ar[t]) * pre[t];            // qs or gs
-            rg[t] = __builtin_amdgcn_rcpf(gate[t]);        // 1/fk_t or 1/f_t
+        for (int t = 0; t < 8; ++t) {
+            run = IOE::mul(r.gown[t], run);
+            pre[t] = run;
+            v[t] = IOE::mul(r.val[t], run);
         }
-        write_tm<OPE>(stage, kside ? T_QT : T_GT, c, v);
-        write_cm<OPE>(stage, kside ? T_QT : T_GT, c, v);
-        write_cf(stage, kside ? F_RFK : F_RF, c, rg);
-        if (kside) write_cf(stage, F_BT, c, pre);
+        const Packed8 vp = pack8<OPE>(v);
+        if (other) {
+            write_tm8(stage, TM_AOS, c, t0, vp);
+            write_cm8(stage, CM_AOS, c, t0, vp);
+        } else {
+            // 1/gate_t = prefix_{t-1} / prefix_t from one reciprocal and the running products
+            float ipre = __builtin_amdgcn_rcpf(pre[7]);
+            float rg[8];
+#pragma unroll
+            for (int t = 7; t >= 1; --t) {
+                rg[t] = pre[t - 1] * ipre;
+                ipre = IOE::mul(r.gown[t], ipre);
+            }
+            rg[0] = base * ipre;
+            write_cm8(stage, CM_AS, c, t0, vp);
+            write_cf8(stage, F_RG, c, t0, rg);
+            if (want_pp) write_cf8(stage, F_PP, c, t0, pre);
+        }
     } else {
-        bad |= gate_check<IOE>(gr);
-        float tot = gate[0];
-#pragma unroll
-        for (int t = 1; t < CH_L; ++t) tot *= gate[t];
-        bad |= (tot >= OPE::MIN_PRODUCT) ? 0u : 1u;
-        const float itot = __builtin_amdgcn_rcpf(tot);
-        float hat[CH_L], til[CH_L], inv[CH_L];
-        float sfx = 1.0f;
-#pragma unroll
-        for (int t = CH_L - 1; t >= 0; --t) {
-            inv[t] = sfx * itot;                            // 1 / prefix_t
-            hat[t] = IOE::to_f32(ar[t]) * sfx;              // kh or xh
-            til[t] = hat[t] * itot;                         // kt or xt
-            sfx *= gate[t];
-        }
-        write_cm<OPE>(stage, kside ? T_KH : T_XH, c, hat);
-        reinterpret_cast<float *>(stage + (kside ? OFF_BLV : OFF_ALV))[c] = tot;
-        if (bmode) {
-            write_tm<OPE>(stage, kside ? T_KH : T_XH, c, hat);
-            write_tm<OPE>(stage, kside ? T_KT : T_XT, c, til);
-            write_cm<OPE>(stage, kside ? T_KT : T_XT, c, til);
-            if (!kside) write_cf(stage, F_IA, c, inv);
+        float hat[8], til[8], inv[8];
+        const float tot = suffix_scale<IOE, OPE>(r, h, true, hat, til, inv, bad);
+        if (h == 0) lv_vec(stage, 0, other ? 0 : 1)[c] = tot;
+        const Packed8 hp = pack8<OPE>(hat), tp = pack8<OPE>(til);
+        if (other) {
+            write_cm8(stage, CM_VOH, c, t0, hp);
+            write_tm8(stage, TM_VOH, c, t0, hp);
+            write_tm8(stage, TM_VOT, c, t0, tp);
+        } else {
+            write_cm8(stage, CM_VH, c, t0, hp);
+            write_cm8(stage, CM_VT, c, t0, tp);
+            write_cf8(stage, F_IP, c, t0, inv);
         }
     }
+}
+
+// R stage, one prep wave: block j of the pair, own or other side, tokens 8h..8h+7, channel c:
+// the suffix-scaled values (channel-major) and the 16-step gate product.  (Every block's gates
+// are range-checked in its B stage.)
+template <typename IOE, typename OPE>
+__device__ __forceinline__ void prep_r(const RawSet &r, unsigned char *stage, int j, int own, int h, int c, u32 &bad) {
+    float hat[8], til[8], inv[8];
+    const float tot = suffix_scale<IOE, OPE>(r, h, false, hat, til, inv, bad);
+    if (h == 0) lv_vec(stage, j, own)[c] = tot;
+    write_cm8(stage, 2 * j + own, c, 8 * h, pack8<OPE>(hat));
 }
 
 template <typename IOE, typename OPE, int NB>
-__device__ __forceinline__ void bwd_prep_waves(const ChunkBwdArgs &p, unsigned char *smem, int tid, int64_t b) {
-    const int role = tid >> 6, c = tid & 63;
-    const int64_t T = p.T;
-    const int64_t row_base = b * T;
-    const u16 *const src[R_NUM] = {reinterpret_cast<const u16 *>(p.f_key), reinterpret_cast<const u16 *>(p.k),
-                                   reinterpret_cast<const u16 *>(p.f),     reinterpret_cast<const u16 *>(p.x),
-                                   reinterpret_cast<const u16 *>(p.q),     reinterpret_cast<const u16 *>(p.g_out)};
-    u16 *const dst[O_NUM] = {reinterpret_cast<u16 *>(p.d_x), reinterpret_cast<u16 *>(p.d_f),
-                             reinterpret_cast<u16 *>(p.d_q), reinterpret_cast<u16 *>(p.d_k),
-                             reinterpret_cast<u16 *>(p.d_f_key)};
-    const Schedule<NB> sched(T, p.NC, p.C);
-    const int total = sched.total;
+__device__ __forceinline__ void split_prep_waves(const ChunkBwdArgs &p, unsigned char *smem, int tid, int64_t b,
+                                                 int side) {
+    const int pw = __builtin_amdgcn_readfirstlane(tid >> 6), c = tid & 63;
+    // B stages: SIMD-balanced assignment of (role, token half); roles 1 and 3 are the heavier ones
+    const int h = pw >> 2;
+    const int role = (h ? (pw ^ 1) : pw) & 3;
+    // R stages: (block of the pair, side, token half)
+    const int rj = (pw >> 1) & 1, rown = pw & 1;
+    const int T = (int)p.T;                              // the launcher admits T < 2^24 only
+    const int64_t row_off = b * p.T * CH_N;
+    // this batch row of: other gate, other value, own gate, own value, other adjoint, own adjoint
+    const u16 *const x = reinterpret_cast<const u16 *>(p.x) + row_off, *const f = reinterpret_cast<const u16 *>(p.f) + row_off;
+    const u16 *const g = reinterpret_cast<const u16 *>(p.g_out) + row_off, *const k = reinterpret_cast<const u16 *>(p.k) + row_off;
+    const u16 *const fk = reinterpret_cast<const u16 *>(p.f_key) + row_off, *const q = reinterpret_cast<const u16 *>(p.q) + row_off;
+    const u16 *const GO = side == 0 ? fk : f, *const VO = side == 0 ? k : x, *const GW = side == 0 ? f : fk;
+    const u16 *const VW = side == 0 ? x : k, *const AO = side == 0 ? q : g, *const AW = side == 0 ? g : q;
+    // the two arrays this wave reads in B stages and in R stages
+    const u16 *const b_gate = role < 2 ? GO : GW;
+    const u16 *const b_val = role == 0 ? AO : role == 1 ? VO : role == 2 ? AW : VW;
+    const u16 *const r_gate = rown ? GW : GO;
+    const u16 *const r_val = rown ? VW : VO;
+    const SplitSchedule<NB> sched(p.T, p.NC, p.C);
     u32 bad = 0;
-    if (tid == 0) {      // both flag slots of the row (the backward kernels report in the first)
-        p.row_flags[b] = 0;
-        p.row_flags[chunk_rows_padded(p.B) + b] = 0;
-    }
-    auto tok0_of = [&](const StageInfo &si) -> int64_t { return (int64_t)si.chunk * p.C + si.block * CH_L; };
 
-    PieceMap pm;
-#pragma unroll
-    for (int m = 0; m < 3; ++m) {
-        const int pi = tid + 256 * m;              // [array or gradient][token][8 pieces]
-        const int a = pi >> 7, tok = (pi >> 3) & 15, piece = pi & 7;
-        const int64_t off = (row_base + tok) * CH_N + 8 * piece;
-        pm.arr[m] = a;
-        pm.tok[m] = tok;
-        pm.ld[m] = src[a] + off;                   // a <= 5 for every piece
-        pm.fill[m] = (a == R_FK || a == R_F) ? (u32)IOE::ONE_BITS * 0x10001u : 0u;
-        pm.st[m] = a < O_NUM ? dst[a] + off : nullptr;
-        pm.out_off[m] = a * BOUT_TILE + (tok * OS + 8 * piece) * 2;
-    }
-
-    // raw inputs of stage m live in RAW[m & 1]; stA / stB carry the even / odd stages two ahead
-    BStage stA, stB;
-    {
-        const StageInfo s0 = sched.at(0);
-        bstage_load(stA, pm, T, tok0_of(s0), s0.bmode);
-        bstage_store(stA, pm, smem + BOFF_RAW, s0.bmode, tid);
-        if (total > 1) {
-            const StageInfo s1 = sched.at(1);
-            bstage_load(stB, pm, T, tok0_of(s1), s1.bmode);
-            bstage_store(stB, pm, smem + BOFF_RAW + BRAW_BYTES, s1.bmode, tid);
-        }
-        if (total > 2) {
-            const StageInfo s2 = sched.at(2);
-            bstage_load(stA, pm, T, tok0_of(s2), s2.bmode);
-        }
-        if (total > 3) {
-            const StageInfo s3 = sched.at(3);
-            bstage_load(stB, pm, T, tok0_of(s3), s3.bmode);
-        }
-        __syncthreads();
-        bwd_prep<IOE, OPE>(smem + BOFF_RAW, smem, role, c, s0.bmode, bad);
-        __syncthreads();
-    }
-
-    auto store_out = [&](int s) {       // gradients of B stage s: LDS tiles -> global, 16 B pieces
-        const StageInfo si = sched.at(s);
-        if (!si.bmode) return;
-        const unsigned char *outp = smem + BOFF_OUT + (s & 1) * BOUT_BYTES;
-        const int64_t t0 = tok0_of(si);
-#pragma unroll
-        for (int m = 0; m < 3; ++m) {
-            if (pm.st[m] != nullptr && t0 + pm.tok[m] < T) {
-                const u16 *tile = reinterpret_cast<const u16 *>(outp + pm.out_off[m]);
-                const uint2 lo = *reinterpret_cast<const uint2 *>(tile);
-                const uint2 hi = *reinterpret_cast<const uint2 *>(tile + 4);
-                *reinterpret_cast<uint4 *>(pm.st[m] + t0 * CH_N) = make_uint4(lo.x, lo.y, hi.x, hi.y);
-            }
-        }
+    const u32 voff_own = (u32)(8 * h * CH_N + c) * 2u, voff_oth = (u32)(8 * (1 - h) * CH_N + c) * 2u;
+    // first token of the block this wave works on in stage st (R stages cover a pair of blocks)
+    auto block_tok = [&](int st) -> int { return (st >> 1) + ((st & 1) ? 0 : rj * CH_L); };
+    auto issue = [&](RawSet &r, int st) {          // raw inputs of stage st (wave-uniform) -> registers
+        const bool bmode = st & 1;
+        const int tok = block_tok(st);
+        const u16 *const gate = bmode ? b_gate : r_gate, *const val = bmode ? b_val : r_val;
+        if (tok + CH_L <= T)
+            raw_issue(r, gate + (u32)tok * CH_N, val + (u32)tok * CH_N, voff_own, voff_oth);
+        else        // the block reaches past the end (or, second block of the last R pair, lies past it)
+            raw_issue_tail(r, gate, val, tok + 8 * h, tok + 8 * (1 - h), T, c);
     };
-
-    PHASE_BEGIN();
-    auto iteration = [&](int s, BStage &st) {       // st holds stage s+2, then takes stage s+4
-        PHASE_SELECT(sched.at(s).bmode ? 0 : 4);
-        if (s + 2 < total) bstage_store(st, pm, smem + BOFF_RAW + (s & 1) * BRAW_BYTES, sched.at(s + 2).bmode, tid);
-        PHASE_MARK(1);
-        if (s > 0) store_out(s - 1);
-        if (s + 4 < total) {
-            const StageInfo s4 = sched.at(s + 4);
-            bstage_load(st, pm, T, tok0_of(s4), s4.bmode);
-        }
-        PHASE_MARK(0);
-        if (s + 1 < total)
-            bwd_prep<IOE, OPE>(smem + BOFF_RAW + ((s + 1) & 1) * BRAW_BYTES, smem + ((s + 1) & 1) * STAGE_BYTES, role, c,
-                               sched.at(s + 1).bmode, bad);
+    // Three register sets rotate: the tiles of stage s are built from `cur`, which was loaded two
+    // stages ago, while `refill` (used up in the stage before) takes the raw inputs of stage s + 2.
+    // The loads are unconditional (past the end: the last stage again), so that the number of loads
+    // in flight is the same on every path and the waits for them can be exact.
+    StageIter<NB> it_load(sched);
+    int st_cur = 0, st_next = 0;                   // descriptors of stages s and s + 1
+    auto prepare = [&](const RawSet &cur, RawSet &refill, int s) {
+        const int st = st_cur;
+        it_load.advance();
+        const int st_new = it_load.cur();
+        issue(refill, st_new);
+        st_cur = st_next;
+        st_next = st_new;
+        // the loads complete in order: one wait for the last of `cur` covers the whole set
+        asm volatile("" ::"v"(cur.val[7]));
+        RawSet raw = cur;
+        const int tok = block_tok(st);
+        if (tok + CH_L > T) raw_patch_tail<IOE>(raw, tok + 8 * h, tok + 8 * (1 - h), T);
+        unsigned char *stage = smem + (s & 1) * STAGE_BYTES;
+        if (st & 1)
+            prep_b<IOE, OPE>(raw, stage, role, h, c, side == 1, bad);
+        else
+            prep_r<IOE, OPE>(raw, stage, rj, rown, h, c, bad);
         PHASE_MARK(2);
         __syncthreads();
         PHASE_MARK(3);
     };
-    for (int s = 0; s < total; s += 2) {
-        iteration(s, stA);
-        if (s + 1 < total) iteration(s + 1, stB);
+
+    // Stages are done in triples (sets A, B, C in turn) with no exit inside a triple, so that the
+    // order of the loads in flight is the same on every path.  First the stages of the last chunk of
+    // the sequence (it may be short), with the general iterator; its first (count % 3) stages are
+    // peeled off, with the sets assigned so that the triples start on A.
+    RawSet setA, setB, setC;
+    int s = 0;
+    PHASE_BEGIN();
+    const int n_last = sched.st_last;
+    const int rem = n_last % 3;
+    st_cur = it_load.cur();
+    it_load.advance();
+    st_next = it_load.cur();
+    if (rem == 0) {
+        issue(setA, st_cur);
+        issue(setB, st_next);
+    } else if (rem == 1) {
+        issue(setC, st_cur);
+        issue(setA, st_next);
+        prepare(setC, setB, 0);
+        s = 1;
+    } else {
+        issue(setB, st_cur);
+        issue(setC, st_next);
+        prepare(setB, setA, 0);
+        prepare(setC, setB, 1);
+        s = 2;
     }
-    store_out(total - 1);
+    for (; s < n_last; s += 3) {
+        prepare(setA, setC, s);
+        prepare(setB, setA, s + 1);
+        prepare(setC, setB, s + 2);
+    }
+
+    // Then the full chunks, last to first.  Inside a chunk the kind of every stage and its block are
+    // compile-time constants (position POS of PER), which leaves a pointer bump per stage for the
+    // scalar unit; PER is a multiple of three, so every chunk starts on set A.  The refill of
+    // position POS + 2 reaches into the chunk below for the last two positions (below the first
+    // chunk: that chunk again, never used).
+    constexpr int PER = (int)SplitSchedule<NB>::PER_CHUNK, NR = NB / 2;
+    static_assert(PER % 3 == 0, "a chunk must take a whole number of register-set triples");
+    const u16 *const r_gate_w = r_gate + rj * CH_L * CH_N, *const r_val_w = r_val + rj * CH_L * CH_N;
+    auto issue_at = [&](RawSet &r, int chunk_tok, auto pos_c) {
+        constexpr int POS = decltype(pos_c)::value;
+        if constexpr (POS < NR) {
+            const u32 e = (u32)(chunk_tok + 2 * POS * CH_L) * CH_N;
+            raw_issue(r, r_gate_w + e, r_val_w + e, voff_own, voff_oth);
+        } else {
+            const u32 e = (u32)(chunk_tok + (NB - 1 - (POS - NR)) * CH_L) * CH_N;
+            raw_issue(r, b_gate + e, b_val + e, voff_own, voff_oth);
+        }
+    };
+    auto prepare_at = [&](const RawSet &cur, RawSet &refill, int chunk_tok, int below_tok, auto pos_c) {
+        constexpr int POS = decltype(pos_c)::value;
+        if constexpr (POS + 2 < PER)
+            issue_at(refill, chunk_tok, std::integral_constant<int, (POS + 2) % PER>{});
+        else
+            issue_at(refill, below_tok, std::integral_constant<int, (POS + 2) % PER>{});
+        // the loads complete in order: one wait for the last of `cur` covers the whole set
+        asm volatile("" ::"v"(cur.val[7]));
+        unsigned char *stage = smem + (s & 1) * STAGE_BYTES;
+        if constexpr (POS >= NR)
+            prep_b<IOE, OPE>(cur, stage, role, h, c, side == 1, bad);
+        else
+            prep_r<IOE, OPE>(cur, stage, rj, rown, h, c, bad);
+        ++s;
+        PHASE_MARK(2);
+        __syncthreads();
+        PHASE_MARK(3);
+    };
+    for (int chunk_tok = (sched.NC - 2) * p.C; chunk_tok >= 0; chunk_tok -= p.C) {
+        const int below_tok = max(chunk_tok - p.C, 0);
+        prepare_at(setA, setC, chunk_tok, below_tok, std::integral_constant<int, 0>{});
+        prepare_at(setB, setA, chunk_tok, below_tok, std::integral_constant<int, 1>{});
+        prepare_at(setC, setB, chunk_tok, below_tok, std::integral_constant<int, 2>{});
+        if constexpr (PER == 6) {
+            prepare_at(setA, setC, chunk_tok, below_tok, std::integral_constant<int, 3>{});
+            prepare_at(setB, setA, chunk_tok, below_tok, std::integral_constant<int, 4>{});
+            prepare_at(setC, setB, chunk_tok, below_tok, std::integral_constant<int, 5>{});
+        }
+    }
+    // Both workgroups of a row see all four gates' blocks and reach the same verdict, so either
+    // order of their writes leaves the same flag.
     if (bad) p.row_flags[b] = 1;
     PHASE_END(4 + (tid >> 6));
 }
 
-// helpers of the matrix waves ----------------------------------------------------------------
-__device__ __forceinline__ const u16 *tm_tile(const unsigned char *stage, int tile) {
-    return reinterpret_cast<const u16 *>(stage + OFF_TM + tile * TM_TILE);
-}
-__device__ __forceinline__ const u16 *cm_tile(const unsigned char *stage, int tile) {
-    return reinterpret_cast<const u16 *>(stage + OFF_CM + tile * CM_TILE);
-}
-__device__ __forceinline__ const float *cf_tile(const unsigned char *stage, int tile) {
-    return reinterpret_cast<const float *>(stage + OFF_CF + tile * CF_TILE);
-}
 template <typename IOE, typename OPE, int NB>
-__device__ __forceinline__ void bwd_matrix_waves(const ChunkBwdArgs &p, unsigned char *smem, int tid, int64_t b) {
+__device__ __forceinline__ void split_matrix_waves(const ChunkBwdArgs &p, unsigned char *smem, int tid, int64_t b,
+                                                   int side) {
     const int w = tid >> 6, l = tid & 63, r = l & 15, g = l >> 4;
-    const int ch = 16 * w + r;       // this lane's d in the D copies and its k in the K copies
-    const int64_t T = p.T, NC = p.NC;
+    const int ch = 16 * w + r;       // this lane's own-side channel
+    const int T = (int)p.T;                              // the launcher admits T < 2^24 only
+    const int64_t NC = p.NC;
     const int C = p.C;
     const u16 *ckpt = reinterpret_cast<const u16 *>(p.ckpt) + b * NC * (CH_N * CH_N);
-    const int nb_last = (int)((T - (NC - 1) * C + CH_L - 1) / CH_L);
+    const int nb_last = (int)((p.T - (NC - 1) * C + CH_L - 1) / CH_L);
+    // this batch row of the gradients this side writes
+    u16 *const d_val = reinterpret_cast<u16 *>(side == 0 ? p.d_x : p.d_k) + b * p.T * CH_N;
+    u16 *const d_gate = reinterpret_cast<u16 *>(side == 0 ? p.d_f : p.d_f_key) + b * p.T * CH_N;
+    u16 *const d_adj = reinterpret_cast<u16 *>(p.d_q) + b * p.T * CH_N;
 
-    floatx4 Sd[4], Sk[4], Gd[4], Gk[4];
-    uint2 svd[NB][4], svk[NB][4];     // block-start states as 16-bit MFMA operands
-    uint2 pfd[4];                     // checkpoint prefetch: D copy rows (4 values each)
-    u16 pfk[16];                      //                      K copy column
-    auto ckpt_issue = [&](int64_t chunk) {
-        const u16 *ck = ckpt + chunk * (CH_N * CH_N);
+    // S[j][i], G[j][i]: own channel ch, other channel 16j + 4g + i
+    floatx4 S[4], G[4];
+    uint4 sv[NB][2];                  // block-start states as 16-bit MFMA operands (other channels 0..31, 32..63)
+    uint2 pf[4];                      // checkpoint prefetch, packed I/O type
+    // memory is [d][k]: side 0 reads 4 adjacent k of row d = ch, side 1 gathers column k = ch
+    auto load_state = [&](const u16 *m, uint2 (&dst)[4]) {
+        if (side == 0) {
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            pfd[j] = ld2(ck + ch * CH_N + 16 * j + 4 * g);
+            for (int j = 0; j < 4; ++j) dst[j] = ld2(m + ch * CH_N + 16 * j + 4 * g);
+        } else {
 #pragma unroll
-            for (int i = 0; i < 4; ++i) pfk[4 * j + i] = ck[(16 * j + 4 * g + i) * CH_N + ch];
-        }
-    };
-    auto ckpt_take = [&]() {
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            float t[4];
-            unpack4<IOE>(pfd[j], t);
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                Sd[j][i] = t[i];
-                Sk[j][i] = IOE::to_f32(pfk[4 * j + i]);
+            for (int j = 0; j < 4; ++j) {
+                const u16 *col = m + (16 * j + 4 * g) * CH_N + ch;
+                dst[j] = make_uint2((u32)col[0] | ((u32)col[CH_N] << 16), (u32)col[2 * CH_N] | ((u32)col[3 * CH_N] << 16));
             }
         }
     };
-    {   // incoming state gradient
-        const u16 *gs = reinterpret_cast<const u16 *>(p.g_state) + b * (CH_N * CH_N);
+    auto take_state = [&](const uint2 (&src)[4], floatx4 (&dst)[4]) {
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             float t[4];
-            unpack4<IOE>(ld2(gs + ch * CH_N + 16 * j + 4 * g), t);
+            unpack4<IOE>(src[j], t);
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                Gd[j][i] = t[i];
-                Gk[j][i] = IOE::to_f32(gs[(16 * j + 4 * g + i) * CH_N + ch]);
-            }
+            for (int i = 0; i < 4; ++i) dst[j][i] = t[i];
         }
+    };
+    load_state(reinterpret_cast<const u16 *>(p.g_state) + b * (CH_N * CH_N), pf);
+    take_state(pf, G);
+    load_state(ckpt + (NC - 1) * (CH_N * CH_N), pf);
+    float carry = 0.f;
+    int s = 0;
+    if (tid == 0) {      // both flag slots of the row (the backward kernels report in the first)
+        p.row_flags[b] = 0;
+        p.row_flags[chunk_rows_padded(p.B) + b] = 0;
     }
-    ckpt_issue(NC - 1);
-    float u_carry = 0.f, v_carry = 0.f;
-    int64_t s = 0;
-    __syncthreads();      // raw inputs of the first stages are in LDS
-    __syncthreads();      // operand tiles of stage 0 are in LDS
     PHASE_BEGIN();
 
+    // every stage starts with the workgroup barrier that publishes its operand tiles
     for (int64_t chunk = NC - 1; chunk >= 0; --chunk) {
         const int nb = chunk == NC - 1 ? nb_last : NB;
-        ckpt_take();
-        if (chunk > 0) ckpt_issue(chunk - 1);
-        // ---- R stages: block-start states, forward in time
+        take_state(pf, S);
+        if (chunk > 0) load_state(ckpt + (chunk - 1) * (CH_N * CH_N), pf);
+        // ---- R stages: block-start states, forward in time, two blocks per stage
 #pragma unroll
-        for (int i = 0; i < NB; ++i) {
-            if (i < nb) {
-                const unsigned char *stage = smem + (s & 1) * STAGE_BYTES;
-                const u16 *KHc = cm_tile(stage, T_KH), *XHc = cm_tile(stage, T_XH);
-                const float *BLV = reinterpret_cast<const float *>(stage + OFF_BLV);
-                const float *ALV = reinterpret_cast<const float *>(stage + OFF_ALV);
-#pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    svd[i][j] = pack4v<OPE>(Sd[j]);
-                    svk[i][j] = pack4v<OPE>(Sk[j]);
-                }
-                const float aL = ALV[ch], bL = BLV[ch];
-                const uint2 xh_d = ld2(XHc + ch * CC + 4 * g), kh_k = ld2(KHc + ch * CC + 4 * g);
-#pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    const float4 bl = *reinterpret_cast<const float4 *>(BLV + 16 * j + 4 * g);
-                    const float4 al = *reinterpret_cast<const float4 *>(ALV + 16 * j + 4 * g);
-                    Sd[j][0] *= aL * bl.x; Sd[j][1] *= aL * bl.y; Sd[j][2] *= aL * bl.z; Sd[j][3] *= aL * bl.w;
-                    Sk[j][0] *= al.x * bL; Sk[j][1] *= al.y * bL; Sk[j][2] *= al.z * bL; Sk[j][3] *= al.w * bL;
-                    Sd[j] = OPE::mfma16(ld2(KHc + (16 * j + r) * CC + 4 * g), xh_d, Sd[j]);
-                    Sk[j] = OPE::mfma16(ld2(XHc + (16 * j + r) * CC + 4 * g), kh_k, Sk[j]);
-                }
-                PHASE_MARK(0);
+        for (int i2 = 0; i2 < NB; i2 += 2) {
+            if (i2 < nb) {
                 __syncthreads();
                 PHASE_MARK(3);
+                const unsigned char *stage = smem + (s & 1) * STAGE_BYTES;
+#pragma unroll
+                for (int jb = 0; jb < 2; ++jb) {
+                    const int i = i2 + jb;
+                    if (i < nb) {
+                        const u16 *VOHc = reinterpret_cast<const u16 *>(stage + OFF_CM + (2 * jb) * CM_TILE);
+                        const u16 *VHc = reinterpret_cast<const u16 *>(stage + OFF_CM + (2 * jb + 1) * CM_TILE);
+                        const float *LX = lv_vec(stage, jb, 0), *LO = lv_vec(stage, jb, 1);
+                        {
+                            const uint2 a0 = pack4v<OPE>(S[0]), a1 = pack4v<OPE>(S[1]), a2 = pack4v<OPE>(S[2]),
+                                        a3 = pack4v<OPE>(S[3]);
+                            sv[i][0] = cat(a0, a1);
+                            sv[i][1] = cat(a2, a3);
+                        }
+                        const float lo = LO[ch];
+                        const uint2 vhc = ld2(VHc + ch * CC + 4 * g);
+#pragma unroll
+                        for (int j = 0; j < 4; ++j) {
+                            const float4 lx = *reinterpret_cast<const float4 *>(LX + 16 * j + 4 * g);
+                            S[j][0] *= lo * lx.x; S[j][1] *= lo * lx.y; S[j][2] *= lo * lx.z; S[j][3] *= lo * lx.w;
+                            S[j] = OPE::mfma16(ld2(VOHc + (16 * j + r) * CC + 4 * g), vhc, S[j]);
+                        }
+                    }
+                }
+                PHASE_MARK(0);
                 ++s;
             }
         }
-        // ---- re-anchor the running sums: u = rowsum(Gb * S_end), v = colsum(Gb * S_end)
+        // ---- re-anchor the running sum of the gate gradient: sum over the other side of Gb * S_end
         {
-            float us = 0.f, vs = 0.f;
+            float us = 0.f;
 #pragma unroll
             for (int j = 0; j < 4; ++j)
 #pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    us += Gd[j][i] * Sd[j][i];
-                    vs += Gk[j][i] * Sk[j][i];
-                }
-            us += __shfl_xor(us, 16, 64);
-            us += __shfl_xor(us, 32, 64);
-            vs += __shfl_xor(vs, 16, 64);
-            vs += __shfl_xor(vs, 32, 64);
-            u_carry = us;
-            v_carry = vs;
+                for (int i = 0; i < 4; ++i) us += G[j][i] * S[j][i];
+            carry = row_sums(us).all;
         }
         // ---- B stages: blocks last to first
 #pragma unroll
         for (int i = NB - 1; i >= 0; --i) {
             if (i < nb) {
+                __syncthreads();
+                PHASE_MARK(2);
                 const unsigned char *stage = smem + (s & 1) * STAGE_BYTES;
-                unsigned char *outp = smem + BOFF_OUT + (s & 1) * BOUT_BYTES;
-                const u16 *QT = tm_tile(stage, T_QT), *KT = tm_tile(stage, T_KT), *GT = tm_tile(stage, T_GT);
-                const u16 *XT = tm_tile(stage, T_XT), *KH = tm_tile(stage, T_KH), *XH = tm_tile(stage, T_XH);
-                const u16 *QTc = cm_tile(stage, T_QT), *KTc = cm_tile(stage, T_KT), *GTc = cm_tile(stage, T_GT);
-                const u16 *XTc = cm_tile(stage, T_XT);
-                const float *BLV = reinterpret_cast<const float *>(stage + OFF_BLV);
-                const float *ALV = reinterpret_cast<const float *>(stage + OFF_ALV);
+                const u16 *AOS = reinterpret_cast<const u16 *>(stage + OFF_TM + TM_AOS * TM_TILE);
+                const u16 *VOT = reinterpret_cast<const u16 *>(stage + OFF_TM + TM_VOT * TM_TILE);
+                const u16 *VOH = reinterpret_cast<const u16 *>(stage + OFF_TM + TM_VOH * TM_TILE);
+                const u16 *AOSc = reinterpret_cast<const u16 *>(stage + OFF_CM + CM_AOS * CM_TILE);
+                const u16 *ASc = reinterpret_cast<const u16 *>(stage + OFF_CM + CM_AS * CM_TILE);
+                const u16 *VTc = reinterpret_cast<const u16 *>(stage + OFF_CM + CM_VT * CM_TILE);
+                const float *LX = lv_vec(stage, 0, 0), *LO = lv_vec(stage, 0, 1);
                 const floatx4 zero = {0.f, 0.f, 0.f, 0.f};
-                // the four 16x16 token-token products (full contraction over 64 channels each)
+                // the 16x16 token-token product, in both orientations (full contraction over 64 channels)
                 const int ro = r * TS + 8 * g;
-                const uint4 kt_lo = ld4(KT + ro), kt_hi = ld4(KT + ro + 32), qt_lo = ld4(QT + ro), qt_hi = ld4(QT + ro + 32);
-                const uint4 gt_lo = ld4(GT + ro), gt_hi = ld4(GT + ro + 32), xt_lo = ld4(XT + ro), xt_hi = ld4(XT + ro + 32);
-                floatx4 pt1 = OPE::mfma32(kt_hi, qt_hi, OPE::mfma32(kt_lo, qt_lo, zero));   // P[t=r][s=4g+i]
-                floatx4 pt2 = OPE::mfma32(qt_hi, kt_hi, OPE::mfma32(qt_lo, kt_lo, zero));   // P[r'=4g+i][t=r]
-                floatx4 wt1 = OPE::mfma32(xt_hi, gt_hi, OPE::mfma32(xt_lo, gt_lo, zero));   // W[t=r][s=4g+i]
-                floatx4 wt2 = OPE::mfma32(gt_hi, xt_hi, OPE::mfma32(gt_lo, xt_lo, zero));   // W[r'=4g+i][t=r]
-                float pd[4], wd[4];     // diagonals for this lane's tokens 4g+i
+                const uint4 vot_lo = ld4(VOT + ro), vot_hi = ld4(VOT + ro + 32);
+                const uint4 aos_lo = ld4(AOS + ro), aos_hi = ld4(AOS + ro + 32);
+                floatx4 pt1 = OPE::mfma32(vot_hi, aos_hi, OPE::mfma32(vot_lo, aos_lo, zero));   // P[t=r][s=4g+i]
+                floatx4 pt2 = OPE::mfma32(aos_hi, vot_hi, OPE::mfma32(aos_lo, vot_lo, zero));   // P[r'=4g+i][t=r]
+                float pd[4];     // diagonal for this lane's tokens 4g+i
+#pragma unroll
+                for (int ii = 0; ii < 4; ++ii) pd[ii] = __shfl(pt1[ii], 20 * g + ii, 64);
 #pragma unroll
                 for (int ii = 0; ii < 4; ++ii) {
-                    pd[ii] = __shfl(pt1[ii], 20 * g + ii, 64);
-                    wd[ii] = __shfl(wt1[ii], 20 * g + ii, 64);
+                    pt1[ii] = (4 * g + ii < r) ? pt1[ii] : 0.f;
+                    pt2[ii] = (4 * g + ii > r) ? pt2[ii] : 0.f;
                 }
+                const uint2 pa_o = pack4v<OPE>(pt1), pa_v = pack4v<OPE>(pt2);
+                const uint2 vtc = ld2(VTc + ch * CC + 4 * g), asc = ld2(ASc + ch * CC + 4 * g);
+                const float lo = LO[ch];
+                const int po = r * TS + 16 * g;
+                // o' uses the block-start state
+                floatx4 oa = OPE::mfma32(ld4(AOS + po + 8), sv[i][1], OPE::mfma32(ld4(AOS + po), sv[i][0], zero));
+                oa += OPE::mfma16(pa_o, vtc, zero);
+                // v' uses the adjoint entering the block, scaled to the block end on the own side
+                floatx4 ga[4];
 #pragma unroll
-                for (int ii = 0; ii < 4; ++ii) {
-                    const bool lower = 4 * g + ii < r, upper = 4 * g + ii > r;
-                    pt1[ii] = lower ? pt1[ii] : 0.f;
-                    wt1[ii] = lower ? wt1[ii] : 0.f;
-                    pt2[ii] = upper ? pt2[ii] : 0.f;
-                    wt2[ii] = upper ? wt2[ii] : 0.f;
-                }
-                const uint2 pa_o = pack4v<OPE>(pt1), pa_x = pack4v<OPE>(pt2), pa_q = pack4v<OPE>(wt1), pa_k = pack4v<OPE>(wt2);
-                const uint2 xtc = ld2(XTc + ch * CC + 4 * g), gtc = ld2(GTc + ch * CC + 4 * g);
-                const uint2 ktc = ld2(KTc + ch * CC + 4 * g), qtc = ld2(QTc + ch * CC + 4 * g);
-                const float aL = ALV[ch], bL = BLV[ch];
-                const int po = r * TS + 4 * g;
-                // o' and dq' use the block-start state
-                floatx4 oa = OPE::mfma32(cat(ld2(QT + po), ld2(QT + po + 16)), cat(svd[i][0], svd[i][1]), zero);
-                oa = OPE::mfma32(cat(ld2(QT + po + 32), ld2(QT + po + 48)), cat(svd[i][2], svd[i][3]), oa);
-                oa += OPE::mfma16(pa_o, xtc, zero);
-                floatx4 dqa = OPE::mfma32(cat(ld2(GT + po), ld2(GT + po + 16)), cat(svk[i][0], svk[i][1]), zero);
-                dqa = OPE::mfma32(cat(ld2(GT + po + 32), ld2(GT + po + 48)), cat(svk[i][2], svk[i][3]), dqa);
-                dqa += OPE::mfma16(pa_q, ktc, zero);
-                // dx' and dk' use the adjoint entering the block, scaled to the block end on one side
-                floatx4 ga[4], gb[4];
-                uint2 gap[4], gbp[4];
+                for (int j = 0; j < 4; ++j) ga[j] = G[j] * lo;
+                const uint4 gp0 = cat(pack4v<OPE>(ga[0]), pack4v<OPE>(ga[1]));
+                const uint4 gp1 = cat(pack4v<OPE>(ga[2]), pack4v<OPE>(ga[3]));
+                floatx4 va = OPE::mfma32(ld4(VOH + po + 8), gp1, OPE::mfma32(ld4(VOH + po), gp0, zero));
+                va += OPE::mfma16(pa_v, asc, zero);
+                // adjoint of the previous block
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
-                    ga[j] = Gd[j] * aL;
-                    gb[j] = Gk[j] * bL;
-                    gap[j] = pack4v<OPE>(ga[j]);
-                    gbp[j] = pack4v<OPE>(gb[j]);
+                    const float4 lx = *reinterpret_cast<const float4 *>(LX + 16 * j + 4 * g);
+                    ga[j][0] *= lx.x; ga[j][1] *= lx.y; ga[j][2] *= lx.z; ga[j][3] *= lx.w;
+                    G[j] = OPE::mfma16(ld2(AOSc + (16 * j + r) * CC + 4 * g), asc, ga[j]);
                 }
-                floatx4 dxa = OPE::mfma32(cat(ld2(KH + po), ld2(KH + po + 16)), cat(gap[0], gap[1]), zero);
-                dxa = OPE::mfma32(cat(ld2(KH + po + 32), ld2(KH + po + 48)), cat(gap[2], gap[3]), dxa);
-                dxa += OPE::mfma16(pa_x, gtc, zero);
-                floatx4 dka = OPE::mfma32(cat(ld2(XH + po), ld2(XH + po + 16)), cat(gbp[0], gbp[1]), zero);
-                dka = OPE::mfma32(cat(ld2(XH + po + 32), ld2(XH + po + 48)), cat(gbp[2], gbp[3]), dka);
-                dka += OPE::mfma16(pa_k, qtc, zero);
-                // adjoint of the previous block: Gb <- (a_L (x) b_L) * Gb + sum_t gs_t (x) qs_t
-#pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    const float4 bl = *reinterpret_cast<const float4 *>(BLV + 16 * j + 4 * g);
-                    const float4 al = *reinterpret_cast<const float4 *>(ALV + 16 * j + 4 * g);
-                    ga[j][0] *= bl.x; ga[j][1] *= bl.y; ga[j][2] *= bl.z; ga[j][3] *= bl.w;
-                    gb[j][0] *= al.x; gb[j][1] *= al.y; gb[j][2] *= al.z; gb[j][3] *= al.w;
-                    Gd[j] = OPE::mfma16(ld2(QTc + (16 * j + r) * CC + 4 * g), gtc, ga[j]);
-                    Gk[j] = OPE::mfma16(ld2(GTc + (16 * j + r) * CC + 4 * g), qtc, gb[j]);
-                }
-                // ---- value side: d_x, d_f for tokens 4g+i, channel ch
+                // ---- gradients for tokens 4g+i, channel ch
                 {
-                    float gsv[4], xtv[4], du[4];
-                    unpack4<OPE>(gtc, gsv);
-                    unpack4<OPE>(xtc, xtv);
+                    float asv[4], vtv[4], du[4];
+                    unpack4<OPE>(asc, asv);
+                    unpack4<OPE>(vtc, vtv);
 #pragma unroll
-                    for (int ii = 0; ii < 4; ++ii) du[ii] = oa[ii] * gsv[ii] - dxa[ii] * xtv[ii];
-                    reverse_running_sum(du, u_carry, g, r);
-                    const float4 rf = *reinterpret_cast<const float4 *>(cf_tile(stage, F_RF) + ch * CC + 4 * g);
-                    const float4 ia = *reinterpret_cast<const float4 *>(cf_tile(stage, F_IA) + ch * CC + 4 * g);
-                    const float rfv[4] = {rf.x, rf.y, rf.z, rf.w}, iav[4] = {ia.x, ia.y, ia.z, ia.w};
-                    u16 *DX = reinterpret_cast<u16 *>(outp + O_DX * BOUT_TILE), *DF = reinterpret_cast<u16 *>(outp + O_DF * BOUT_TILE);
-#pragma unroll
-                    for (int ii = 0; ii < 4; ++ii) {
-                        DX[(4 * g + ii) * OS + ch] = cvt1<IOE>(iav[ii] * (dxa[ii] + gsv[ii] * pd[ii]));
-                        DF[(4 * g + ii) * OS + ch] = cvt1<IOE>(du[ii] * rfv[ii]);
+                    for (int ii = 0; ii < 4; ++ii) du[ii] = oa[ii] * asv[ii] - va[ii] * vtv[ii];
+                    reverse_running_sum_swap(du, carry, g);
+                    const float *cf = reinterpret_cast<const float *>(stage + OFF_CF) + ch * CC + 4 * g;
+                    const float4 rg = *reinterpret_cast<const float4 *>(cf + F_RG * (CF_TILE / 4));
+                    const float4 ip = *reinterpret_cast<const float4 *>(cf + F_IP * (CF_TILE / 4));
+                    const float rgv[4] = {rg.x, rg.y, rg.z, rg.w}, ipv[4] = {ip.x, ip.y, ip.z, ip.w};
+                    // 16 lanes write 32 contiguous bytes of a token row; the four waves complete the row.
+                    // Only the last block of the sequence can reach past its end.
+                    const int tg = (int)chunk * C + i * CH_L + 4 * g;         // this lane's first token
+                    const u32 go = (u32)tg * CH_N + (u32)ch;
+                    float ppv[4] = {0.f, 0.f, 0.f, 0.f};
+                    if (side == 1) {
+                        const float4 pp = *reinterpret_cast<const float4 *>(cf + F_PP * (CF_TILE / 4));
+                        ppv[0] = pp.x; ppv[1] = pp.y; ppv[2] = pp.z; ppv[3] = pp.w;
                     }
-                }
-                // ---- key side: d_q, d_k, d_f_key for tokens 4g+i, channel ch
-                {
-                    float qsv[4], ktv[4], dv[4];
-                    unpack4<OPE>(qtc, qsv);
-                    unpack4<OPE>(ktc, ktv);
+                    auto store = [&](int ii) {
+                        d_val[go + ii * CH_N] = cvt1<IOE>(ipv[ii] * (va[ii] + asv[ii] * pd[ii]));
+                        d_gate[go + ii * CH_N] = cvt1<IOE>(du[ii] * rgv[ii]);
+                        if (side == 1) d_adj[go + ii * CH_N] = cvt1<IOE>(ppv[ii] * (oa[ii] + vtv[ii] * pd[ii]));
+                    };
+                    if ((int)chunk * C + (i + 1) * CH_L <= T) {
 #pragma unroll
-                    for (int ii = 0; ii < 4; ++ii) dv[ii] = dqa[ii] * qsv[ii] - dka[ii] * ktv[ii];
-                    reverse_running_sum(dv, v_carry, g, r);
-                    const float4 bt = *reinterpret_cast<const float4 *>(cf_tile(stage, F_BT) + ch * CC + 4 * g);
-                    const float4 rk = *reinterpret_cast<const float4 *>(cf_tile(stage, F_RFK) + ch * CC + 4 * g);
-                    const float btv[4] = {bt.x, bt.y, bt.z, bt.w}, rkv[4] = {rk.x, rk.y, rk.z, rk.w};
-                    u16 *DQ = reinterpret_cast<u16 *>(outp + O_DQ * BOUT_TILE), *DK = reinterpret_cast<u16 *>(outp + O_DK * BOUT_TILE);
-                    u16 *DFK = reinterpret_cast<u16 *>(outp + O_DFK * BOUT_TILE);
+                        for (int ii = 0; ii < 4; ++ii) store(ii);
+                    } else {
 #pragma unroll
-                    for (int ii = 0; ii < 4; ++ii) {
-                        DQ[(4 * g + ii) * OS + ch] = cvt1<IOE>(btv[ii] * (dqa[ii] + ktv[ii] * wd[ii]));
-                        DK[(4 * g + ii) * OS + ch] =
-                            cvt1<IOE>(__builtin_amdgcn_rcpf(btv[ii]) * (dka[ii] + qsv[ii] * wd[ii]));
-                        DFK[(4 * g + ii) * OS + ch] = cvt1<IOE>(dv[ii] * rkv[ii]);
+                        for (int ii = 0; ii < 4; ++ii)
+                            if (tg + ii < T) store(ii);
                     }
                 }
                 PHASE_MARK(1);
-                __syncthreads();
-                PHASE_MARK(2);
                 ++s;
             }
         }
     }
-    // d_s0 = adjoint after the first block
-    {
+    // d_s0 = adjoint after the first block (value side only: rows of [d][k] are contiguous there)
+    if (side == 0) {
         u16 *ds = reinterpret_cast<u16 *>(p.d_s0) + b * (CH_N * CH_N);
 #pragma unroll
-        for (int j = 0; j < 4; ++j) *reinterpret_cast<uint2 *>(ds + ch * CH_N + 16 * j + 4 * g) = pack4v<IOE>(Gd[j]);
+        for (int j = 0; j < 4; ++j) *reinterpret_cast<uint2 *>(ds + ch * CH_N + 16 * j + 4 * g) = pack4v<IOE>(G[j]);
     }
     PHASE_END(tid >> 6);
 }
 
 template <typename IOE, typename OPE, int NB>
-__global__ __launch_bounds__(BWD_THREADS) void lfw_bwd_chunk_kernel(ChunkBwdArgs p) {
+__global__ __launch_bounds__(SP_THREADS) void lfw_bwd_chunk_kernel(ChunkBwdArgs p, int rows_padded) {
     extern __shared__ __align__(16) unsigned char smem[];
     const int tid = threadIdx.x;
-    const int64_t b = blockIdx.x;
+    // blockIdx = side * rows_padded + row with rows_padded a multiple of 8: the two workgroups of a
+    // row land on the same XCD and share its L2 for the inputs both of them read
+    const int side = (int)blockIdx.x >= rows_padded ? 1 : 0;
+    const int64_t b = (int)blockIdx.x - side * rows_padded;
+    if (b >= p.B) return;
     // both branches execute exactly 2 + (number of stages) workgroup barriers
     if (tid < 256)
-        bwd_matrix_waves<IOE, OPE, NB>(p, smem, tid, b);
+        split_matrix_waves<IOE, OPE, NB>(p, smem, tid, b, side);
     else
-        bwd_prep_waves<IOE, OPE, NB>(p, smem, tid - 256, b);
+        split_prep_waves<IOE, OPE, NB>(p, smem, tid - 256, b, side);
 }
 
 template <typename IOE, typename OPE, int NB> int launch(const ChunkBwdArgs &a, hipStream_t stream) {
     auto kern = lfw_bwd_chunk_kernel<IOE, OPE, NB>;
     // more than 64 KB of dynamic LDS has to be enabled per function (and per device)
     int rc = check_hip(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, BWD_SMEM),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, SP_SMEM),
                        "hipFuncSetAttribute(backward chunk kernel)");
     if (rc) return rc;
-    if (a.B > 0x7fffffffLL) return fail(T2FW_ERR_UNSUPPORTED, "B=%lld is too large", (long long)a.B);
-    hipLaunchKernelGGL(kern, dim3((unsigned)a.B), dim3(BWD_THREADS), BWD_SMEM, stream, a);
+    if (a.B > 0x1fffffffLL) return fail(T2FW_ERR_UNSUPPORTED, "B=%lld is too large", (long long)a.B);
+    if (a.T >= CHUNK_MAX_T) return fail(T2FW_ERR_UNSUPPORTED, "T=%lld is too long for 32-bit row offsets", (long long)a.T);
+    const int rows_padded = (int)((a.B + 7) / 8 * 8);
+    hipLaunchKernelGGL(kern, dim3(2u * (unsigned)rows_padded), dim3(SP_THREADS), SP_SMEM, stream, a, rows_padded);
     return check_hip(hipGetLastError(), "lfw_bwd_chunk_kernel launch");
 }
 

@@ -77,32 +77,43 @@ def test_config_like_inputs(dtype, gate_mean, state_std, B, T, C):
     check_against_oracle((x, f, q, k, fk, s), go, gs, C, dtype, expect_flagged=0)
 
 
-@pytest.mark.parametrize("flags", [4, 8], ids=["whole_row", "split_by_side"])
-@pytest.mark.parametrize("dtype,B,T,C", [(torch.float16, 4, 1024, 64), (torch.bfloat16, 3, 112, 64),
-                                         (torch.float16, 2, 48, 32), (torch.float16, 3, 16, 64),
-                                         (torch.bfloat16, 2, 80, 64), (torch.float16, 2, 77, 32)])
-def test_both_backward_kernels(flags, dtype, B, T, C):
-    """The backward has two matrix-core kernels (one workgroup per batch row, or one per side of the
-    state); the library picks by batch size, the flags force either.  T = 77 is not a multiple of 16,
-    which the split kernel does not take: the call must still succeed (whole-row kernel)."""
+@pytest.mark.parametrize("dtype,B,T,C", [(torch.bfloat16, 3, 112, 64), (torch.float16, 2, 48, 32),
+                                         (torch.float16, 3, 16, 64), (torch.bfloat16, 2, 80, 64),
+                                         (torch.float16, 2, 77, 32), (torch.float16, 3, 15, 64),
+                                         (torch.bfloat16, 2, 65, 64), (torch.float16, 2, 113, 64)])
+def test_short_and_ragged_last_chunks(dtype, B, T, C):
+    """Last chunks of 1..4 blocks, with and without a partial last block (the backward handles the
+    last chunk of a sequence with a general schedule and the full chunks with a fixed one)."""
     x, f, q, k, fk, s, go, gs = make_config_inputs(B, T, 64, 64, dtype, seed=100 + T, gate_mean=2.5, state_std=0.3)
-    check_against_oracle((x, f, q, k, fk, s), go, gs, C, dtype, flags=flags, expect_flagged=0)
+    check_against_oracle((x, f, q, k, fk, s), go, gs, C, dtype, expect_flagged=0)
 
 
-@pytest.mark.parametrize("flags", [4, 8], ids=["whole_row", "split_by_side"])
-def test_both_backward_kernels_flag_the_same_rows(flags):
-    B, T = 3, 96
+def test_flagged_rows_with_a_partial_last_block():
+    B, T = 3, 90
     x, f, q, k, fk, s, go, gs = make_config_inputs(B, T, 64, 64, torch.float16, seed=11, state_std=0.3)
     f, fk = f.clone(), fk.clone()
     f[0, 40, 9] = 0.0
-    fk[2, 90, 63] = 2.0
-    out, nxt, ckpt, grads, flagged = run_abi((x, f, q, k, fk, s), go, gs, 32, flags=flags)
+    fk[2, 89, 63] = 2.0                 # in the partial last block
+    out, nxt, ckpt, grads, flagged = run_abi((x, f, q, k, fk, s), go, gs, 32)
     assert flagged == (2, 2), flagged
     r_grads = c_oracle.lfw_backward(go, gs, x, f, q, k, fk, s)
     for n, g, r in zip(NAMES, grads, r_grads):
         assert_close(g[0:1], r[0:1], torch.float16, n + "[flagged row 0]")
         assert_close(g[2:3], r[2:3], torch.float16, n + "[flagged row 2]")
         assert_close(g, r, torch.float16, n, tol=TOL_CHUNK_GATE if n in ("d_f", "d_f_key") else TOL_CHUNK)
+
+
+def test_no_fixup_flag_reports_but_does_not_repair():
+    from t2fw_amd import _lib
+    B, T = 2, 64
+    x, f, q, k, fk, s, go, gs = make_config_inputs(B, T, 64, 64, torch.float16, seed=12, state_std=0.3)
+    f = f.clone()
+    f[1, 5, 2] = 0.0
+    out, nxt, ckpt, grads, flagged = run_abi((x, f, q, k, fk, s), go, gs, 64, flags=_lib.FLAG_NO_FIXUP)
+    assert flagged == (1, 1), flagged
+    # the unflagged row is valid without the exact kernels having run
+    r_out, _ = c_oracle.lfw_forward(x[:1], f[:1], q[:1], k[:1], fk[:1], s[:1])
+    assert_close(out[:1], r_out, torch.float16, "outputs[row 0]", tol=TOL_CHUNK)
 
 
 def test_wide_gate_distribution_stays_on_the_chunked_path():
