@@ -88,6 +88,25 @@ def test_short_and_ragged_last_chunks(dtype, B, T, C):
     check_against_oracle((x, f, q, k, fk, s), go, gs, C, dtype, expect_flagged=0)
 
 
+def test_batch_larger_than_half_the_device():
+    """With more than 128 rows the forward runs one workgroup per row (below that, two); the
+    backward's grid exceeds the number of CUs."""
+    B, T = 136, 80
+    x, f, q, k, fk, s, go, gs = make_config_inputs(B, T, 64, 64, torch.float16, seed=31, state_std=0.2)
+    f = f.clone()
+    f[135, 70, 50] = 1.25               # one row for the exact kernels, in the last workgroup
+    out, nxt, ckpt, grads, flagged = run_abi((x, f, q, k, fk, s), go, gs, 64)
+    assert flagged == (1, 1), flagged
+    rows = [0, 63, 64, 127, 128, 135]
+    sub = [t[rows] for t in (x, f, q, k, fk, s)]
+    r_out, r_nxt = c_oracle.lfw_forward(*sub)
+    r_grads = c_oracle.lfw_backward(go[rows], gs[rows], *sub)
+    assert_close(out[rows], r_out, torch.float16, "outputs", tol=TOL_CHUNK)
+    assert_close(nxt[rows], r_nxt, torch.float16, "next_state", tol=TOL_CHUNK)
+    for n, g, r in zip(NAMES, grads, r_grads):
+        assert_close(g[rows], r, torch.float16, n, tol=TOL_CHUNK_GATE if n in ("d_f", "d_f_key") else TOL_CHUNK)
+
+
 def test_flagged_rows_with_a_partial_last_block():
     B, T = 3, 90
     x, f, q, k, fk, s, go, gs = make_config_inputs(B, T, 64, 64, torch.float16, seed=11, state_std=0.3)
