@@ -141,6 +141,19 @@ int t2fw_dfw_backward(const void *g_out, const void *g_state,
                       int64_t B, int64_t T, int64_t D, int64_t M,
                       int32_t dtype, void *stream);
 
+/*
+ * Sigmoid gating of both forget gates in one launch: f = sigmoid(f_logit) [n_f elements],
+ * f_key = sigmoid(fk_logit) [n_fk elements]; outputs may alias the inputs.  The reference leaves
+ * the non-linearity to the caller (functional_lfw.py:25-30); dtype f32 / f16 / bf16.
+ */
+int t2fw_gate_forward(const void *f_logit, const void *fk_logit, void *f, void *f_key,
+                      int64_t n_f, int64_t n_fk, int32_t dtype, void *stream);
+
+/* d_logit = d_gate * gate * (1 - gate) for both gates; outputs may alias d_f / d_f_key. */
+int t2fw_gate_backward(const void *d_f, const void *d_f_key, const void *f, const void *f_key,
+                       void *d_f_logit, void *d_fk_logit,
+                       int64_t n_f, int64_t n_fk, int32_t dtype, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

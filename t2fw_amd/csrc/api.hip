@@ -4,6 +4,7 @@
 #include "lfw_scan.hpp"
 #include "lfw_chunk.hpp"
 #include "dfw_scan.hpp"
+#include "gate.hpp"
 #include "lfw_step.hpp"
 
 #include <cstring>
@@ -299,6 +300,35 @@ int t2fw_dfw_backward(const void *g_out, const void *g_state, const void *q, con
     a.d_q = d_q; a.d_k = d_k; a.d_v = d_v; a.d_s0 = d_s0;
     a.B = B; a.T = T; a.D = D; a.M = M;
     return dfw_backward(a, dtype, st);
+}
+
+int t2fw_gate_forward(const void *f_logit, const void *fk_logit, void *f, void *f_key, int64_t n_f, int64_t n_fk,
+                      int32_t dtype, void *stream) {
+    const size_t es = elem_size(dtype);
+    if (es == 0) return fail(T2FW_ERR_BAD_DTYPE, "unknown dtype code %d", dtype);
+    if (n_f < 0 || n_fk < 0) return fail(T2FW_ERR_BAD_SHAPE, "element counts must be non-negative");
+    if ((n_f > 0 && (f_logit == nullptr || f == nullptr)) || (n_fk > 0 && (fk_logit == nullptr || f_key == nullptr)))
+        return fail(T2FW_ERR_NULL_POINTER, "null gate pointer");
+    if (!aligned16({f_logit, fk_logit, f, f_key})) return fail(T2FW_ERR_MISALIGNED, "gate arrays must be 16-byte aligned");
+    GateFwdArgs a{};
+    a.f_logit = f_logit; a.fk_logit = fk_logit; a.f = f; a.f_key = f_key; a.n_f = n_f; a.n_fk = n_fk;
+    return gate_forward(a, dtype, static_cast<hipStream_t>(stream));
+}
+
+int t2fw_gate_backward(const void *d_f, const void *d_f_key, const void *f, const void *f_key, void *d_f_logit,
+                       void *d_fk_logit, int64_t n_f, int64_t n_fk, int32_t dtype, void *stream) {
+    const size_t es = elem_size(dtype);
+    if (es == 0) return fail(T2FW_ERR_BAD_DTYPE, "unknown dtype code %d", dtype);
+    if (n_f < 0 || n_fk < 0) return fail(T2FW_ERR_BAD_SHAPE, "element counts must be non-negative");
+    if ((n_f > 0 && (d_f == nullptr || f == nullptr || d_f_logit == nullptr)) ||
+        (n_fk > 0 && (d_f_key == nullptr || f_key == nullptr || d_fk_logit == nullptr)))
+        return fail(T2FW_ERR_NULL_POINTER, "null gate pointer");
+    if (!aligned16({d_f, d_f_key, f, f_key, d_f_logit, d_fk_logit}))
+        return fail(T2FW_ERR_MISALIGNED, "gate arrays must be 16-byte aligned");
+    GateBwdArgs a{};
+    a.d_f = d_f; a.d_f_key = d_f_key; a.f = f; a.f_key = f_key; a.d_f_logit = d_f_logit; a.d_fk_logit = d_fk_logit;
+    a.n_f = n_f; a.n_fk = n_fk;
+    return gate_backward(a, dtype, static_cast<hipStream_t>(stream));
 }
 
 }  // extern "C"

@@ -45,6 +45,79 @@ def _dtype_code(dtype):
         raise RuntimeError("t2fw: unsupported dtype %s" % dtype)
 
 
+def _lfw_forward(value, forget, query, key, f_key, state, need_grad):
+    """Checks as in t2fw/functional_lfw.py:42-49 and t2fw/csrc/lfw.cpp:24-26,36-41, then the forward
+    kernels.  Returns (outputs, next_state, ckpt or None, checkpoint interval, flags)."""
+    assert value.shape == forget.shape
+    assert query.shape == key.shape
+    assert query.shape == f_key.shape
+    assert forget.dtype == value.dtype
+    assert query.dtype == value.dtype
+    assert f_key.dtype == value.dtype
+    assert state.dtype == value.dtype
+    assert key.dtype == value.dtype
+    for t, n in ((value, "x"), (forget, "f"), (query, "query"), (key, "key"),
+                 (f_key, "f_key"), (state, "state")):
+        _check_input(t, n)
+    if value.dim() != 3 or query.dim() != 3 or state.dim() != 3:
+        raise RuntimeError("t2fw: expected x,f [B,T,D]; q,k,f_key [B,T,K]; state [B,D,K]")
+    B, T, D = value.shape
+    K = query.shape[2]
+    if query.shape[0] != B or query.shape[1] != T or tuple(state.shape) != (B, D, K):
+        raise RuntimeError("t2fw: inconsistent shapes x %s, query %s, state %s"
+                           % (tuple(value.shape), tuple(query.shape), tuple(state.shape)))
+    code = _dtype_code(value.dtype)
+    lib = _lib.load()
+    C = _ckpt_interval()
+    flags = _flags()
+    dev = value.device
+    with torch.cuda.device(dev):
+        outputs = torch.empty_like(value)
+        next_state = torch.empty_like(state)
+        ckpt = None
+        if need_grad:
+            nc = lib.t2fw_lfw_num_ckpt(T, C)
+            ckpt = torch.empty((B, nc, D, K), dtype=value.dtype, device=dev)
+        ws_bytes = lib.t2fw_lfw_workspace_bytes(B, T, D, K, C, code, flags)
+        ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev) if ws_bytes else None
+        _lib.check(lib.t2fw_lfw_forward(
+            _lib.ptr(value), _lib.ptr(forget), _lib.ptr(query), _lib.ptr(key), _lib.ptr(f_key),
+            _lib.ptr(state), _lib.ptr(outputs), _lib.ptr(next_state), _lib.ptr(ckpt),
+            B, T, D, K, C, code, flags, _lib.ptr(ws), ws_bytes,
+            _lib.current_stream_handle(dev)))
+    return outputs, next_state, ckpt, C, flags
+
+
+def _lfw_backward(grad_output, grad_state, value, forget, query, key, f_key, state, ckpt, C, flags):
+    """The backward kernels; gradients in the order of t2fw/csrc/lfw.cpp:95."""
+    # t2fw/functional_lfw.py:71-72
+    assert grad_state.dtype == value.dtype
+    assert grad_output.dtype == value.dtype
+    grad_output = grad_output.contiguous()
+    grad_state = grad_state.contiguous()
+    B, T, D = value.shape
+    K = query.shape[2]
+    code = _dtype_code(value.dtype)
+    lib = _lib.load()
+    dev = value.device
+    with torch.cuda.device(dev):
+        d_x = torch.empty_like(value)
+        d_f = torch.empty_like(forget)
+        d_q = torch.empty_like(query)
+        d_k = torch.empty_like(key)
+        d_fk = torch.empty_like(f_key)
+        d_s = torch.empty_like(state)
+        ws_bytes = lib.t2fw_lfw_workspace_bytes(B, T, D, K, C, code, flags)
+        ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev) if ws_bytes else None
+        _lib.check(lib.t2fw_lfw_backward(
+            _lib.ptr(grad_output), _lib.ptr(grad_state), _lib.ptr(value), _lib.ptr(forget),
+            _lib.ptr(query), _lib.ptr(key), _lib.ptr(f_key), _lib.ptr(state), _lib.ptr(ckpt),
+            _lib.ptr(d_x), _lib.ptr(d_f), _lib.ptr(d_q), _lib.ptr(d_k), _lib.ptr(d_fk), _lib.ptr(d_s),
+            B, T, D, K, C, code, flags, _lib.ptr(ws), ws_bytes,
+            _lib.current_stream_handle(dev)))
+    return d_x, d_f, d_q, d_k, d_fk, d_s
+
+
 class LFWFunction(torch.autograd.Function):
     """Decay update rule S_t = S_{t-1} * (f_t (x) f_key_t) + x_t (x) k_t, o_t = S_t q_t.
     Inputs are already gated (no sigmoid is applied here), as in the reference."""
@@ -52,45 +125,8 @@ class LFWFunction(torch.autograd.Function):
     @staticmethod
     def forward(ctx, value, forget, query, key, f_key, state):
         """Return: (outputs [B,T,D], final state [B,D,K])"""
-        # same asserts as t2fw/functional_lfw.py:42-49
-        assert value.shape == forget.shape
-        assert query.shape == key.shape
-        assert query.shape == f_key.shape
-        assert forget.dtype == value.dtype
-        assert query.dtype == value.dtype
-        assert f_key.dtype == value.dtype
-        assert state.dtype == value.dtype
-        assert key.dtype == value.dtype
-        for t, n in ((value, "x"), (forget, "f"), (query, "query"), (key, "key"),
-                     (f_key, "f_key"), (state, "state")):
-            _check_input(t, n)
-        if value.dim() != 3 or query.dim() != 3 or state.dim() != 3:
-            raise RuntimeError("t2fw: expected x,f [B,T,D]; q,k,f_key [B,T,K]; state [B,D,K]")
-        B, T, D = value.shape
-        K = query.shape[2]
-        if query.shape[0] != B or query.shape[1] != T or tuple(state.shape) != (B, D, K):
-            raise RuntimeError("t2fw: inconsistent shapes x %s, query %s, state %s"
-                               % (tuple(value.shape), tuple(query.shape), tuple(state.shape)))
-        code = _dtype_code(value.dtype)
-        lib = _lib.load()
         need_grad = any(ctx.needs_input_grad)
-        C = _ckpt_interval()
-        flags = _flags()
-        dev = value.device
-        with torch.cuda.device(dev):
-            outputs = torch.empty_like(value)
-            next_state = torch.empty_like(state)
-            ckpt = None
-            if need_grad:
-                nc = lib.t2fw_lfw_num_ckpt(T, C)
-                ckpt = torch.empty((B, nc, D, K), dtype=value.dtype, device=dev)
-            ws_bytes = lib.t2fw_lfw_workspace_bytes(B, T, D, K, C, code, flags)
-            ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev) if ws_bytes else None
-            _lib.check(lib.t2fw_lfw_forward(
-                _lib.ptr(value), _lib.ptr(forget), _lib.ptr(query), _lib.ptr(key), _lib.ptr(f_key),
-                _lib.ptr(state), _lib.ptr(outputs), _lib.ptr(next_state), _lib.ptr(ckpt),
-                B, T, D, K, C, code, flags, _lib.ptr(ws), ws_bytes,
-                _lib.current_stream_handle(dev)))
+        outputs, next_state, ckpt, C, flags = _lfw_forward(value, forget, query, key, f_key, state, need_grad)
         if need_grad:
             ctx.save_for_backward(value, forget, query, key, f_key, state, ckpt)
             ctx.ckpt_interval = C
@@ -100,34 +136,57 @@ class LFWFunction(torch.autograd.Function):
     @staticmethod
     def backward(ctx, grad_output, grad_state):
         value, forget, query, key, f_key, state, ckpt = ctx.saved_tensors
-        # t2fw/functional_lfw.py:71-72
-        assert grad_state.dtype == value.dtype
-        assert grad_output.dtype == value.dtype
-        grad_output = grad_output.contiguous()
-        grad_state = grad_state.contiguous()
-        B, T, D = value.shape
-        K = query.shape[2]
-        code = _dtype_code(value.dtype)
+        return _lfw_backward(grad_output, grad_state, value, forget, query, key, f_key, state, ckpt,
+                             ctx.ckpt_interval, ctx.flags)
+
+
+def sigmoid_gates(f_logit, fk_logit, out_f=None, out_fk=None):
+    """f = sigmoid(f_logit), f_key = sigmoid(fk_logit) in one launch (no autograd)."""
+    for t, n in ((f_logit, "f_logit"), (fk_logit, "fk_logit")):
+        _check_input(t, n)
+    assert f_logit.dtype == fk_logit.dtype
+    lib = _lib.load()
+    dev = f_logit.device
+    with torch.cuda.device(dev):
+        f = torch.empty_like(f_logit) if out_f is None else out_f
+        fk = torch.empty_like(fk_logit) if out_fk is None else out_fk
+        _lib.check(lib.t2fw_gate_forward(_lib.ptr(f_logit), _lib.ptr(fk_logit), _lib.ptr(f), _lib.ptr(fk),
+                                         f_logit.numel(), fk_logit.numel(), _dtype_code(f_logit.dtype),
+                                         _lib.current_stream_handle(dev)))
+    return f, fk
+
+
+class LFWGatedFunction(torch.autograd.Function):
+    """``LFWFunction`` on gate *logits*: f = sigmoid(f_logit), f_key = sigmoid(fk_logit) are computed
+    by one streaming kernel for both gates, the gates (not the logits) are kept for backward, and
+    the gate gradients are turned into logit gradients in place by one more kernel.  The reference
+    leaves the non-linearity to the caller (t2fw/functional_lfw.py:25-30), where it costs two
+    elementwise passes forward and several backward, plus a second saved tensor per gate."""
+
+    @staticmethod
+    def forward(ctx, value, f_logit, query, key, fk_logit, state):
+        assert value.shape == f_logit.shape and query.shape == fk_logit.shape
+        assert f_logit.dtype == value.dtype and fk_logit.dtype == value.dtype
+        forget, f_key = sigmoid_gates(f_logit, fk_logit)
+        need_grad = any(ctx.needs_input_grad)
+        outputs, next_state, ckpt, C, flags = _lfw_forward(value, forget, query, key, f_key, state, need_grad)
+        if need_grad:
+            ctx.save_for_backward(value, forget, query, key, f_key, state, ckpt)
+            ctx.ckpt_interval = C
+            ctx.flags = flags
+        return outputs, next_state
+
+    @staticmethod
+    def backward(ctx, grad_output, grad_state):
+        value, forget, query, key, f_key, state, ckpt = ctx.saved_tensors
+        d_x, d_f, d_q, d_k, d_fk, d_s = _lfw_backward(grad_output, grad_state, value, forget, query, key, f_key,
+                                                      state, ckpt, ctx.ckpt_interval, ctx.flags)
         lib = _lib.load()
-        C = ctx.ckpt_interval
-        flags = ctx.flags
         dev = value.device
         with torch.cuda.device(dev):
-            d_x = torch.empty_like(value)
-            d_f = torch.empty_like(forget)
-            d_q = torch.empty_like(query)
-            d_k = torch.empty_like(key)
-            d_fk = torch.empty_like(f_key)
-            d_s = torch.empty_like(state)
-            ws_bytes = lib.t2fw_lfw_workspace_bytes(B, T, D, K, C, code, flags)
-            ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev) if ws_bytes else None
-            _lib.check(lib.t2fw_lfw_backward(
-                _lib.ptr(grad_output), _lib.ptr(grad_state), _lib.ptr(value), _lib.ptr(forget),
-                _lib.ptr(query), _lib.ptr(key), _lib.ptr(f_key), _lib.ptr(state), _lib.ptr(ckpt),
-                _lib.ptr(d_x), _lib.ptr(d_f), _lib.ptr(d_q), _lib.ptr(d_k), _lib.ptr(d_fk), _lib.ptr(d_s),
-                B, T, D, K, C, code, flags, _lib.ptr(ws), ws_bytes,
-                _lib.current_stream_handle(dev)))
-        # order of t2fw/csrc/lfw.cpp:95
+            _lib.check(lib.t2fw_gate_backward(_lib.ptr(d_f), _lib.ptr(d_fk), _lib.ptr(forget), _lib.ptr(f_key),
+                                              _lib.ptr(d_f), _lib.ptr(d_fk), d_f.numel(), d_fk.numel(),
+                                              _dtype_code(value.dtype), _lib.current_stream_handle(dev)))
         return d_x, d_f, d_q, d_k, d_fk, d_s
 
 
