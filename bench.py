@@ -5,7 +5,7 @@ A "step" is one forward + backward pass of the decay-rule recurrence over one ba
 synthetic input already resident in HBM, at the headline configuration
 (B*H=96, T=1024, D=K=64, fp16 I/O, checkpoint interval 64).  Prints ONE JSON line.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg3|cfg2|cfg4|cfg5|copy256]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg3|cfg3_heads|cfg2|cfg4|cfg5|copy256]
                     [--no-cpu-baseline]
 
 value      = B*T*steps / wall time of the timed region, in Mtokens/s (token = one
@@ -35,6 +35,8 @@ WORKLOADS = {
     # name: (B, T, D, K, dtype, gate_mean, state_std, backward)
     "cfg2": dict(B=96, T=1024, D=64, K=64, dtype="float16", gate_mean=2.0, state_std=0.0, backward=False),
     "cfg3": dict(B=96, T=1024, D=64, K=64, dtype="float16", gate_mean=2.0, state_std=0.0, backward=True),
+    # cfg3 with the head axis kept next to the channels: tensors [8, 1024, 12, 64], head-strided entry points
+    "cfg3_heads": dict(B=96, H=12, T=1024, D=64, K=64, dtype="float16", gate_mean=2.0, state_std=0.0, backward=True),
     "cfg4": dict(B=128, T=8192, D=64, K=64, dtype="bfloat16", gate_mean=3.0, state_std=0.1, backward=True),
     "cfg5": dict(B=49152, T=1, D=64, K=64, dtype="float16", gate_mean=2.0, state_std=0.0, backward=False),
 }
@@ -83,6 +85,7 @@ def main():
     lib = _lib.load()
     w = WORKLOADS[args.workload]
     B, T, D, K = w["B"], w["T"], w["D"], w["K"]
+    H = w.get("H")                     # None: folded rows [B, T, D]; else rows are the heads of [B / H, T, H, D] tensors
     dtype = getattr(torch, w["dtype"])
     es = torch.empty((), dtype=dtype).element_size()
     C = args.ckpt_interval
@@ -102,6 +105,9 @@ def main():
     for i in range(nsets):
         x, f, q, k, fk, s, go, gs = make_config_inputs(B, T, D, K, dtype, seed=i, gate_mean=w["gate_mean"],
                                                         state_std=w["state_std"])
+        if H:
+            heads = lambda t: t.view(B // H, H, T, t.shape[2]).transpose(1, 2).contiguous()
+            x, f, q, k, fk, go = (heads(t) for t in (x, f, q, k, fk, go))
         ins = [t.to(dev) for t in (x, f, q, k, fk, s)]
         d = dict(ins=ins, out=torch.empty_like(ins[0]), nxt=torch.empty_like(ins[5]),
                  ws=torch.empty(max(ws_bytes, 1), dtype=torch.uint8, device=dev))
@@ -112,17 +118,20 @@ def main():
         sets.append(d)
     stream = _lib.current_stream_handle(dev)
 
+    dims = (B // H, T, H, D, K) if H else (B, T, D, K)
+    lfw_forward = lib.t2fw_lfw_forward_heads if H else lib.t2fw_lfw_forward
+    lfw_backward = lib.t2fw_lfw_backward_heads if H else lib.t2fw_lfw_backward
+
     def fwd(d):
-        _lib.check(lib.t2fw_lfw_forward(*[_lib.ptr(t) for t in d["ins"]], _lib.ptr(d["out"]), _lib.ptr(d["nxt"]),
-                                        _lib.ptr(d.get("ckpt")), B, T, D, K, C, code, flags,
-                                        _lib.ptr(d["ws"]), ws_bytes, stream))
+        _lib.check(lfw_forward(*[_lib.ptr(t) for t in d["ins"]], _lib.ptr(d["out"]), _lib.ptr(d["nxt"]),
+                               _lib.ptr(d.get("ckpt")), *dims, C, code, flags, _lib.ptr(d["ws"]), ws_bytes, stream))
 
     def bwd(d):
         i = d["ins"]
         g = d["grads"]
-        _lib.check(lib.t2fw_lfw_backward(_lib.ptr(d["go"]), _lib.ptr(d["gs"]), *[_lib.ptr(t) for t in i],
-                                         _lib.ptr(d["ckpt"]), *[_lib.ptr(t) for t in g], B, T, D, K, C, code,
-                                         flags, _lib.ptr(d["ws"]), ws_bytes, stream))
+        _lib.check(lfw_backward(_lib.ptr(d["go"]), _lib.ptr(d["gs"]), *[_lib.ptr(t) for t in i],
+                                _lib.ptr(d["ckpt"]), *[_lib.ptr(t) for t in g], *dims, C, code,
+                                flags, _lib.ptr(d["ws"]), ws_bytes, stream))
 
     def step(i):
         d = sets[i % nsets]
@@ -185,7 +194,7 @@ def main():
 
     # the same step through the autograd API (allocations and Python dispatch included)
     autograd = None
-    if backward:
+    if backward and not H:
         from t2fw.functional_lfw import LFWFunction
         os.environ["T2FW_CKPT_INTERVAL"] = str(C)
         leaves = [[t.detach().clone().requires_grad_(True) for t in d["ins"]] for d in sets[:2]]

@@ -13,6 +13,8 @@
  *   lfw_backward  (t2fw/csrc/lfw.cpp:50-96) =
  *     lfw_cuda_backward (lfw_kernel.cu:173-228)
  *     + six einsums (lfw.cpp:84-93)                      t2fw_lfw_backward
+ *   the same with the caller's head-folding copies
+ *     (layout required by lfw.cpp:24-26) absorbed        t2fw_lfw_forward_heads, t2fw_lfw_backward_heads
  *   T=1 use of lfw_forward in generation
  *     (tests/benchmark.py:86-88,104-105)                 t2fw_lfw_step
  *   dfw lfw_forward  (t2fw/csrc/dfw.cpp:27-39,
@@ -115,6 +117,35 @@ int t2fw_lfw_backward(const void *g_out, const void *g_state,
                       int64_t B, int64_t T, int64_t D, int64_t K,
                       int32_t C, int32_t dtype, int32_t flags,
                       void *workspace, size_t workspace_bytes, void *stream);
+
+/*
+ * The same two calls for tensors that keep the head axis next to the channels, as the
+ * projections of an attention-shaped layer produce them:
+ *       x, f, out, g_out, d_x, d_f           [B, T, H, D]
+ *       q, k, f_key, d_q, d_k, d_f_key       [B, T, H, K]
+ *       s0, next_state, g_state, d_s0        [B, H, D, K]
+ *       ckpt                                 [B * H, ceil(T / C), D, K]
+ * Every (batch, head) pair is one recurrence.  The reference takes only the folded,
+ * contiguous [B * H, T, D] layout (checks in t2fw/csrc/lfw.cpp:24-26), which costs its
+ * caller a transposing copy per input and per gradient; here the kernels step over the
+ * head axis themselves.  H = 1 is the folded layout.  The workspace is that of B * H rows
+ * (t2fw_lfw_workspace_bytes(B * H, ...)).  The matrix-core kernels need T * H < 2^24.
+ */
+int t2fw_lfw_forward_heads(const void *x, const void *f, const void *q, const void *k,
+                           const void *f_key, const void *s0,
+                           void *out, void *next_state, void *ckpt,
+                           int64_t B, int64_t T, int64_t H, int64_t D, int64_t K,
+                           int32_t C, int32_t dtype, int32_t flags,
+                           void *workspace, size_t workspace_bytes, void *stream);
+
+int t2fw_lfw_backward_heads(const void *g_out, const void *g_state,
+                            const void *x, const void *f, const void *q, const void *k,
+                            const void *f_key, const void *s0, const void *ckpt,
+                            void *d_x, void *d_f, void *d_q, void *d_k, void *d_f_key,
+                            void *d_s0,
+                            int64_t B, int64_t T, int64_t H, int64_t D, int64_t K,
+                            int32_t C, int32_t dtype, int32_t flags,
+                            void *workspace, size_t workspace_bytes, void *stream);
 
 /*
  * One generation step (T = 1) that may update the state in place

@@ -32,6 +32,8 @@ SIGNATURES = {
     "t2fw_lfw_workspace_bytes": (_sz, [_i64, _i64, _i64, _i64, _i32, _i32, _i32]),
     "t2fw_lfw_forward": (ctypes.c_int, [_vp] * 9 + [_i64] * 4 + [_i32] * 3 + [_vp, _sz, _vp]),
     "t2fw_lfw_backward": (ctypes.c_int, [_vp] * 15 + [_i64] * 4 + [_i32] * 3 + [_vp, _sz, _vp]),
+    "t2fw_lfw_forward_heads": (ctypes.c_int, [_vp] * 9 + [_i64] * 5 + [_i32] * 3 + [_vp, _sz, _vp]),
+    "t2fw_lfw_backward_heads": (ctypes.c_int, [_vp] * 15 + [_i64] * 5 + [_i32] * 3 + [_vp, _sz, _vp]),
     "t2fw_lfw_step": (ctypes.c_int, [_vp] * 8 + [_i64] * 3 + [_i32, _vp]),
     "t2fw_gate_forward": (ctypes.c_int, [_vp] * 4 + [_i64] * 2 + [_i32, _vp]),
     "t2fw_gate_backward": (ctypes.c_int, [_vp] * 6 + [_i64] * 2 + [_i32, _vp]),

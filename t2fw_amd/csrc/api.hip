@@ -109,10 +109,12 @@ size_t t2fw_lfw_workspace_bytes(int64_t B, int64_t T, int64_t D, int64_t K, int3
     return 0;
 }
 
-int t2fw_lfw_forward(const void *x, const void *f, const void *q, const void *k, const void *f_key,
-                     const void *s0, void *out, void *next_state, void *ckpt, int64_t B, int64_t T,
-                     int64_t D, int64_t K, int32_t C, int32_t dtype, int32_t flags, void *workspace,
-                     size_t workspace_bytes, void *stream) {
+// B batch rows; heads = 1: rows are contiguous [T, D|K] slabs, heads = H > 1: row b is head b % H of
+// [B / H, T, H, D|K] tensors (x, f, q, k, f_key, out); states and checkpoints are per row either way
+static int lfw_forward_rows(const void *x, const void *f, const void *q, const void *k, const void *f_key,
+                            const void *s0, void *out, void *next_state, void *ckpt, int64_t B, int64_t T,
+                            int64_t heads, int64_t D, int64_t K, int32_t C, int32_t dtype, int32_t flags,
+                            void *workspace, size_t workspace_bytes, void *stream) {
     const size_t es = elem_size(dtype);
     if (es == 0) return fail(T2FW_ERR_BAD_DTYPE, "unknown dtype code %d", dtype);
     int rc = check_dims(B, T, D, K);
@@ -145,10 +147,11 @@ int t2fw_lfw_forward(const void *x, const void *f, const void *q, const void *k,
     a.row_select = nullptr;
     a.row_select2 = nullptr;
     a.B = B; a.T = T; a.D = D; a.K = K;
+    a.heads = (int32_t)heads;
     a.C = ckpt ? C : 1;
     a.NC = ckpt ? t2fw_lfw_num_ckpt(T, C) : 1;
 
-    if (chunk_shape_ok(D, K, dtype, flags) && (ckpt == nullptr || C % 32 == 0) && T < CHUNK_MAX_T &&
+    if (chunk_shape_ok(D, K, dtype, flags) && (ckpt == nullptr || C % 32 == 0) && T * heads < CHUNK_MAX_T &&
         aligned16({x, f, q, k, f_key, s0, out, next_state, ckpt})) {
         if (workspace == nullptr || workspace_bytes < row_flag_bytes(B))
             return fail(T2FW_ERR_WORKSPACE, "workspace of %zu bytes needed, %zu given", row_flag_bytes(B),
@@ -158,6 +161,7 @@ int t2fw_lfw_forward(const void *x, const void *f, const void *q, const void *k,
         c.out = out; c.next_state = next_state; c.ckpt = ckpt;
         c.row_flags = static_cast<int32_t *>(workspace);
         c.B = B; c.T = T; c.NC = a.NC; c.C = a.C;
+        c.heads = (int32_t)heads;
         const int op = (dtype == T2FW_F16 && (flags & T2FW_FLAG_FP16_OPERANDS)) ? 1 : 0;
         // two workgroups per batch row while that still fits the device in one wave of workgroups
         const int cus = compute_units();
@@ -171,12 +175,35 @@ int t2fw_lfw_forward(const void *x, const void *f, const void *q, const void *k,
     return scan_forward(a, dtype, st);
 }
 
-int t2fw_lfw_backward(const void *g_out, const void *g_state, const void *x, const void *f, const void *q,
-                      const void *k, const void *f_key, const void *s0, const void *ckpt, void *d_x,
-                      void *d_f, void *d_q, void *d_k, void *d_f_key, void *d_s0, int64_t B, int64_t T,
-                      int64_t D, int64_t K, int32_t C, int32_t dtype, int32_t flags, void *workspace,
-                      size_t workspace_bytes, void *stream) {
-    (void)s0;
+static int check_heads(int64_t B, int64_t H) {
+    if (B < 0 || H < 1 || H > 65536) return fail(T2FW_ERR_BAD_SHAPE, "B=%lld must be non-negative and H=%lld in [1, 65536]", (long long)B, (long long)H);
+    if ((long double)B * (long double)H > 4.0e18L) return fail(T2FW_ERR_BAD_SHAPE, "B*H is too large");
+    return T2FW_OK;
+}
+
+int t2fw_lfw_forward(const void *x, const void *f, const void *q, const void *k, const void *f_key,
+                     const void *s0, void *out, void *next_state, void *ckpt, int64_t B, int64_t T,
+                     int64_t D, int64_t K, int32_t C, int32_t dtype, int32_t flags, void *workspace,
+                     size_t workspace_bytes, void *stream) {
+    return lfw_forward_rows(x, f, q, k, f_key, s0, out, next_state, ckpt, B, T, 1, D, K, C, dtype, flags, workspace,
+                            workspace_bytes, stream);
+}
+
+int t2fw_lfw_forward_heads(const void *x, const void *f, const void *q, const void *k, const void *f_key,
+                           const void *s0, void *out, void *next_state, void *ckpt, int64_t B, int64_t T,
+                           int64_t H, int64_t D, int64_t K, int32_t C, int32_t dtype, int32_t flags,
+                           void *workspace, size_t workspace_bytes, void *stream) {
+    const int rc = check_heads(B, H);
+    if (rc) return rc;
+    return lfw_forward_rows(x, f, q, k, f_key, s0, out, next_state, ckpt, B * H, T, H, D, K, C, dtype, flags, workspace,
+                            workspace_bytes, stream);
+}
+
+static int lfw_backward_rows(const void *g_out, const void *g_state, const void *x, const void *f, const void *q,
+                             const void *k, const void *f_key, const void *ckpt, void *d_x, void *d_f, void *d_q,
+                             void *d_k, void *d_f_key, void *d_s0, int64_t B, int64_t T, int64_t heads, int64_t D,
+                             int64_t K, int32_t C, int32_t dtype, int32_t flags, void *workspace,
+                             size_t workspace_bytes, void *stream) {
     const size_t es = elem_size(dtype);
     if (es == 0) return fail(T2FW_ERR_BAD_DTYPE, "unknown dtype code %d", dtype);
     int rc = check_dims(B, T, D, K);
@@ -204,9 +231,10 @@ int t2fw_lfw_backward(const void *g_out, const void *g_state, const void *x, con
     a.d_x = d_x; a.d_f = d_f; a.d_q = d_q; a.d_k = d_k; a.d_f_key = d_f_key; a.d_s0 = d_s0;
     a.row_select = nullptr;
     a.B = B; a.T = T; a.D = D; a.K = K; a.C = C;
+    a.heads = (int32_t)heads;
     a.NC = t2fw_lfw_num_ckpt(T, C);
 
-    if (chunk_shape_ok(D, K, dtype, flags) && (C == 32 || C == 64) && T < CHUNK_MAX_T &&
+    if (chunk_shape_ok(D, K, dtype, flags) && (C == 32 || C == 64) && T * heads < CHUNK_MAX_T &&
         aligned16({g_out, g_state, x, f, q, k, f_key, ckpt, d_x, d_f, d_q, d_k, d_f_key, d_s0})) {
         if (workspace == nullptr || workspace_bytes < row_flag_bytes(B))
             return fail(T2FW_ERR_WORKSPACE, "workspace of %zu bytes needed, %zu given", row_flag_bytes(B),
@@ -216,12 +244,35 @@ int t2fw_lfw_backward(const void *g_out, const void *g_state, const void *x, con
         c.d_x = d_x; c.d_f = d_f; c.d_q = d_q; c.d_k = d_k; c.d_f_key = d_f_key; c.d_s0 = d_s0;
         c.row_flags = static_cast<int32_t *>(workspace);
         c.B = B; c.T = T; c.NC = a.NC; c.C = C;
+        c.heads = (int32_t)heads;
         const int op = (dtype == T2FW_F16 && (flags & T2FW_FLAG_FP16_OPERANDS)) ? 1 : 0;
         if ((rc = chunk_backward(c, dtype, op, st))) return rc;
         a.row_select = c.row_flags;      // rows the chunked form could not take
         if (flags & T2FW_FLAG_NO_FIXUP) return T2FW_OK;
     }
     return scan_backward(a, dtype, st);
+}
+
+int t2fw_lfw_backward(const void *g_out, const void *g_state, const void *x, const void *f, const void *q,
+                      const void *k, const void *f_key, const void *s0, const void *ckpt, void *d_x,
+                      void *d_f, void *d_q, void *d_k, void *d_f_key, void *d_s0, int64_t B, int64_t T,
+                      int64_t D, int64_t K, int32_t C, int32_t dtype, int32_t flags, void *workspace,
+                      size_t workspace_bytes, void *stream) {
+    (void)s0;
+    return lfw_backward_rows(g_out, g_state, x, f, q, k, f_key, ckpt, d_x, d_f, d_q, d_k, d_f_key, d_s0, B, T, 1, D, K, C,
+                             dtype, flags, workspace, workspace_bytes, stream);
+}
+
+int t2fw_lfw_backward_heads(const void *g_out, const void *g_state, const void *x, const void *f, const void *q,
+                            const void *k, const void *f_key, const void *s0, const void *ckpt, void *d_x, void *d_f,
+                            void *d_q, void *d_k, void *d_f_key, void *d_s0, int64_t B, int64_t T, int64_t H,
+                            int64_t D, int64_t K, int32_t C, int32_t dtype, int32_t flags, void *workspace,
+                            size_t workspace_bytes, void *stream) {
+    (void)s0;
+    const int rc = check_heads(B, H);
+    if (rc) return rc;
+    return lfw_backward_rows(g_out, g_state, x, f, q, k, f_key, ckpt, d_x, d_f, d_q, d_k, d_f_key, d_s0, B * H, T, H, D, K,
+                             C, dtype, flags, workspace, workspace_bytes, stream);
 }
 
 int t2fw_lfw_step(const void *x, const void *f, const void *q, const void *k, const void *f_key, const void *s0,

@@ -21,6 +21,15 @@ int fail(int code, const char *fmt, ...);   // records the message, returns code
 int check_hip(hipError_t e, const char *what);
 
 // ----------------------------------------------------------------------------------
+// layout of the [.., T, .., width] tensors: batch rows are either contiguous [T, width] slabs
+// (heads = 1) or the heads of a [B / heads, T, heads, width] tensor.  Token t of row b sits at
+// element (row_first_token(b, T, heads) + t * heads) * width.
+// ----------------------------------------------------------------------------------
+__host__ __device__ inline int64_t row_first_token(int64_t b, int64_t T, int64_t heads) {
+    return heads == 1 ? b * T : (b / heads) * T * heads + b % heads;
+}
+
+// ----------------------------------------------------------------------------------
 // element types: IO is what lives in HBM, Acc is what the recurrence is carried in
 // ----------------------------------------------------------------------------------
 template <typename IO> struct AccOf { using type = float; };

@@ -28,6 +28,7 @@ struct ChunkFwdArgs {
     int32_t *row_flags;                // [2 * chunk_rows_padded(B)]: set to 1 for rows the exact kernels must redo
     int64_t B, T, NC;
     int32_t C;                         // checkpoint interval, multiple of 32
+    int32_t heads;                     // 1: rows are [T, 64] slabs; H > 1: row b is head b % H of a [B / H, T, H, 64] tensor
 };
 
 struct ChunkBwdArgs {
@@ -36,6 +37,7 @@ struct ChunkBwdArgs {
     int32_t *row_flags;                // as for the forward
     int64_t B, T, NC;
     int32_t C;
+    int32_t heads;                     // as for the forward (inputs, g_out and the five [.., T, .., 64] gradients)
 };
 
 // Kernels that split a batch row over two workgroups index them as half * chunk_rows_padded(B) + row
@@ -46,7 +48,7 @@ __host__ __device__ inline int64_t chunk_rows_padded(int64_t B) { return (B + 7)
 int chunk_forward(const ChunkFwdArgs &a, int dtype, int op, bool split, hipStream_t stream);
 // two workgroups per batch row (one per side of the state)
 int chunk_backward(const ChunkBwdArgs &a, int dtype, int op, hipStream_t stream);
-constexpr int64_t CHUNK_MAX_T = 1 << 24;      // the forward and the split backward kernel address a batch row with 32-bit offsets
+constexpr int64_t CHUNK_MAX_T = 1 << 24;      // the kernels address a batch row with 32-bit offsets: T * heads must stay below this
 
 #if defined(__HIPCC__)
 

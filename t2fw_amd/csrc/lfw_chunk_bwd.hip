@@ -159,31 +159,69 @@ static_assert(SplitSchedule<4>::PER_CHUNK <= 8, "a chunk's stages must fit the 6
 // 24 two-byte loads, coalesced over the wave's 64 channels.  They go straight to registers,
 // two stages ahead of their use: the block's first token of an array is a scalar base, the
 // lane's channel and token half a constant vector offset, the token inside the half an
-// immediate one.
+// immediate one (for rows that are heads of a [B, T, H, 64] tensor see TokenMap).
 struct RawSet {
     u16 gown[8], goth[8], val[8];
 };
 
-// gate, val: wave-uniform addresses of the block's first token; voff_own / voff_oth: byte offsets of
-// (own / other token half, channel) inside a block
-__device__ __forceinline__ void raw_issue(RawSet &r, const u16 *gate, const u16 *val, u32 voff_own, u32 voff_oth) {
-    auto at = [&](const u16 *base, u32 voff, int t) -> u16 {
-        return *reinterpret_cast<const u16 *>(reinterpret_cast<const unsigned char *>(base + t * CH_N) + voff);
-    };
+// Where the sixteen tokens of a block are, seen from a prep lane.  Consecutive tokens are ts elements
+// apart.  HEADS = false: ts = 64; the token half and the channel make up a constant vector offset
+// (voff_own / voff_oth), the token inside the half is an immediate one.  HEADS = true: ts is a
+// run-time multiple of 64; the token half moves the scalar base (shift_own / shift_oth elements) and
+// tok_off[t] = 2 * (channel + t * ts) is the vector offset of token t of a half.
+template <bool HEADS> struct TokenMap {
+    u32 ts, voff_own, voff_oth, shift_own, shift_oth, tok_off[8];
+    __device__ __forceinline__ TokenMap(u32 ts_, int h, int c) {
+        ts = HEADS ? ts_ : (u32)CH_N;
+        voff_own = (u32)(8 * h * CH_N + c) * 2u;
+        voff_oth = (u32)(8 * (1 - h) * CH_N + c) * 2u;
+        shift_own = 8u * (u32)h * ts;
+        shift_oth = 8u * (u32)(1 - h) * ts;
 #pragma unroll
-    for (int t = 0; t < 8; ++t) r.goth[t] = at(gate, voff_oth, t);
+        for (int t = 0; t < 8; ++t) {
+            tok_off[t] = 2u * ((u32)c + (u32)t * ts);
+        }
+    }
+};
+
+// gate, val: wave-uniform addresses of the block's first token
+template <bool HEADS>
+__device__ __forceinline__ void raw_issue(RawSet &r, const u16 *gate, const u16 *val, TokenMap<HEADS> &m) {
+    if constexpr (!HEADS) {
+        auto at = [&](const u16 *base, u32 voff, int t) -> u16 {
+            return *reinterpret_cast<const u16 *>(reinterpret_cast<const unsigned char *>(base + t * CH_N) + voff);
+        };
 #pragma unroll
-    for (int t = 0; t < 8; ++t) r.gown[t] = at(gate, voff_own, t);
+        for (int t = 0; t < 8; ++t) r.goth[t] = at(gate, m.voff_oth, t);
 #pragma unroll
-    for (int t = 0; t < 8; ++t) r.val[t] = at(val, voff_own, t);
+        for (int t = 0; t < 8; ++t) r.gown[t] = at(gate, m.voff_own, t);
+#pragma unroll
+        for (int t = 0; t < 8; ++t) r.val[t] = at(val, m.voff_own, t);
+    } else {
+        // The offsets are made opaque at every use: they then stay in eight 32-bit registers (no
+        // re-derivation from the channel, no widened copies hoisted out of the loops), which is the
+        // form the scalar-base addressing mode of the loads takes.
+#pragma unroll
+        for (int t = 0; t < 8; ++t) asm volatile("" : "+v"(m.tok_off[t]));
+        auto at = [&](const u16 *base, int t) -> u16 {
+            return *reinterpret_cast<const u16 *>(reinterpret_cast<const unsigned char *>(base) + m.tok_off[t]);
+        };
+        const u16 *const go = gate + m.shift_own, *const gx = gate + m.shift_oth, *const vo = val + m.shift_own;
+#pragma unroll
+        for (int t = 0; t < 8; ++t) r.goth[t] = at(gx, t);
+#pragma unroll
+        for (int t = 0; t < 8; ++t) r.gown[t] = at(go, t);
+#pragma unroll
+        for (int t = 0; t < 8; ++t) r.val[t] = at(vo, t);
+    }
 }
 
 // The same for a block that reaches past the end of the sequence (T % 16 != 0, last chunk only):
 // tokens past the end are read from the last one, with the same number of loads, and replaced by
 // raw_patch_tail when the set is taken.  row_gate, row_val: token 0 of the batch row.
 __device__ __forceinline__ void raw_issue_tail(RawSet &r, const u16 *row_gate, const u16 *row_val, int tok_own,
-                                               int tok_oth, int T, int c) {
-    auto at = [&](const u16 *base, int tok) -> u16 { return base[(u32)min(tok, T - 1) * CH_N + c]; };
+                                               int tok_oth, int T, int c, u32 ts) {
+    auto at = [&](const u16 *base, int tok) -> u16 { return base[(u32)min(tok, T - 1) * ts + c]; };
 #pragma unroll
     for (int t = 0; t < 8; ++t) r.goth[t] = at(row_gate, tok_oth + t);
 #pragma unroll
@@ -340,7 +378,7 @@ __device__ __forceinline__ void prep_r(const RawSet &r, unsigned char *stage, in
     write_cm8(stage, 2 * j + own, c, 8 * h, pack8<OPE>(hat));
 }
 
-template <typename IOE, typename OPE, int NB>
+template <typename IOE, typename OPE, int NB, bool HEADS>
 __device__ __forceinline__ void split_prep_waves(const ChunkBwdArgs &p, unsigned char *smem, int tid, int64_t b,
                                                  int side) {
     const int pw = __builtin_amdgcn_readfirstlane(tid >> 6), c = tid & 63;
@@ -349,8 +387,8 @@ __device__ __forceinline__ void split_prep_waves(const ChunkBwdArgs &p, unsigned
     const int role = (h ? (pw ^ 1) : pw) & 3;
     // R stages: (block of the pair, side, token half)
     const int rj = (pw >> 1) & 1, rown = pw & 1;
-    const int T = (int)p.T;                              // the launcher admits T < 2^24 only
-    const int64_t row_off = b * p.T * CH_N;
+    const int T = (int)p.T;                              // the launcher admits T * heads < 2^24 only
+    const int64_t row_off = row_first_token(b, p.T, HEADS ? p.heads : 1) * CH_N;
     // this batch row of: other gate, other value, own gate, own value, other adjoint, own adjoint
     const u16 *const x = reinterpret_cast<const u16 *>(p.x) + row_off, *const f = reinterpret_cast<const u16 *>(p.f) + row_off;
     const u16 *const g = reinterpret_cast<const u16 *>(p.g_out) + row_off, *const k = reinterpret_cast<const u16 *>(p.k) + row_off;
@@ -365,7 +403,8 @@ __device__ __forceinline__ void split_prep_waves(const ChunkBwdArgs &p, unsigned
     const SplitSchedule<NB> sched(p.T, p.NC, p.C);
     u32 bad = 0;
 
-    const u32 voff_own = (u32)(8 * h * CH_N + c) * 2u, voff_oth = (u32)(8 * (1 - h) * CH_N + c) * 2u;
+    TokenMap<HEADS> tmap(HEADS ? (u32)p.heads * CH_N : (u32)CH_N, h, c);
+    const u32 ts = tmap.ts;                              // elements between consecutive tokens
     // first token of the block this wave works on in stage st (R stages cover a pair of blocks)
     auto block_tok = [&](int st) -> int { return (st >> 1) + ((st & 1) ? 0 : rj * CH_L); };
     auto issue = [&](RawSet &r, int st) {          // raw inputs of stage st (wave-uniform) -> registers
@@ -373,9 +412,9 @@ __device__ __forceinline__ void split_prep_waves(const ChunkBwdArgs &p, unsigned
         const int tok = block_tok(st);
         const u16 *const gate = bmode ? b_gate : r_gate, *const val = bmode ? b_val : r_val;
         if (tok + CH_L <= T)
-            raw_issue(r, gate + (u32)tok * CH_N, val + (u32)tok * CH_N, voff_own, voff_oth);
+            raw_issue<HEADS>(r, gate + (u32)tok * ts, val + (u32)tok * ts, tmap);
         else        // the block reaches past the end (or, second block of the last R pair, lies past it)
-            raw_issue_tail(r, gate, val, tok + 8 * h, tok + 8 * (1 - h), T, c);
+            raw_issue_tail(r, gate, val, tok + 8 * h, tok + 8 * (1 - h), T, c, ts);
     };
     // Three register sets rotate: the tiles of stage s are built from `cur`, which was loaded two
     // stages ago, while `refill` (used up in the stage before) takes the raw inputs of stage s + 2.
@@ -445,15 +484,15 @@ __device__ __forceinline__ void split_prep_waves(const ChunkBwdArgs &p, unsigned
     // chunk: that chunk again, never used).
     constexpr int PER = (int)SplitSchedule<NB>::PER_CHUNK, NR = NB / 2;
     static_assert(PER % 3 == 0, "a chunk must take a whole number of register-set triples");
-    const u16 *const r_gate_w = r_gate + rj * CH_L * CH_N, *const r_val_w = r_val + rj * CH_L * CH_N;
+    const u16 *const r_gate_w = r_gate + (u32)(rj * CH_L) * ts, *const r_val_w = r_val + (u32)(rj * CH_L) * ts;
     auto issue_at = [&](RawSet &r, int chunk_tok, auto pos_c) {
         constexpr int POS = decltype(pos_c)::value;
         if constexpr (POS < NR) {
-            const u32 e = (u32)(chunk_tok + 2 * POS * CH_L) * CH_N;
-            raw_issue(r, r_gate_w + e, r_val_w + e, voff_own, voff_oth);
+            const u32 e = (u32)(chunk_tok + 2 * POS * CH_L) * ts;
+            raw_issue<HEADS>(r, r_gate_w + e, r_val_w + e, tmap);
         } else {
-            const u32 e = (u32)(chunk_tok + (NB - 1 - (POS - NR)) * CH_L) * CH_N;
-            raw_issue(r, b_gate + e, b_val + e, voff_own, voff_oth);
+            const u32 e = (u32)(chunk_tok + (NB - 1 - (POS - NR)) * CH_L) * ts;
+            raw_issue<HEADS>(r, b_gate + e, b_val + e, tmap);
         }
     };
     auto prepare_at = [&](const RawSet &cur, RawSet &refill, int chunk_tok, int below_tok, auto pos_c) {
@@ -491,7 +530,7 @@ __device__ __forceinline__ void split_prep_waves(const ChunkBwdArgs &p, unsigned
     PHASE_END(4 + (tid >> 6));
 }
 
-template <typename IOE, typename OPE, int NB>
+template <typename IOE, typename OPE, int NB, bool HEADS>
 __device__ __forceinline__ void split_matrix_waves(const ChunkBwdArgs &p, unsigned char *smem, int tid, int64_t b,
                                                    int side) {
     const int w = tid >> 6, l = tid & 63, r = l & 15, g = l >> 4;
@@ -502,9 +541,11 @@ __device__ __forceinline__ void split_matrix_waves(const ChunkBwdArgs &p, unsign
     const u16 *ckpt = reinterpret_cast<const u16 *>(p.ckpt) + b * NC * (CH_N * CH_N);
     const int nb_last = (int)((p.T - (NC - 1) * C + CH_L - 1) / CH_L);
     // this batch row of the gradients this side writes
-    u16 *const d_val = reinterpret_cast<u16 *>(side == 0 ? p.d_x : p.d_k) + b * p.T * CH_N;
-    u16 *const d_gate = reinterpret_cast<u16 *>(side == 0 ? p.d_f : p.d_f_key) + b * p.T * CH_N;
-    u16 *const d_adj = reinterpret_cast<u16 *>(p.d_q) + b * p.T * CH_N;
+    const int64_t row_off = row_first_token(b, p.T, HEADS ? p.heads : 1) * CH_N;
+    const u32 ts = HEADS ? (u32)p.heads * CH_N : (u32)CH_N;       // elements between consecutive tokens
+    u16 *const d_val = reinterpret_cast<u16 *>(side == 0 ? p.d_x : p.d_k) + row_off;
+    u16 *const d_gate = reinterpret_cast<u16 *>(side == 0 ? p.d_f : p.d_f_key) + row_off;
+    u16 *const d_adj = reinterpret_cast<u16 *>(p.d_q) + row_off;
 
     // S[j][i], G[j][i]: own channel ch, other channel 16j + 4g + i
     floatx4 S[4], G[4];
@@ -657,16 +698,16 @@ __device__ __forceinline__ void split_matrix_waves(const ChunkBwdArgs &p, unsign
                     // 16 lanes write 32 contiguous bytes of a token row; the four waves complete the row.
                     // Only the last block of the sequence can reach past its end.
                     const int tg = (int)chunk * C + i * CH_L + 4 * g;         // this lane's first token
-                    const u32 go = (u32)tg * CH_N + (u32)ch;
+                    const u32 go = (u32)tg * ts + (u32)ch;
                     float ppv[4] = {0.f, 0.f, 0.f, 0.f};
                     if (side == 1) {
                         const float4 pp = *reinterpret_cast<const float4 *>(cf + F_PP * (CF_TILE / 4));
                         ppv[0] = pp.x; ppv[1] = pp.y; ppv[2] = pp.z; ppv[3] = pp.w;
                     }
                     auto store = [&](int ii) {
-                        d_val[go + ii * CH_N] = cvt1<IOE>(ipv[ii] * (va[ii] + asv[ii] * pd[ii]));
-                        d_gate[go + ii * CH_N] = cvt1<IOE>(du[ii] * rgv[ii]);
-                        if (side == 1) d_adj[go + ii * CH_N] = cvt1<IOE>(ppv[ii] * (oa[ii] + vtv[ii] * pd[ii]));
+                        d_val[go + ii * ts] = cvt1<IOE>(ipv[ii] * (va[ii] + asv[ii] * pd[ii]));
+                        d_gate[go + ii * ts] = cvt1<IOE>(du[ii] * rgv[ii]);
+                        if (side == 1) d_adj[go + ii * ts] = cvt1<IOE>(ppv[ii] * (oa[ii] + vtv[ii] * pd[ii]));
                     };
                     if ((int)chunk * C + (i + 1) * CH_L <= T) {
 #pragma unroll
@@ -691,7 +732,7 @@ __device__ __forceinline__ void split_matrix_waves(const ChunkBwdArgs &p, unsign
     PHASE_END(tid >> 6);
 }
 
-template <typename IOE, typename OPE, int NB>
+template <typename IOE, typename OPE, int NB, bool HEADS>
 __global__ __launch_bounds__(SP_THREADS) void lfw_bwd_chunk_kernel(ChunkBwdArgs p, int rows_padded) {
     extern __shared__ __align__(16) unsigned char smem[];
     const int tid = threadIdx.x;
@@ -702,28 +743,29 @@ __global__ __launch_bounds__(SP_THREADS) void lfw_bwd_chunk_kernel(ChunkBwdArgs 
     if (b >= p.B) return;
     // both branches execute exactly 2 + (number of stages) workgroup barriers
     if (tid < 256)
-        split_matrix_waves<IOE, OPE, NB>(p, smem, tid, b, side);
+        split_matrix_waves<IOE, OPE, NB, HEADS>(p, smem, tid, b, side);
     else
-        split_prep_waves<IOE, OPE, NB>(p, smem, tid - 256, b, side);
+        split_prep_waves<IOE, OPE, NB, HEADS>(p, smem, tid - 256, b, side);
 }
 
-template <typename IOE, typename OPE, int NB> int launch(const ChunkBwdArgs &a, hipStream_t stream) {
-    auto kern = lfw_bwd_chunk_kernel<IOE, OPE, NB>;
+template <typename IOE, typename OPE, int NB, bool HEADS> int launch(const ChunkBwdArgs &a, hipStream_t stream) {
+    auto kern = lfw_bwd_chunk_kernel<IOE, OPE, NB, HEADS>;
     // more than 64 KB of dynamic LDS has to be enabled per function (and per device)
     int rc = check_hip(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, SP_SMEM),
                        "hipFuncSetAttribute(backward chunk kernel)");
     if (rc) return rc;
     if (a.B > 0x1fffffffLL) return fail(T2FW_ERR_UNSUPPORTED, "B=%lld is too large", (long long)a.B);
-    if (a.T >= CHUNK_MAX_T) return fail(T2FW_ERR_UNSUPPORTED, "T=%lld is too long for 32-bit row offsets", (long long)a.T);
+    if (a.heads < 1 || a.T * a.heads >= CHUNK_MAX_T)
+        return fail(T2FW_ERR_UNSUPPORTED, "T=%lld with %d heads is too long for 32-bit row offsets", (long long)a.T, a.heads);
     const int rows_padded = (int)((a.B + 7) / 8 * 8);
     hipLaunchKernelGGL(kern, dim3(2u * (unsigned)rows_padded), dim3(SP_THREADS), SP_SMEM, stream, a, rows_padded);
     return check_hip(hipGetLastError(), "lfw_bwd_chunk_kernel launch");
 }
 
 template <typename IOE, typename OPE> int by_nb(const ChunkBwdArgs &a, hipStream_t stream) {
-    if (a.C == 64) return launch<IOE, OPE, 4>(a, stream);
-    if (a.C == 32) return launch<IOE, OPE, 2>(a, stream);
+    if (a.C == 64) return a.heads == 1 ? launch<IOE, OPE, 4, false>(a, stream) : launch<IOE, OPE, 4, true>(a, stream);
+    if (a.C == 32) return a.heads == 1 ? launch<IOE, OPE, 2, false>(a, stream) : launch<IOE, OPE, 2, true>(a, stream);
     return fail(T2FW_ERR_UNSUPPORTED, "the chunked backward kernel takes checkpoint intervals 32 or 64");
 }
 

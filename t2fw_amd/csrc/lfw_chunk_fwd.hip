@@ -57,23 +57,43 @@ template <int NV> struct RawSet {
 
 // gate, val0, val1 (NV = 2 only): wave-uniform addresses of token 0 of the batch row; tok_own / tok_oth:
 // first of the eight own / other tokens; lane_bytes = 2 * channel.  All sixteen tokens must exist.
-template <int NV>
+// Consecutive tokens are ts elements apart.  HEADS = false: ts = 64, the token inside the half is an
+// immediate offset.  HEADS = true: ts is a run-time multiple of 64; tok_blk is the block's first
+// token (wave-uniform) and own_off[t] / oth_off[t] are the lane's byte offsets of its own / other
+// eight tokens from there (channel included; kept in registers for the whole sequence).
+template <int NV, bool HEADS>
 __device__ __forceinline__ void raw_issue(RawSet<NV> &r, const u16 *gate, const u16 *val0, const u16 *val1, int tok_own,
-                                          int tok_oth, u32 lane_bytes) {
+                                          int tok_oth, u32 lane_bytes, int tok_blk, u32 ts, const u32 (&own_off)[8],
+                                          const u32 (&oth_off)[8]) {
     const u16 *const val[2] = {val0, val1};
-    auto at = [&](const u16 *base, int tok) -> const u16 * {
-        return reinterpret_cast<const u16 *>(reinterpret_cast<const unsigned char *>(base + (u32)tok * CH_N) + lane_bytes);
-    };
-    const u16 *go = at(gate, tok_own), *gx = at(gate, tok_oth);
+    if constexpr (!HEADS) {
+        auto at = [&](const u16 *base, int tok) -> const u16 * {
+            return reinterpret_cast<const u16 *>(reinterpret_cast<const unsigned char *>(base + (u32)tok * CH_N) + lane_bytes);
+        };
+        const u16 *go = at(gate, tok_own), *gx = at(gate, tok_oth);
 #pragma unroll
-    for (int t = 0; t < 8; ++t) r.goth[t] = gx[t * CH_N];
+        for (int t = 0; t < 8; ++t) r.goth[t] = gx[t * CH_N];
 #pragma unroll
-    for (int t = 0; t < 8; ++t) r.gown[t] = go[t * CH_N];
+        for (int t = 0; t < 8; ++t) r.gown[t] = go[t * CH_N];
 #pragma unroll
-    for (int a = 0; a < NV; ++a) {
-        const u16 *va = at(val[a], tok_own);
+        for (int a = 0; a < NV; ++a) {
+            const u16 *va = at(val[a], tok_own);
 #pragma unroll
-        for (int t = 0; t < 8; ++t) r.val[a][t] = va[t * CH_N];
+            for (int t = 0; t < 8; ++t) r.val[a][t] = va[t * CH_N];
+        }
+    } else {
+        auto ld = [&](const u16 *base, u32 off) -> u16 {
+            return *reinterpret_cast<const u16 *>(reinterpret_cast<const unsigned char *>(base + (u32)tok_blk * ts) + off);
+        };
+#pragma unroll
+        for (int t = 0; t < 8; ++t) r.goth[t] = ld(gate, oth_off[t]);
+#pragma unroll
+        for (int t = 0; t < 8; ++t) r.gown[t] = ld(gate, own_off[t]);
+#pragma unroll
+        for (int a = 0; a < NV; ++a) {
+#pragma unroll
+            for (int t = 0; t < 8; ++t) r.val[a][t] = ld(val[a], own_off[t]);
+        }
     }
 }
 
@@ -81,10 +101,10 @@ __device__ __forceinline__ void raw_issue(RawSet<NV> &r, const u16 *gate, const 
 // one (and replaced by raw_take_tail).
 template <int NV>
 __device__ __forceinline__ void raw_issue_tail(RawSet<NV> &r, const u16 *gate, const u16 *val0, const u16 *val1,
-                                               int tok_own, int tok_oth, int T, u32 lane_bytes) {
+                                               int tok_own, int tok_oth, int T, u32 lane_bytes, u32 ts) {
     const u16 *const val[2] = {val0, val1};
     auto at = [&](const u16 *base, int tok) -> const u16 * {
-        return reinterpret_cast<const u16 *>(reinterpret_cast<const unsigned char *>(base + (u32)min(tok, T - 1) * CH_N) +
+        return reinterpret_cast<const u16 *>(reinterpret_cast<const unsigned char *>(base + (u32)min(tok, T - 1) * ts) +
                                              lane_bytes);
     };
 #pragma unroll
@@ -198,18 +218,25 @@ __device__ __forceinline__ float scale_half(const RawF<NV> &f, int h, float (&pr
 // c: this lane's channel; hh: block of the step (wave-uniform); h: token half (wave-uniform, or
 // per lane when a wave covers both halves of 32 channels); flag_slot: where this workgroup
 // reports rows the chunked form cannot take.
-template <typename IOE, typename OPE, bool KEY>
+template <typename IOE, typename OPE, bool KEY, bool HEADS>
 __device__ __forceinline__ void fwd_prep_side(const ChunkFwdArgs &p, unsigned char *smem, int tid, int64_t b, int c,
                                               int hh, int h, int64_t flag_slot) {
     constexpr int NV = KEY ? 2 : 1;
     const int T = (int)p.T;                                // the launcher admits T < 2^24 only
-    const int64_t row_off = b * p.T * CH_N;
+    const int64_t row_off = row_first_token(b, p.T, HEADS ? p.heads : 1) * CH_N;
+    const u32 ts = HEADS ? (u32)p.heads * CH_N : (u32)CH_N;        // elements between consecutive tokens
     const u16 *const gate = reinterpret_cast<const u16 *>(KEY ? p.f_key : p.f) + row_off;
     const u16 *const val0 = reinterpret_cast<const u16 *>(KEY ? p.k : p.x) + row_off;
     const u16 *const val1 = reinterpret_cast<const u16 *>(p.q) + row_off;      // key side only
     const int nfull = T / CH_STEP;                         // full 32-token steps; a partial one may follow
     const int off_own = CH_L * hh + 8 * h, off_oth = CH_L * hh + 8 * (1 - h);   // inside a step
     const u32 lane_bytes = 2u * (u32)c;
+    u32 own_off[8], oth_off[8];                            // HEADS only: vector offsets of the sixteen tokens
+#pragma unroll
+    for (int t = 0; t < 8; ++t) {
+        own_off[t] = HEADS ? lane_bytes + 2u * (u32)(8 * h + t) * ts : 0u;
+        oth_off[t] = HEADS ? lane_bytes + 2u * (u32)(8 * (1 - h) + t) * ts : 0u;
+    }
     u32 bad = 0;
 
     // this wave's share of the operand tiles of step n
@@ -237,7 +264,8 @@ __device__ __forceinline__ void fwd_prep_side(const ChunkFwdArgs &p, unsigned ch
     };
     auto issue = [&](RawSet<NV> &r, int step, u32 lb) {
         const int st = min(step, nfull - 1);       // past the last full step: that step again (never used)
-        raw_issue<NV>(r, gate, val0, val1, st * CH_STEP + off_own, st * CH_STEP + off_oth, lb);
+        raw_issue<NV, HEADS>(r, gate, val0, val1, st * CH_STEP + off_own, st * CH_STEP + off_oth, lb,
+                             st * CH_STEP + CH_L * hh, ts, own_off, oth_off);
     };
     // builds the tiles of full step n, which r holds; r then takes step n + 2
     auto prepare = [&](RawSet<NV> &r, int n) {
@@ -259,6 +287,16 @@ __device__ __forceinline__ void fwd_prep_side(const ChunkFwdArgs &p, unsigned ch
                            "v"(f.gown[6]), "v"(f.gown[7]), "v"(f.val[0][0]), "v"(f.val[0][1]), "v"(f.val[0][2]),
                            "v"(f.val[0][3]), "v"(f.val[0][4]), "v"(f.val[0][5]), "v"(f.val[0][6]), "v"(f.val[0][7]),
                            "v"(f.goth_prod), "v"(f.bad));
+        }
+        if constexpr (HEADS) {      // the token offsets carry the same dependency (and stay in registers)
+            asm volatile(""
+                         : "+v"(own_off[0]), "+v"(own_off[1]), "+v"(own_off[2]), "+v"(own_off[3]), "+v"(own_off[4]),
+                           "+v"(own_off[5]), "+v"(own_off[6]), "+v"(own_off[7])
+                         : "v"(lb));
+            asm volatile(""
+                         : "+v"(oth_off[0]), "+v"(oth_off[1]), "+v"(oth_off[2]), "+v"(oth_off[3]), "+v"(oth_off[4]),
+                           "+v"(oth_off[5]), "+v"(oth_off[6]), "+v"(oth_off[7])
+                         : "v"(lb));
         }
         issue(r, n + 2, lb);
         build(f, n);
@@ -297,7 +335,7 @@ __device__ __forceinline__ void fwd_prep_side(const ChunkFwdArgs &p, unsigned ch
     if (nfull * CH_STEP < T) {      // the partial step at the end
         RawSet<NV> r;
         const int t_own = nfull * CH_STEP + off_own, t_oth = nfull * CH_STEP + off_oth;
-        raw_issue_tail<NV>(r, gate, val0, val1, t_own, t_oth, T, lane_bytes);
+        raw_issue_tail<NV>(r, gate, val0, val1, t_own, t_oth, T, lane_bytes, ts);
         build(raw_take_tail<IOE, NV>(r, t_own, t_oth, T), nfull);
         __syncthreads();
     }
@@ -317,14 +355,15 @@ __device__ __forceinline__ void store_state(const floatx4 (&S)[4], u16 *dst, int
         *reinterpret_cast<uint2 *>(dst + d * CH_N + 16 * j + 4 * g) = pack4<IOE>(S[j]);
 }
 
-template <typename IOE, typename OPE>
+template <typename IOE, typename OPE, bool HEADS>
 __device__ __forceinline__ void fwd_matrix_waves(const ChunkFwdArgs &p, unsigned char *smem, int tid, int64_t b,
                                                  int dbase, int64_t flag_slot, bool clear_other_slot) {
     const int w = tid >> 6, l = tid & 63, r = l & 15, g = l >> 4;
     const int d = dbase + 16 * w + r;          // this lane's state row (value channel)
     const int T = (int)p.T;
     u16 *ckpt = reinterpret_cast<u16 *>(p.ckpt);
-    u16 *const out = reinterpret_cast<u16 *>(p.out) + b * p.T * CH_N;
+    u16 *const out = reinterpret_cast<u16 *>(p.out) + row_first_token(b, p.T, HEADS ? p.heads : 1) * CH_N;
+    const u32 ts = HEADS ? (u32)p.heads * CH_N : (u32)CH_N;        // elements between consecutive tokens
     // S[j][i]: value channel d, key channel 16j + 4g + i
     floatx4 S[4];
     {
@@ -390,14 +429,14 @@ __device__ __forceinline__ void fwd_matrix_waves(const ChunkFwdArgs &p, unsigned
             const float asv[4] = {as.x, as.y, as.z, as.w};
             // 16 lanes write 32 contiguous bytes of a token row; the four waves complete the row
             const int tg = n * CH_STEP + tok0 + 4 * g;
-            const u32 go = (u32)tg * CH_N + (u32)d;
+            const u32 go = (u32)tg * ts + (u32)d;
             if ((n + 1) * CH_STEP <= T) {
 #pragma unroll
-                for (int i = 0; i < 4; ++i) out[go + i * CH_N] = cvt1<IOE>((o[i] + oi[i]) * asv[i]);
+                for (int i = 0; i < 4; ++i) out[go + i * ts] = cvt1<IOE>((o[i] + oi[i]) * asv[i]);
             } else {
 #pragma unroll
                 for (int i = 0; i < 4; ++i)
-                    if (tg + i < T) out[go + i * CH_N] = cvt1<IOE>((o[i] + oi[i]) * asv[i]);
+                    if (tg + i < T) out[go + i * ts] = cvt1<IOE>((o[i] + oi[i]) * asv[i]);
             }
             // S_L = (a_L (x) b_L) * S0 + sum_s xh_s (x) kh_s
             const float aL = AL[hh * CH_N + d];
@@ -418,22 +457,22 @@ __device__ __forceinline__ void fwd_matrix_waves(const ChunkFwdArgs &p, unsigned
     PHASE_END(tid >> 6);
 }
 
-template <typename IOE, typename OPE>
+template <typename IOE, typename OPE, bool HEADS>
 __global__ __launch_bounds__(FWD_THREADS) void lfw_fwd_chunk_kernel(ChunkFwdArgs p) {
     extern __shared__ __align__(16) unsigned char smem[];
     const int tid = threadIdx.x;
     const int64_t b = blockIdx.x;
     // every wave executes exactly (number of steps) workgroup barriers
     if (tid < 256) {
-        fwd_matrix_waves<IOE, OPE>(p, smem, tid, b, 0, b, true);
+        fwd_matrix_waves<IOE, OPE, HEADS>(p, smem, tid, b, 0, b, true);
     } else {
         // prep wave pw: (side, block of the step, token half); each SIMD gets one wave of each side
         const int pw = __builtin_amdgcn_readfirstlane((tid - 256) >> 6);
         const int hh = (pw >> 1) & 1, h = pw >> 2;
         if (((pw ^ h) & 1) == 0)
-            fwd_prep_side<IOE, OPE, true>(p, smem, tid - 256, b, tid & 63, hh, h, b);
+            fwd_prep_side<IOE, OPE, true, HEADS>(p, smem, tid - 256, b, tid & 63, hh, h, b);
         else
-            fwd_prep_side<IOE, OPE, false>(p, smem, tid - 256, b, tid & 63, hh, h, b);
+            fwd_prep_side<IOE, OPE, false, HEADS>(p, smem, tid - 256, b, tid & 63, hh, h, b);
     }
 }
 
@@ -441,7 +480,7 @@ __global__ __launch_bounds__(FWD_THREADS) void lfw_fwd_chunk_kernel(ChunkFwdArgs
 // 8, so that the two halves of a row land on the same XCD and share its L2 for the key-side
 // inputs both of them read.  Each half reports flagged rows in a slot of its own (the value-side
 // gates it checks are its own 32 channels): row_flags[row] and row_flags[rows_padded + row].
-template <typename IOE, typename OPE>
+template <typename IOE, typename OPE, bool HEADS>
 __global__ __launch_bounds__(FWD_THREADS_HALF) void lfw_fwd_chunk_half_kernel(ChunkFwdArgs p, int rows_padded) {
     extern __shared__ __align__(16) unsigned char smem[];
     const int tid = threadIdx.x;
@@ -452,22 +491,23 @@ __global__ __launch_bounds__(FWD_THREADS_HALF) void lfw_fwd_chunk_half_kernel(Ch
     // waves: 0, 1 matrix; 2..5 key side (block, token half); 6, 7 value side (block; a lane takes
     // one of the half's 32 channels and one token half).  SIMD i runs waves i and i + 4.
     if (tid < 128) {
-        fwd_matrix_waves<IOE, OPE>(p, smem, tid, b, 32 * half, slot, false);
+        fwd_matrix_waves<IOE, OPE, HEADS>(p, smem, tid, b, 32 * half, slot, false);
     } else if (tid < 384) {
         const int pw = __builtin_amdgcn_readfirstlane((tid - 128) >> 6);
-        fwd_prep_side<IOE, OPE, true>(p, smem, tid - 128, b, tid & 63, pw & 1, pw >> 1, slot);
+        fwd_prep_side<IOE, OPE, true, HEADS>(p, smem, tid - 128, b, tid & 63, pw & 1, pw >> 1, slot);
     } else {
         const int pw = __builtin_amdgcn_readfirstlane((tid - 384) >> 6);
-        fwd_prep_side<IOE, OPE, false>(p, smem, tid - 128, b, 32 * half + (tid & 31), pw, (tid >> 5) & 1, slot);
+        fwd_prep_side<IOE, OPE, false, HEADS>(p, smem, tid - 128, b, 32 * half + (tid & 31), pw, (tid >> 5) & 1, slot);
     }
 }
 
-template <typename IOE, typename OPE> int launch(const ChunkFwdArgs &a, bool split, hipStream_t stream) {
+template <typename IOE, typename OPE, bool HEADS> int launch(const ChunkFwdArgs &a, bool split, hipStream_t stream) {
     if (a.B > 0x1fffffffLL) return fail(T2FW_ERR_UNSUPPORTED, "B=%lld is too large", (long long)a.B);
-    if (a.T >= CHUNK_MAX_T) return fail(T2FW_ERR_UNSUPPORTED, "T=%lld is too long for 32-bit row offsets", (long long)a.T);
+    if (a.heads < 1 || a.T * a.heads >= CHUNK_MAX_T)
+        return fail(T2FW_ERR_UNSUPPORTED, "T=%lld with %d heads is too long for 32-bit row offsets", (long long)a.T, a.heads);
     // more than 64 KB of dynamic LDS has to be enabled per function (and per device)
     if (split) {
-        auto kern = lfw_fwd_chunk_half_kernel<IOE, OPE>;
+        auto kern = lfw_fwd_chunk_half_kernel<IOE, OPE, HEADS>;
         int rc = check_hip(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
                                                hipFuncAttributeMaxDynamicSharedMemorySize, FWD_SMEM),
                            "hipFuncSetAttribute(forward chunk kernel, two workgroups per row)");
@@ -476,7 +516,7 @@ template <typename IOE, typename OPE> int launch(const ChunkFwdArgs &a, bool spl
         hipLaunchKernelGGL(kern, dim3(2u * (unsigned)rows_padded), dim3(FWD_THREADS_HALF), FWD_SMEM, stream, a, rows_padded);
         return check_hip(hipGetLastError(), "lfw_fwd_chunk_half_kernel launch");
     }
-    auto kern = lfw_fwd_chunk_kernel<IOE, OPE>;
+    auto kern = lfw_fwd_chunk_kernel<IOE, OPE, HEADS>;
     int rc = check_hip(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, FWD_SMEM),
                        "hipFuncSetAttribute(forward chunk kernel)");
@@ -488,8 +528,15 @@ template <typename IOE, typename OPE> int launch(const ChunkFwdArgs &a, bool spl
 }  // namespace
 
 int chunk_forward(const ChunkFwdArgs &a, int dtype, int op, bool split, hipStream_t stream) {
-    if (dtype == T2FW_F16) return op == 1 ? launch<Fp16, Fp16>(a, split, stream) : launch<Fp16, Bf16>(a, split, stream);
-    if (dtype == T2FW_BF16) return launch<Bf16, Bf16>(a, split, stream);
+    if (a.heads == 1) {
+        if (dtype == T2FW_F16)
+            return op == 1 ? launch<Fp16, Fp16, false>(a, split, stream) : launch<Fp16, Bf16, false>(a, split, stream);
+        if (dtype == T2FW_BF16) return launch<Bf16, Bf16, false>(a, split, stream);
+    } else {
+        if (dtype == T2FW_F16)
+            return op == 1 ? launch<Fp16, Fp16, true>(a, split, stream) : launch<Fp16, Bf16, true>(a, split, stream);
+        if (dtype == T2FW_BF16) return launch<Bf16, Bf16, true>(a, split, stream);
+    }
     return fail(T2FW_ERR_UNSUPPORTED, "the chunked kernels take fp16 or bf16 tensors");
 }
 

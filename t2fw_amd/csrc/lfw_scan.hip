@@ -39,6 +39,7 @@ __device__ __forceinline__ void fwd_scan_body(const ScanFwdArgs &p, int64_t b, i
     Acc *outL = rowL + (size_t)tb * 2 * g.rows;          // [tb][rows]
 
     const int64_t T = p.T, D = p.D, K = p.K;
+    const int64_t line0 = row_first_token(b, T, p.heads);      // [.., D] line of this row's step 0
     const int64_t d0 = (int64_t)tile * g.rows;
     const int64_t d = d0 + g.r;
     const bool row_ok = d < D;
@@ -54,7 +55,7 @@ __device__ __forceinline__ void fwd_scan_body(const ScanFwdArgs &p, int64_t b, i
         S[j] = (row_ok && g.k0 + j < K) ? to_acc(s0[(b * D + d) * K + g.k0 + j]) : Acc(0);
 
     Prefetch<IO, 3, 2> pf;
-    block_load(pf, g, colp, rowp, b, T, 0, (int)(T < tb ? T : tb), K, D, d0);
+    block_load(pf, g, colp, rowp, b, T, 0, (int)(T < tb ? T : tb), K, D, d0, p.heads);
 
     int until_ckpt = 0;          // steps until the next checkpoint is due
     int64_t chunk = 0;
@@ -66,13 +67,13 @@ __device__ __forceinline__ void fwd_scan_body(const ScanFwdArgs &p, int64_t b, i
         // flush the previous block's outputs, then publish this block's inputs
         for (int idx = threadIdx.x; idx < n_prev * g.rows; idx += SCAN_THREADS) {
             const int tt = idx / g.rows, rr = idx % g.rows;
-            if (d0 + rr < D) out[(b * T + t_prev + tt) * D + d0 + rr] = from_acc<IO>(outL[idx]);
+            if (d0 + rr < D) out[(line0 + (t_prev + tt) * p.heads) * D + d0 + rr] = from_acc<IO>(outL[idx]);
         }
         block_store<IO, Acc, 3, 2>(pf, g, colL, rowL, tb);
         __syncthreads();
         if (t0 + tb < T) {
             const int64_t tn = t0 + tb;
-            block_load(pf, g, colp, rowp, b, T, tn, (int)(T - tn < tb ? T - tn : tb), K, D, d0);
+            block_load(pf, g, colp, rowp, b, T, tn, (int)(T - tn < tb ? T - tn : tb), K, D, d0, p.heads);
         }
         for (int tt = 0; tt < n; ++tt) {
             if (ckpt != nullptr) {
@@ -108,7 +109,7 @@ __device__ __forceinline__ void fwd_scan_body(const ScanFwdArgs &p, int64_t b, i
     __syncthreads();
     for (int idx = threadIdx.x; idx < n_prev * g.rows; idx += SCAN_THREADS) {
         const int tt = idx / g.rows, rr = idx % g.rows;
-        if (d0 + rr < D) out[(b * T + t_prev + tt) * D + d0 + rr] = from_acc<IO>(outL[idx]);
+        if (d0 + rr < D) out[(line0 + (t_prev + tt) * p.heads) * D + d0 + rr] = from_acc<IO>(outL[idx]);
     }
     if (row_ok) {
 #pragma unroll
@@ -161,6 +162,7 @@ __device__ __forceinline__ void bwd_scan_body(const ScanBwdArgs &p, int64_t b, i
     Acc *subL = outL + (size_t)SEG * 3 * g.rows;         // [nseg_max][KPL][SCAN_THREADS]
 
     const int64_t T = p.T;
+    const int64_t line0 = row_first_token(b, T, p.heads);      // [.., D|K] line of this row's step 0
     const int64_t nrows = SIDE == 0 ? p.D : p.K, ncols = SIDE == 0 ? p.K : p.D;
     const int64_t row0 = (int64_t)tile * g.rows;
     const int64_t row = row0 + g.r;
@@ -209,7 +211,7 @@ __device__ __forceinline__ void bwd_scan_body(const ScanBwdArgs &p, int64_t b, i
                 for (int j = 0; j < KPL; ++j) subL[((size_t)s * KPL + j) * SCAN_THREADS + threadIdx.x] = S[j];
                 if (s == nseg - 1) break;
                 const int64_t t0 = tc0 + (int64_t)s * SEG;
-                block_load(pf, g, colp, rowp, b, T, t0, SEG, ncols, nrows, row0);
+                block_load(pf, g, colp, rowp, b, T, t0, SEG, ncols, nrows, row0, p.heads);
                 __syncthreads();
                 block_store<IO, Acc, 3, 3>(pf, g, colL, rowL, SEG);
                 __syncthreads();
@@ -238,7 +240,7 @@ __device__ __forceinline__ void bwd_scan_body(const ScanBwdArgs &p, int64_t b, i
 #pragma unroll
                 for (int j = 0; j < KPL; ++j) st[0][j] = el_ok(j) ? to_acc(ck[st_off(j)]) : Acc(0);
                 for (int s2 = 0; s2 < s; ++s2) {
-                    block_load(pf, g, colp, rowp, b, T, tc0 + (int64_t)s2 * SEG, SEG, ncols, nrows, row0);
+                    block_load(pf, g, colp, rowp, b, T, tc0 + (int64_t)s2 * SEG, SEG, ncols, nrows, row0, p.heads);
                     __syncthreads();
                     block_store<IO, Acc, 3, 3>(pf, g, colL, rowL, SEG);
                     __syncthreads();
@@ -253,7 +255,7 @@ __device__ __forceinline__ void bwd_scan_body(const ScanBwdArgs &p, int64_t b, i
                     }
                 }
             }
-            block_load(pf, g, colp, rowp, b, T, t0, n, ncols, nrows, row0);
+            block_load(pf, g, colp, rowp, b, T, t0, n, ncols, nrows, row0, p.heads);
             __syncthreads();
             block_store<IO, Acc, 3, 3>(pf, g, colL, rowL, SEG);
             __syncthreads();
@@ -299,7 +301,7 @@ __device__ __forceinline__ void bwd_scan_body(const ScanBwdArgs &p, int64_t b, i
             for (int idx = threadIdx.x; idx < n * g.rows; idx += SCAN_THREADS) {
                 const int tt = idx / g.rows, rr = idx % g.rows;
                 if (row0 + rr < nrows) {
-                    const int64_t o = (b * T + t0 + tt) * nrows + row0 + rr;
+                    const int64_t o = (line0 + (t0 + tt) * p.heads) * nrows + row0 + rr;
                     d_a[o] = from_acc<IO>(outL[(tt * 3 + 0) * g.rows + rr]);
                     d_gate[o] = from_acc<IO>(outL[(tt * 3 + 1) * g.rows + rr]);
                     if (SIDE == 1) d_u[o] = from_acc<IO>(outL[(tt * 3 + 2) * g.rows + rr]);

@@ -12,6 +12,7 @@ struct ScanFwdArgs {
     const int32_t *row_select2;         // ... unless this second per-row array (may be null) is nonzero there
     int64_t B, T, D, K, NC;
     int32_t C, kg, tb, ntiles;
+    int32_t heads;                      // 1, or H: row b is head b % H of [B/H, T, H, D|K] tensors (x, f, q, k, f_key, out)
 };
 
 struct ScanBwdArgs {
@@ -20,6 +21,7 @@ struct ScanBwdArgs {
     const int32_t *row_select;
     int64_t B, T, D, K, NC;
     int32_t C, kg, use_sub, ntiles;
+    int32_t heads;                      // as for the forward (inputs, g_out and the five [.., T, .., D|K] gradients)
 };
 
 int scan_forward(const ScanFwdArgs &a, int dtype, hipStream_t stream);

@@ -39,16 +39,19 @@ template <typename IO, int NCA, int NRA> struct Prefetch {
 };
 
 // Issue the global loads of a block of n steps starting at step t0 of batch row b.
-// colp[a] are [B,T,ncols] arrays, rowp[a] are [B,T,nrows] arrays; this workgroup
-// needs all columns and rows [row0, row0 + rows).
+// colp[a] are [B,T,ncols] arrays, rowp[a] are [B,T,nrows] arrays (heads = 1), or
+// [B/heads,T,heads,ncols] and [B/heads,T,heads,nrows] with row b = (batch, head); this
+// workgroup needs all columns and rows [row0, row0 + rows).
 template <typename IO, int NCA, int NRA>
 __device__ __forceinline__ void block_load(Prefetch<IO, NCA, NRA> &pf, const Tile &g,
                                            const IO *const (&colp)[NCA],
                                            const IO *const (&rowp)[NRA],
                                            int64_t b, int64_t T, int64_t t0, int n,
-                                           int64_t ncols, int64_t nrows, int64_t row0) {
+                                           int64_t ncols, int64_t nrows, int64_t row0, int64_t heads = 1) {
     const int csub = threadIdx.x % g.CW, tsub = threadIdx.x / g.CW;
-    const int64_t cbase = (b * T + t0) * ncols;
+    const int64_t line0 = row_first_token(b, T, heads) + t0 * heads;      // [.., width] line of step t0
+    const int64_t cstep = heads * ncols, rstep = heads * nrows;           // elements between consecutive steps
+    const int64_t cbase = line0 * ncols;
 #pragma unroll
     for (int m = 0; m < PFC; ++m) {
         const int tt = tsub + g.SP * (m >> g.lncc);
@@ -56,17 +59,17 @@ __device__ __forceinline__ void block_load(Prefetch<IO, NCA, NRA> &pf, const Til
         const bool ok = tt < n && c < ncols;
 #pragma unroll
         for (int a = 0; a < NCA; ++a)
-            pf.c[a][m] = ok ? colp[a][cbase + (int64_t)tt * ncols + c] : IO(0);
+            pf.c[a][m] = ok ? colp[a][cbase + (int64_t)tt * cstep + c] : IO(0);
     }
     const int rsub = threadIdx.x % g.rows, tsr = threadIdx.x / g.rows;
-    const int64_t rbase = (b * T + t0) * nrows + row0;
+    const int64_t rbase = line0 * nrows + row0;
 #pragma unroll
     for (int m = 0; m < PFR; ++m) {
         const int tt = tsr + g.SPR * m;
         const bool ok = tt < n && row0 + rsub < nrows;
 #pragma unroll
         for (int a = 0; a < NRA; ++a)
-            pf.r[a][m] = ok ? rowp[a][rbase + (int64_t)tt * nrows + rsub] : IO(0);
+            pf.r[a][m] = ok ? rowp[a][rbase + (int64_t)tt * rstep + rsub] : IO(0);
     }
 }
 

@@ -45,9 +45,11 @@ def _dtype_code(dtype):
         raise RuntimeError("t2fw: unsupported dtype %s" % dtype)
 
 
-def _lfw_forward(value, forget, query, key, f_key, state, need_grad):
+def _lfw_forward(value, forget, query, key, f_key, state, need_grad, heads=False):
     """Checks as in t2fw/functional_lfw.py:42-49 and t2fw/csrc/lfw.cpp:24-26,36-41, then the forward
-    kernels.  Returns (outputs, next_state, ckpt or None, checkpoint interval, flags)."""
+    kernels.  heads=False: x,f [B,T,D]; q,k,f_key [B,T,K]; state [B,D,K].  heads=True: x,f [B,T,H,D];
+    q,k,f_key [B,T,H,K]; state [B,H,D,K].  Returns (outputs, next_state, ckpt or None, checkpoint
+    interval, flags)."""
     assert value.shape == forget.shape
     assert query.shape == key.shape
     assert query.shape == f_key.shape
@@ -59,11 +61,15 @@ def _lfw_forward(value, forget, query, key, f_key, state, need_grad):
     for t, n in ((value, "x"), (forget, "f"), (query, "query"), (key, "key"),
                  (f_key, "f_key"), (state, "state")):
         _check_input(t, n)
-    if value.dim() != 3 or query.dim() != 3 or state.dim() != 3:
-        raise RuntimeError("t2fw: expected x,f [B,T,D]; q,k,f_key [B,T,K]; state [B,D,K]")
-    B, T, D = value.shape
-    K = query.shape[2]
-    if query.shape[0] != B or query.shape[1] != T or tuple(state.shape) != (B, D, K):
+    nd = 4 if heads else 3
+    if value.dim() != nd or query.dim() != nd or state.dim() != nd:
+        raise RuntimeError("t2fw: expected x,f [B,T,H,D]; q,k,f_key [B,T,H,K]; state [B,H,D,K]" if heads else
+                           "t2fw: expected x,f [B,T,D]; q,k,f_key [B,T,K]; state [B,D,K]")
+    B, T = value.shape[:2]
+    H = value.shape[2] if heads else 1
+    D, K = value.shape[-1], query.shape[-1]
+    if tuple(query.shape[:-1]) != tuple(value.shape[:-1]) or \
+            tuple(state.shape) != ((B, H, D, K) if heads else (B, D, K)):
         raise RuntimeError("t2fw: inconsistent shapes x %s, query %s, state %s"
                            % (tuple(value.shape), tuple(query.shape), tuple(state.shape)))
     code = _dtype_code(value.dtype)
@@ -77,26 +83,29 @@ def _lfw_forward(value, forget, query, key, f_key, state, need_grad):
         ckpt = None
         if need_grad:
             nc = lib.t2fw_lfw_num_ckpt(T, C)
-            ckpt = torch.empty((B, nc, D, K), dtype=value.dtype, device=dev)
-        ws_bytes = lib.t2fw_lfw_workspace_bytes(B, T, D, K, C, code, flags)
+            ckpt = torch.empty((B * H, nc, D, K), dtype=value.dtype, device=dev)
+        ws_bytes = lib.t2fw_lfw_workspace_bytes(B * H, T, D, K, C, code, flags)
         ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev) if ws_bytes else None
-        _lib.check(lib.t2fw_lfw_forward(
-            _lib.ptr(value), _lib.ptr(forget), _lib.ptr(query), _lib.ptr(key), _lib.ptr(f_key),
-            _lib.ptr(state), _lib.ptr(outputs), _lib.ptr(next_state), _lib.ptr(ckpt),
-            B, T, D, K, C, code, flags, _lib.ptr(ws), ws_bytes,
-            _lib.current_stream_handle(dev)))
+        ptrs = (_lib.ptr(value), _lib.ptr(forget), _lib.ptr(query), _lib.ptr(key), _lib.ptr(f_key),
+                _lib.ptr(state), _lib.ptr(outputs), _lib.ptr(next_state), _lib.ptr(ckpt))
+        tail = (D, K, C, code, flags, _lib.ptr(ws), ws_bytes, _lib.current_stream_handle(dev))
+        if heads:
+            _lib.check(lib.t2fw_lfw_forward_heads(*ptrs, B, T, H, *tail))
+        else:
+            _lib.check(lib.t2fw_lfw_forward(*ptrs, B, T, *tail))
     return outputs, next_state, ckpt, C, flags
 
 
-def _lfw_backward(grad_output, grad_state, value, forget, query, key, f_key, state, ckpt, C, flags):
-    """The backward kernels; gradients in the order of t2fw/csrc/lfw.cpp:95."""
+def _lfw_backward(grad_output, grad_state, value, forget, query, key, f_key, state, ckpt, C, flags, heads=False):
+    """The backward kernels; gradients in the order of t2fw/csrc/lfw.cpp:95, laid out as their inputs."""
     # t2fw/functional_lfw.py:71-72
     assert grad_state.dtype == value.dtype
     assert grad_output.dtype == value.dtype
     grad_output = grad_output.contiguous()
     grad_state = grad_state.contiguous()
-    B, T, D = value.shape
-    K = query.shape[2]
+    B, T = value.shape[:2]
+    H = value.shape[2] if heads else 1
+    D, K = value.shape[-1], query.shape[-1]
     code = _dtype_code(value.dtype)
     lib = _lib.load()
     dev = value.device
@@ -107,14 +116,16 @@ def _lfw_backward(grad_output, grad_state, value, forget, query, key, f_key, sta
         d_k = torch.empty_like(key)
         d_fk = torch.empty_like(f_key)
         d_s = torch.empty_like(state)
-        ws_bytes = lib.t2fw_lfw_workspace_bytes(B, T, D, K, C, code, flags)
+        ws_bytes = lib.t2fw_lfw_workspace_bytes(B * H, T, D, K, C, code, flags)
         ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev) if ws_bytes else None
-        _lib.check(lib.t2fw_lfw_backward(
-            _lib.ptr(grad_output), _lib.ptr(grad_state), _lib.ptr(value), _lib.ptr(forget),
-            _lib.ptr(query), _lib.ptr(key), _lib.ptr(f_key), _lib.ptr(state), _lib.ptr(ckpt),
-            _lib.ptr(d_x), _lib.ptr(d_f), _lib.ptr(d_q), _lib.ptr(d_k), _lib.ptr(d_fk), _lib.ptr(d_s),
-            B, T, D, K, C, code, flags, _lib.ptr(ws), ws_bytes,
-            _lib.current_stream_handle(dev)))
+        ptrs = (_lib.ptr(grad_output), _lib.ptr(grad_state), _lib.ptr(value), _lib.ptr(forget),
+                _lib.ptr(query), _lib.ptr(key), _lib.ptr(f_key), _lib.ptr(state), _lib.ptr(ckpt),
+                _lib.ptr(d_x), _lib.ptr(d_f), _lib.ptr(d_q), _lib.ptr(d_k), _lib.ptr(d_fk), _lib.ptr(d_s))
+        tail = (D, K, C, code, flags, _lib.ptr(ws), ws_bytes, _lib.current_stream_handle(dev))
+        if heads:
+            _lib.check(lib.t2fw_lfw_backward_heads(*ptrs, B, T, H, *tail))
+        else:
+            _lib.check(lib.t2fw_lfw_backward(*ptrs, B, T, *tail))
     return d_x, d_f, d_q, d_k, d_fk, d_s
 
 
@@ -156,6 +167,16 @@ def sigmoid_gates(f_logit, fk_logit, out_f=None, out_fk=None):
     return f, fk
 
 
+def _gate_backward_inplace(d_f, d_fk, forget, f_key):
+    """d_f, d_fk: gate gradients on entry, logit gradients d_gate * gate * (1 - gate) on return."""
+    lib = _lib.load()
+    dev = d_f.device
+    with torch.cuda.device(dev):
+        _lib.check(lib.t2fw_gate_backward(_lib.ptr(d_f), _lib.ptr(d_fk), _lib.ptr(forget), _lib.ptr(f_key),
+                                          _lib.ptr(d_f), _lib.ptr(d_fk), d_f.numel(), d_fk.numel(),
+                                          _dtype_code(d_f.dtype), _lib.current_stream_handle(dev)))
+
+
 class LFWGatedFunction(torch.autograd.Function):
     """``LFWFunction`` on gate *logits*: f = sigmoid(f_logit), f_key = sigmoid(fk_logit) are computed
     by one streaming kernel for both gates, the gates (not the logits) are kept for backward, and
@@ -181,13 +202,45 @@ class LFWGatedFunction(torch.autograd.Function):
         value, forget, query, key, f_key, state, ckpt = ctx.saved_tensors
         d_x, d_f, d_q, d_k, d_fk, d_s = _lfw_backward(grad_output, grad_state, value, forget, query, key, f_key,
                                                       state, ckpt, ctx.ckpt_interval, ctx.flags)
-        lib = _lib.load()
-        dev = value.device
-        with torch.cuda.device(dev):
-            _lib.check(lib.t2fw_gate_backward(_lib.ptr(d_f), _lib.ptr(d_fk), _lib.ptr(forget), _lib.ptr(f_key),
-                                              _lib.ptr(d_f), _lib.ptr(d_fk), d_f.numel(), d_fk.numel(),
-                                              _dtype_code(value.dtype), _lib.current_stream_handle(dev)))
+        _gate_backward_inplace(d_f, d_fk, forget, f_key)
         return d_x, d_f, d_q, d_k, d_fk, d_s
+
+
+class LFWHeadsFunction(torch.autograd.Function):
+    """The decay rule on tensors that keep the head axis next to the channels: x, f ``[B,T,H,D]``;
+    q, k, f_key ``[B,T,H,K]``; state ``[B,H,D,K]``; returns outputs ``[B,T,H,D]`` and the final state
+    ``[B,H,D,K]``.  Every (batch, head) pair is one recurrence.  The reference needs the folded,
+    contiguous ``[B*H,T,D]`` layout (t2fw/csrc/lfw.cpp:24-26), i.e. ``transpose(1, 2).contiguous()``
+    on five inputs and the inverse on the outputs and on six gradients; here the kernels stride
+    over the head axis and those copies disappear.
+
+    ``logits=True``: ``f`` and ``f_key`` are gate logits and the sigmoid is applied here (as in
+    ``LFWGatedFunction``); the gradients returned for them are then logit gradients."""
+
+    @staticmethod
+    def forward(ctx, value, forget, query, key, f_key, state, logits=False):
+        if logits:
+            assert value.shape == forget.shape and query.shape == f_key.shape
+            assert forget.dtype == value.dtype and f_key.dtype == value.dtype
+            forget, f_key = sigmoid_gates(forget, f_key)
+        need_grad = any(ctx.needs_input_grad)
+        outputs, next_state, ckpt, C, flags = _lfw_forward(value, forget, query, key, f_key, state, need_grad,
+                                                           heads=True)
+        if need_grad:
+            ctx.save_for_backward(value, forget, query, key, f_key, state, ckpt)
+            ctx.ckpt_interval = C
+            ctx.flags = flags
+            ctx.logits = bool(logits)
+        return outputs, next_state
+
+    @staticmethod
+    def backward(ctx, grad_output, grad_state):
+        value, forget, query, key, f_key, state, ckpt = ctx.saved_tensors
+        d_x, d_f, d_q, d_k, d_fk, d_s = _lfw_backward(grad_output, grad_state, value, forget, query, key, f_key,
+                                                      state, ckpt, ctx.ckpt_interval, ctx.flags, heads=True)
+        if ctx.logits:
+            _gate_backward_inplace(d_f, d_fk, forget, f_key)
+        return d_x, d_f, d_q, d_k, d_fk, d_s, None
 
 
 def lfw_step(x, f, query, key, f_key, state, out=None, inplace=True):
