@@ -704,10 +704,12 @@ __device__ __forceinline__ void split_matrix_waves(const ChunkBwdArgs &p, unsign
                         const float4 pp = *reinterpret_cast<const float4 *>(cf + F_PP * (CF_TILE / 4));
                         ppv[0] = pp.x; ppv[1] = pp.y; ppv[2] = pp.z; ppv[3] = pp.w;
                     }
+                    // one address per array; the four tokens are immediate offsets from it (folded rows)
+                    u16 *const pv = d_val + go, *const pg = d_gate + go, *const pa = d_adj + go;
                     auto store = [&](int ii) {
-                        d_val[go + ii * ts] = cvt1<IOE>(ipv[ii] * (va[ii] + asv[ii] * pd[ii]));
-                        d_gate[go + ii * ts] = cvt1<IOE>(du[ii] * rgv[ii]);
-                        if (side == 1) d_adj[go + ii * ts] = cvt1<IOE>(ppv[ii] * (oa[ii] + vtv[ii] * pd[ii]));
+                        pv[ii * ts] = cvt1<IOE>(ipv[ii] * (va[ii] + asv[ii] * pd[ii]));
+                        pg[ii * ts] = cvt1<IOE>(du[ii] * rgv[ii]);
+                        if (side == 1) pa[ii * ts] = cvt1<IOE>(ppv[ii] * (oa[ii] + vtv[ii] * pd[ii]));
                     };
                     if ((int)chunk * C + (i + 1) * CH_L <= T) {
 #pragma unroll

@@ -429,14 +429,14 @@ __device__ __forceinline__ void fwd_matrix_waves(const ChunkFwdArgs &p, unsigned
             const float asv[4] = {as.x, as.y, as.z, as.w};
             // 16 lanes write 32 contiguous bytes of a token row; the four waves complete the row
             const int tg = n * CH_STEP + tok0 + 4 * g;
-            const u32 go = (u32)tg * ts + (u32)d;
+            u16 *const po = out + ((u32)tg * ts + (u32)d);      // the four tokens: immediate offsets (folded rows)
             if ((n + 1) * CH_STEP <= T) {
 #pragma unroll
-                for (int i = 0; i < 4; ++i) out[go + i * ts] = cvt1<IOE>((o[i] + oi[i]) * asv[i]);
+                for (int i = 0; i < 4; ++i) po[i * ts] = cvt1<IOE>((o[i] + oi[i]) * asv[i]);
             } else {
 #pragma unroll
                 for (int i = 0; i < 4; ++i)
-                    if (tg + i < T) out[go + i * ts] = cvt1<IOE>((o[i] + oi[i]) * asv[i]);
+                    if (tg + i < T) po[i * ts] = cvt1<IOE>((o[i] + oi[i]) * asv[i]);
             }
             // S_L = (a_L (x) b_L) * S0 + sum_s xh_s (x) kh_s
             const float aL = AL[hh * CH_N + d];
