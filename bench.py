@@ -215,6 +215,27 @@ def main():
         torch.cuda.synchronize()
         autograd = {"ms_per_step": round((time.perf_counter() - t0) / n_a * 1e3, 4)}
         autograd["value"] = round(B * T / autograd["ms_per_step"] / 1e3, 1)
+        # ... and recorded once into a HIP graph and replayed: the host cost of issuing the step
+        # through autograd (which exceeds the GPU time at small shapes) disappears
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            astep(0)
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            o, n = LFWFunction.apply(*leaves[0])
+            torch.autograd.backward([o, n], [sets[0]["go"], sets[0]["gs"]])
+        for i in range(5):
+            graph.replay()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for i in range(n_a):
+            graph.replay()
+        torch.cuda.synchronize()
+        autograd["graph_replay_ms_per_step"] = round((time.perf_counter() - t0) / n_a * 1e3, 4)
+        autograd["graph_replay_value"] = round(B * T / autograd["graph_replay_ms_per_step"] / 1e3, 1)
 
     cpu = None
     if not args.no_cpu_baseline:
