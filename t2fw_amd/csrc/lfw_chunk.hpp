@@ -27,7 +27,7 @@ struct ChunkFwdArgs {
     void *out, *next_state, *ckpt;     // ckpt may be null
     int32_t *row_flags;                // [2 * chunk_rows_padded(B)]: set to 1 for rows the exact kernels must redo
     int64_t B, T, NC;
-    int32_t C;                         // checkpoint interval, multiple of 32
+    int32_t C;                         // checkpoint interval: 16 (every block) or a multiple of 32
     int32_t heads;                     // 1: rows are [T, 64] slabs; H > 1: row b is head b % H of a [B / H, T, H, 64] tensor
 };
 

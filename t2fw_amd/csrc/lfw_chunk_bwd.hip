@@ -83,8 +83,10 @@ __device__ __forceinline__ const float *lv_vec(const unsigned char *stage, int j
 // Chunks are visited from the last one down; a chunk with nb blocks takes ceil(nb/2) "R"
 // stages of two blocks each (forward in time), then nb "B" stages (blocks nb-1..0).
 // A stage is one int: (first token of its first block) * 2 + (1 for a B stage).
+// NB = 1 means a checkpoint per block (C = 16): the state at every block start comes from memory, so
+// only the last block of the sequence takes an R stage (for the state at the end of the sequence).
 template <int NB> struct SplitSchedule {
-    static constexpr unsigned PER_CHUNK = NB / 2 + NB;
+    static constexpr unsigned PER_CHUNK = NB == 1 ? 1 : NB / 2 + NB;
     int NC, C, total, nb_last, st_last;
     __device__ SplitSchedule(int64_t T, int64_t NC_, int C_) {
         NC = (int)NC_;
@@ -93,23 +95,6 @@ template <int NB> struct SplitSchedule {
         nb_last = (len_last + CH_L - 1) / CH_L;
         st_last = (nb_last + 1) / 2 + nb_last;
         total = st_last + (NC - 1) * (int)PER_CHUNK;
-    }
-    __device__ int at(int s) const {
-        int chunk, local, nb;
-        if (s < st_last) {
-            chunk = NC - 1;
-            local = s;
-            nb = nb_last;
-        } else {
-            const unsigned s2 = (unsigned)(s - st_last);
-            chunk = NC - 2 - (int)(s2 / PER_CHUNK);
-            local = (int)(s2 % PER_CHUNK);
-            nb = NB;
-        }
-        const int nr = (nb + 1) / 2;
-        const bool bmode = local >= nr;
-        const int block = bmode ? nb - 1 - (local - nr) : 2 * local;
-        return ((chunk * C + block * CH_L) << 1) | (bmode ? 1 : 0);
     }
 };
 
@@ -142,7 +127,7 @@ template <int NB> struct StageIter {
                 base2 -= C2;
                 local = 0;
                 count = (int)SplitSchedule<NB>::PER_CHUNK;
-                table = table_of(NB);
+                table = NB == 1 ? (uint64_t)1 /* one B stage, block 0 */ : table_of(NB);
             }
         }
     }
@@ -422,6 +407,7 @@ __device__ __forceinline__ void split_prep_waves(const ChunkBwdArgs &p, unsigned
     // in flight is the same on every path and the waits for them can be exact.
     StageIter<NB> it_load(sched);
     int st_cur = 0, st_next = 0;                   // descriptors of stages s and s + 1
+    PHASE_BEGIN();
     auto prepare = [&](const RawSet &cur, RawSet &refill, int s) {
         const int st = st_cur;
         it_load.advance();
@@ -450,8 +436,8 @@ __device__ __forceinline__ void split_prep_waves(const ChunkBwdArgs &p, unsigned
     // peeled off, with the sets assigned so that the triples start on A.
     RawSet setA, setB, setC;
     int s = 0;
-    PHASE_BEGIN();
-    const int n_last = sched.st_last;
+    // (with a checkpoint per block, also as many of the following blocks as make the rest a multiple of three)
+    const int n_last = sched.st_last + (NB == 1 ? (sched.NC - 1) % 3 : 0);
     const int rem = n_last % 3;
     st_cur = it_load.cur();
     it_load.advance();
@@ -477,51 +463,73 @@ __device__ __forceinline__ void split_prep_waves(const ChunkBwdArgs &p, unsigned
         prepare(setC, setB, s + 2);
     }
 
-    // Then the full chunks, last to first.  Inside a chunk the kind of every stage and its block are
-    // compile-time constants (position POS of PER), which leaves a pointer bump per stage for the
-    // scalar unit; PER is a multiple of three, so every chunk starts on set A.  The refill of
-    // position POS + 2 reaches into the chunk below for the last two positions (below the first
-    // chunk: that chunk again, never used).
-    constexpr int PER = (int)SplitSchedule<NB>::PER_CHUNK, NR = NB / 2;
-    static_assert(PER % 3 == 0, "a chunk must take a whole number of register-set triples");
-    const u16 *const r_gate_w = r_gate + (u32)(rj * CH_L) * ts, *const r_val_w = r_val + (u32)(rj * CH_L) * ts;
-    auto issue_at = [&](RawSet &r, int chunk_tok, auto pos_c) {
-        constexpr int POS = decltype(pos_c)::value;
-        if constexpr (POS < NR) {
-            const u32 e = (u32)(chunk_tok + 2 * POS * CH_L) * ts;
-            raw_issue<HEADS>(r, r_gate_w + e, r_val_w + e, tmap);
-        } else {
-            const u32 e = (u32)(chunk_tok + (NB - 1 - (POS - NR)) * CH_L) * ts;
-            raw_issue<HEADS>(r, b_gate + e, b_val + e, tmap);
+    if constexpr (NB != 1) {
+        // Then the full chunks, last to first.  Inside a chunk the kind of every stage and its block are
+        // compile-time constants (position POS of PER), which leaves a pointer bump per stage for the
+        // scalar unit; PER is a multiple of three, so every chunk starts on set A.  The refill of
+        // position POS + 2 reaches into the chunk below for the last two positions (below the first
+        // chunk: that chunk again, never used).
+        constexpr int PER = (int)SplitSchedule<NB>::PER_CHUNK, NR = NB / 2;
+        static_assert(PER % 3 == 0, "a chunk must take a whole number of register-set triples");
+        const u16 *const r_gate_w = r_gate + (u32)(rj * CH_L) * ts, *const r_val_w = r_val + (u32)(rj * CH_L) * ts;
+        auto issue_at = [&](RawSet &r, int chunk_tok, auto pos_c) {
+            constexpr int POS = decltype(pos_c)::value;
+            if constexpr (POS < NR) {
+                const u32 e = (u32)(chunk_tok + 2 * POS * CH_L) * ts;
+                raw_issue<HEADS>(r, r_gate_w + e, r_val_w + e, tmap);
+            } else {
+                const u32 e = (u32)(chunk_tok + (NB - 1 - (POS - NR)) * CH_L) * ts;
+                raw_issue<HEADS>(r, b_gate + e, b_val + e, tmap);
+            }
+        };
+        auto prepare_at = [&](const RawSet &cur, RawSet &refill, int chunk_tok, int below_tok, auto pos_c) {
+            constexpr int POS = decltype(pos_c)::value;
+            if constexpr (POS + 2 < PER)
+                issue_at(refill, chunk_tok, std::integral_constant<int, (POS + 2) % PER>{});
+            else
+                issue_at(refill, below_tok, std::integral_constant<int, (POS + 2) % PER>{});
+            // the loads complete in order: one wait for the last of `cur` covers the whole set
+            asm volatile("" ::"v"(cur.val[7]));
+            unsigned char *stage = smem + (s & 1) * STAGE_BYTES;
+            if constexpr (POS >= NR)
+                prep_b<IOE, OPE>(cur, stage, role, h, c, side == 1, bad);
+            else
+                prep_r<IOE, OPE>(cur, stage, rj, rown, h, c, bad);
+            ++s;
+            PHASE_MARK(2);
+            __syncthreads();
+            PHASE_MARK(3);
+        };
+        for (int chunk_tok = (sched.NC - 2) * p.C; chunk_tok >= 0; chunk_tok -= p.C) {
+            const int below_tok = max(chunk_tok - p.C, 0);
+            prepare_at(setA, setC, chunk_tok, below_tok, std::integral_constant<int, 0>{});
+            prepare_at(setB, setA, chunk_tok, below_tok, std::integral_constant<int, 1>{});
+            prepare_at(setC, setB, chunk_tok, below_tok, std::integral_constant<int, 2>{});
+            if constexpr (PER == 6) {
+                prepare_at(setA, setC, chunk_tok, below_tok, std::integral_constant<int, 3>{});
+                prepare_at(setB, setA, chunk_tok, below_tok, std::integral_constant<int, 4>{});
+                prepare_at(setC, setB, chunk_tok, below_tok, std::integral_constant<int, 5>{});
+            }
         }
-    };
-    auto prepare_at = [&](const RawSet &cur, RawSet &refill, int chunk_tok, int below_tok, auto pos_c) {
-        constexpr int POS = decltype(pos_c)::value;
-        if constexpr (POS + 2 < PER)
-            issue_at(refill, chunk_tok, std::integral_constant<int, (POS + 2) % PER>{});
-        else
-            issue_at(refill, below_tok, std::integral_constant<int, (POS + 2) % PER>{});
-        // the loads complete in order: one wait for the last of `cur` covers the whole set
-        asm volatile("" ::"v"(cur.val[7]));
-        unsigned char *stage = smem + (s & 1) * STAGE_BYTES;
-        if constexpr (POS >= NR)
-            prep_b<IOE, OPE>(cur, stage, role, h, c, side == 1, bad);
-        else
-            prep_r<IOE, OPE>(cur, stage, rj, rown, h, c, bad);
-        ++s;
-        PHASE_MARK(2);
-        __syncthreads();
-        PHASE_MARK(3);
-    };
-    for (int chunk_tok = (sched.NC - 2) * p.C; chunk_tok >= 0; chunk_tok -= p.C) {
-        const int below_tok = max(chunk_tok - p.C, 0);
-        prepare_at(setA, setC, chunk_tok, below_tok, std::integral_constant<int, 0>{});
-        prepare_at(setB, setA, chunk_tok, below_tok, std::integral_constant<int, 1>{});
-        prepare_at(setC, setB, chunk_tok, below_tok, std::integral_constant<int, 2>{});
-        if constexpr (PER == 6) {
-            prepare_at(setA, setC, chunk_tok, below_tok, std::integral_constant<int, 3>{});
-            prepare_at(setB, setA, chunk_tok, below_tok, std::integral_constant<int, 4>{});
-            prepare_at(setC, setB, chunk_tok, below_tok, std::integral_constant<int, 5>{});
+    } else {
+        // A checkpoint per block: what is left are B stages of full blocks, a multiple of three of
+        // them, last to first; set A holds the highest one, set B the one below it.
+        auto prepare_block = [&](const RawSet &cur, RawSet &refill, int refill_tok) {
+            const u32 e = (u32)max(refill_tok, 0) * ts;      // below the first block: that block again, never used
+            raw_issue<HEADS>(refill, b_gate + e, b_val + e, tmap);
+            // the loads complete in order: one wait for the last of `cur` covers the whole set
+            asm volatile("" ::"v"(cur.val[7]));
+            prep_b<IOE, OPE>(cur, smem + (s & 1) * STAGE_BYTES, role, h, c, side == 1, bad);
+            ++s;
+            PHASE_MARK(2);
+            __syncthreads();
+            PHASE_MARK(3);
+        };
+        const int nblocks = (sched.NC - 1) / 3 * 3;
+        for (int tok = (nblocks - 1) * CH_L; tok >= 0; tok -= 3 * CH_L) {
+            prepare_block(setA, setC, tok - 2 * CH_L);
+            prepare_block(setB, setA, tok - 3 * CH_L);
+            prepare_block(setC, setB, tok - 4 * CH_L);
         }
     }
     // Both workgroups of a row see all four gates' blocks and reach the same verdict, so either
@@ -576,6 +584,59 @@ __device__ __forceinline__ void split_matrix_waves(const ChunkBwdArgs &p, unsign
     load_state(reinterpret_cast<const u16 *>(p.g_state) + b * (CH_N * CH_N), pf);
     take_state(pf, G);
     load_state(ckpt + (NC - 1) * (CH_N * CH_N), pf);
+    // A checkpoint per block (NB = 1): the block-start state of every block but the last comes
+    // straight from memory: raw loads (side 0: four 8-byte loads, side 1: sixteen 2-byte loads of a
+    // column) issued at the start of the stage above and put together at its end; `top` keeps the raw
+    // state of the latest block whose start is a multiple of four blocks (for the anchor).
+    u32 ahead[NB == 1 ? 16 : 1];
+    uint2 below[4] = {};             // raw start state of the block below the current one
+    uint2 top[4] = {pf[0], pf[1], pf[2], pf[3]};
+    auto fetch_ahead = [&](const u16 *m) {
+        if (side == 0) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const uint2 v = ld2(m + ch * CH_N + 16 * j + 4 * g);
+                ahead[(2 * j) % (NB == 1 ? 16 : 1)] = v.x;
+                ahead[(2 * j + 1) % (NB == 1 ? 16 : 1)] = v.y;
+            }
+#pragma unroll
+            for (int j = 8; j < (NB == 1 ? 16 : 1); ++j) ahead[j] = 0;
+        } else {
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) ahead[(4 * j + i) % (NB == 1 ? 16 : 1)] = m[(16 * j + 4 * g + i) * CH_N + ch];
+        }
+    };
+    auto take_ahead = [&](uint2 (&dst)[4]) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            constexpr int M = NB == 1 ? 16 : 1;
+            if (side == 0)
+                dst[j] = make_uint2(ahead[(2 * j) % M], ahead[(2 * j + 1) % M]);
+            else
+                dst[j] = make_uint2(ahead[(4 * j) % M] | (ahead[(4 * j + 1) % M] << 16),
+                                    ahead[(4 * j + 2) % M] | (ahead[(4 * j + 3) % M] << 16));
+        }
+    };
+    // raw state (I/O type, four values per 32-bit pair) -> the two MFMA operands
+    auto to_operands = [&](const uint2 (&raw)[4], uint4 &lo, uint4 &hi) {
+        if constexpr (std::is_same<IOE, OPE>::value) {
+            lo = cat(raw[0], raw[1]);
+            hi = cat(raw[2], raw[3]);
+        } else {
+            uint2 o[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                float t[4];
+                unpack4<IOE>(raw[j], t);
+                const floatx4 v = {t[0], t[1], t[2], t[3]};
+                o[j] = pack4v<OPE>(v);
+            }
+            lo = cat(o[0], o[1]);
+            hi = cat(o[2], o[3]);
+        }
+    };
     float carry = 0.f;
     int s = 0;
     if (tid == 0) {      // both flag slots of the row (the backward kernels report in the first)
@@ -586,20 +647,24 @@ __device__ __forceinline__ void split_matrix_waves(const ChunkBwdArgs &p, unsign
 
     // every stage starts with the workgroup barrier that publishes its operand tiles
     for (int64_t chunk = NC - 1; chunk >= 0; --chunk) {
-        const int nb = chunk == NC - 1 ? nb_last : NB;
-        take_state(pf, S);
-        if (chunk > 0) load_state(ckpt + (chunk - 1) * (CH_N * CH_N), pf);
+        const bool last = chunk == NC - 1;
+        const int nb = last ? nb_last : NB;
+        const bool recompute = NB != 1 || last;              // this chunk has R stages
+        if (recompute) {
+            take_state(pf, S);
+            if (NB != 1 && chunk > 0) load_state(ckpt + (chunk - 1) * (CH_N * CH_N), pf);
+        }
         // ---- R stages: block-start states, forward in time, two blocks per stage
 #pragma unroll
         for (int i2 = 0; i2 < NB; i2 += 2) {
-            if (i2 < nb) {
+            if (i2 < nb && recompute) {
                 __syncthreads();
                 PHASE_MARK(3);
                 const unsigned char *stage = smem + (s & 1) * STAGE_BYTES;
 #pragma unroll
                 for (int jb = 0; jb < 2; ++jb) {
-                    const int i = i2 + jb;
-                    if (i < nb) {
+                    const int i = (i2 + jb) % NB;           // (i2 + jb < NB wherever the branch below is taken)
+                    if (i2 + jb < nb) {
                         const u16 *VOHc = reinterpret_cast<const u16 *>(stage + OFF_CM + (2 * jb) * CM_TILE);
                         const u16 *VHc = reinterpret_cast<const u16 *>(stage + OFF_CM + (2 * jb + 1) * CM_TILE);
                         const float *LX = lv_vec(stage, jb, 0), *LO = lv_vec(stage, jb, 1);
@@ -624,7 +689,9 @@ __device__ __forceinline__ void split_matrix_waves(const ChunkBwdArgs &p, unsign
             }
         }
         // ---- re-anchor the running sum of the gate gradient: sum over the other side of Gb * S_end
-        {
+        // (with a checkpoint per block: every fourth block, S_end = the start state of the block above)
+        if (NB == 1 && !last && (chunk & 3) == 3) take_state(top, S);
+        if (recompute || (chunk & 3) == 3) {
             float us = 0.f;
 #pragma unroll
             for (int j = 0; j < 4; ++j)
@@ -647,6 +714,18 @@ __device__ __forceinline__ void split_matrix_waves(const ChunkBwdArgs &p, unsign
                 const u16 *VTc = reinterpret_cast<const u16 *>(stage + OFF_CM + CM_VT * CM_TILE);
                 const float *LX = lv_vec(stage, 0, 0), *LO = lv_vec(stage, 0, 1);
                 const floatx4 zero = {0.f, 0.f, 0.f, 0.f};
+                // the state at the start of this block, as MFMA operands
+                uint4 sb0 = sv[i][0], sb1 = sv[i][1];
+                if constexpr (NB == 1) {
+                    if (!last) {
+                        to_operands(below, sb0, sb1);
+                        if ((chunk & 3) == 0) {
+#pragma unroll
+                            for (int j = 0; j < 4; ++j) top[j] = below[j];
+                        }
+                    }
+                    if (chunk > 0) fetch_ahead(ckpt + (chunk - 1) * (CH_N * CH_N));
+                }
                 // the 16x16 token-token product, in both orientations (full contraction over 64 channels)
                 const int ro = r * TS + 8 * g;
                 const uint4 vot_lo = ld4(VOT + ro), vot_hi = ld4(VOT + ro + 32);
@@ -666,7 +745,7 @@ __device__ __forceinline__ void split_matrix_waves(const ChunkBwdArgs &p, unsign
                 const float lo = LO[ch];
                 const int po = r * TS + 16 * g;
                 // o' uses the block-start state
-                floatx4 oa = OPE::mfma32(ld4(AOS + po + 8), sv[i][1], OPE::mfma32(ld4(AOS + po), sv[i][0], zero));
+                floatx4 oa = OPE::mfma32(ld4(AOS + po + 8), sb1, OPE::mfma32(ld4(AOS + po), sb0, zero));
                 oa += OPE::mfma16(pa_o, vtc, zero);
                 // v' uses the adjoint entering the block, scaled to the block end on the own side
                 floatx4 ga[4];
@@ -703,6 +782,11 @@ __device__ __forceinline__ void split_matrix_waves(const ChunkBwdArgs &p, unsign
                     if (side == 1) {
                         const float4 pp = *reinterpret_cast<const float4 *>(cf + F_PP * (CF_TILE / 4));
                         ppv[0] = pp.x; ppv[1] = pp.y; ppv[2] = pp.z; ppv[3] = pp.w;
+                    }
+                    // The state of the block below has had this stage's arithmetic to arrive; it is taken
+                    // before the stores are issued, so that the wait for it never includes them.
+                    if constexpr (NB == 1) {
+                        if (chunk > 0) take_ahead(below);
                     }
                     // one address per array; the four tokens are immediate offsets from it (folded rows)
                     u16 *const pv = d_val + go, *const pg = d_gate + go, *const pa = d_adj + go;
@@ -766,9 +850,10 @@ template <typename IOE, typename OPE, int NB, bool HEADS> int launch(const Chunk
 }
 
 template <typename IOE, typename OPE> int by_nb(const ChunkBwdArgs &a, hipStream_t stream) {
+    if (a.C == 16) return a.heads == 1 ? launch<IOE, OPE, 1, false>(a, stream) : launch<IOE, OPE, 1, true>(a, stream);
     if (a.C == 64) return a.heads == 1 ? launch<IOE, OPE, 4, false>(a, stream) : launch<IOE, OPE, 4, true>(a, stream);
     if (a.C == 32) return a.heads == 1 ? launch<IOE, OPE, 2, false>(a, stream) : launch<IOE, OPE, 2, true>(a, stream);
-    return fail(T2FW_ERR_UNSUPPORTED, "the chunked backward kernel takes checkpoint intervals 32 or 64");
+    return fail(T2FW_ERR_UNSUPPORTED, "the chunked backward kernel takes checkpoint intervals 16, 32 or 64");
 }
 
 }  // namespace

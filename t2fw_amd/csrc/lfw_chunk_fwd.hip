@@ -397,7 +397,7 @@ __device__ __forceinline__ void fwd_matrix_waves(const ChunkFwdArgs &p, unsigned
         const float *AS = reinterpret_cast<const float *>(ops + OFF_AS);
         const float *BL = reinterpret_cast<const float *>(ops + OFF_BL);
         const float *AL = reinterpret_cast<const float *>(ops + OFF_AL);
-        if (ckpt != nullptr) {          // checkpoint interval is a multiple of the step
+        if (ckpt != nullptr && p.C != CH_L) {          // checkpoint interval is a multiple of the step
             if (until_ckpt == 0) {
                 store_state<IOE>(S, ckpt + (b * p.NC + chunk) * (CH_N * CH_N), d, g);
                 until_ckpt = p.C;
@@ -408,6 +408,9 @@ __device__ __forceinline__ void fwd_matrix_waves(const ChunkFwdArgs &p, unsigned
 #pragma unroll
         for (int hh = 0; hh < 2; ++hh) {
             const int tok0 = CH_L * hh;
+            // a checkpoint per block: the state at the start of every block that has a token
+            if (ckpt != nullptr && p.C == CH_L && n * CH_STEP + tok0 < T)
+                store_state<IOE>(S, ckpt + (b * p.NC + 2 * n + hh) * (CH_N * CH_N), d, g);
             // P^T[s,t] = kt_s . qs_t, kept for s <= t, as the A operand of the intra product
             const u16 *krow = KT + (tok0 + r) * TS + 8 * g;
             const u16 *qrow = QT + (tok0 + r) * TS + 8 * g;
