@@ -15,6 +15,8 @@
 //
 // Replaces lfw_cuda_fwd_kernel + the output einsum of the reference
 // (t2fw/csrc/lfw_kernel.cu:18-59, t2fw/csrc/lfw.cpp:45); semantics t2fw/torch.py:21-31.
+#include <type_traits>
+
 #include "lfw_chunk.hpp"
 
 // Build-time diagnostic (-DT2FW_PHASE_TIMERS): workgroup 0 accumulates shader-clock ticks
@@ -377,7 +379,6 @@ __device__ __forceinline__ void fwd_matrix_waves(const ChunkFwdArgs &p, unsigned
             S[j][3] = IOE::to_f32((u16)(v.y >> 16));
         }
     }
-    const int nsteps = (T + CH_STEP - 1) / CH_STEP;
     int until_ckpt = 0;
     int64_t chunk = 0;
     if (tid == 0) {
@@ -385,7 +386,12 @@ __device__ __forceinline__ void fwd_matrix_waves(const ChunkFwdArgs &p, unsigned
         if (clear_other_slot) p.row_flags[chunk_rows_padded(p.B) + b] = 0;
     }
     PHASE_BEGIN();
-    for (int n = 0; n < nsteps; ++n) {
+    // One step (two blocks).  FULL: all 32 tokens exist, which leaves the body without a branch
+    // around its stores, so that the LDS reads of the whole step can be scheduled ahead of the
+    // matrix products that use them.
+    // BLK: a checkpoint per block (inside the step) instead of one every C tokens (at its start).
+    auto step = [&](int n, auto full_c, auto blk_c) {
+        constexpr bool FULL = decltype(full_c)::value, BLK = decltype(blk_c)::value;
         __syncthreads();        // the operand tiles of step n are in LDS
         PHASE_MARK(3);
         const unsigned char *ops = smem + (n & 1) * OPS_BYTES;
@@ -397,7 +403,7 @@ __device__ __forceinline__ void fwd_matrix_waves(const ChunkFwdArgs &p, unsigned
         const float *AS = reinterpret_cast<const float *>(ops + OFF_AS);
         const float *BL = reinterpret_cast<const float *>(ops + OFF_BL);
         const float *AL = reinterpret_cast<const float *>(ops + OFF_AL);
-        if (ckpt != nullptr && p.C != CH_L) {          // checkpoint interval is a multiple of the step
+        if (!BLK && ckpt != nullptr) {          // checkpoint interval is a multiple of the step
             if (until_ckpt == 0) {
                 store_state<IOE>(S, ckpt + (b * p.NC + chunk) * (CH_N * CH_N), d, g);
                 until_ckpt = p.C;
@@ -409,7 +415,7 @@ __device__ __forceinline__ void fwd_matrix_waves(const ChunkFwdArgs &p, unsigned
         for (int hh = 0; hh < 2; ++hh) {
             const int tok0 = CH_L * hh;
             // a checkpoint per block: the state at the start of every block that has a token
-            if (ckpt != nullptr && p.C == CH_L && n * CH_STEP + tok0 < T)
+            if (BLK && (FULL || n * CH_STEP + tok0 < T))
                 store_state<IOE>(S, ckpt + (b * p.NC + 2 * n + hh) * (CH_N * CH_N), d, g);
             // P^T[s,t] = kt_s . qs_t, kept for s <= t, as the A operand of the intra product
             const u16 *krow = KT + (tok0 + r) * TS + 8 * g;
@@ -433,7 +439,7 @@ __device__ __forceinline__ void fwd_matrix_waves(const ChunkFwdArgs &p, unsigned
             // 16 lanes write 32 contiguous bytes of a token row; the four waves complete the row
             const int tg = n * CH_STEP + tok0 + 4 * g;
             u16 *const po = out + ((u32)tg * ts + (u32)d);      // the four tokens: immediate offsets (folded rows)
-            if ((n + 1) * CH_STEP <= T) {
+            if constexpr (FULL) {
 #pragma unroll
                 for (int i = 0; i < 4; ++i) po[i * ts] = cvt1<IOE>((o[i] + oi[i]) * asv[i]);
             } else {
@@ -455,6 +461,14 @@ __device__ __forceinline__ void fwd_matrix_waves(const ChunkFwdArgs &p, unsigned
             }
             PHASE_MARK(hh);
         }
+    };
+    const int nfull = T / CH_STEP;
+    if (ckpt != nullptr && p.C == CH_L) {
+        for (int n = 0; n < nfull; ++n) step(n, std::true_type{}, std::true_type{});
+        if (nfull * CH_STEP < T) step(nfull, std::false_type{}, std::true_type{});
+    } else {
+        for (int n = 0; n < nfull; ++n) step(n, std::true_type{}, std::false_type{});
+        if (nfull * CH_STEP < T) step(nfull, std::false_type{}, std::false_type{});
     }
     store_state<IOE>(S, reinterpret_cast<u16 *>(p.next_state) + b * (CH_N * CH_N), d, g);
     PHASE_END(tid >> 6);
