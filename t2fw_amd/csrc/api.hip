@@ -246,7 +246,7 @@ static int lfw_backward_rows(const void *g_out, const void *g_state, const void 
         c.B = B; c.T = T; c.NC = a.NC; c.C = C;
         c.heads = (int32_t)heads;
         const int op = (dtype == T2FW_F16 && (flags & T2FW_FLAG_FP16_OPERANDS)) ? 1 : 0;
-        if ((rc = chunk_backward(c, dtype, op, st))) return rc;
+        if ((rc = (C == 16 || (flags & 8)) ? chunk_backward(c, dtype, op, st) : chunk_backward_pair(c, dtype, op, st))) return rc;
         a.row_select = c.row_flags;      // rows the chunked form could not take
         if (flags & T2FW_FLAG_NO_FIXUP) return T2FW_OK;
     }

@@ -48,6 +48,8 @@ __host__ __device__ inline int64_t chunk_rows_padded(int64_t B) { return (B + 7)
 int chunk_forward(const ChunkFwdArgs &a, int dtype, int op, bool split, hipStream_t stream);
 // two workgroups per batch row (one per side of the state)
 int chunk_backward(const ChunkBwdArgs &a, int dtype, int op, hipStream_t stream);
+// the same with stages of two blocks (checkpoint intervals 32 and 64)
+int chunk_backward_pair(const ChunkBwdArgs &a, int dtype, int op, hipStream_t stream);
 constexpr int64_t CHUNK_MAX_T = 1 << 24;      // the kernels address a batch row with 32-bit offsets: T * heads must stay below this
 
 #if defined(__HIPCC__)

@@ -496,9 +496,9 @@ __device__ __forceinline__ void split_prep_waves(const ChunkBwdArgs &p, unsigned
             else
                 prep_r<IOE, OPE>(cur, stage, rj, rown, h, c, bad);
             ++s;
-            PHASE_MARK(2);
+            PHASE_MARK(POS >= NR ? 2 : 0);
             __syncthreads();
-            PHASE_MARK(3);
+            PHASE_MARK(POS >= NR ? 3 : 1);
         };
         for (int chunk_tok = (sched.NC - 2) * p.C; chunk_tok >= 0; chunk_tok -= p.C) {
             const int below_tok = max(chunk_tok - p.C, 0);
@@ -538,9 +538,11 @@ __device__ __forceinline__ void split_prep_waves(const ChunkBwdArgs &p, unsigned
     PHASE_END(4 + (tid >> 6));
 }
 
-template <typename IOE, typename OPE, int NB, bool HEADS>
-__device__ __forceinline__ void split_matrix_waves(const ChunkBwdArgs &p, unsigned char *smem, int tid, int64_t b,
-                                                   int side) {
+// SIDE is a template parameter here: the stores at the end of a stage (and the state loads) then
+// carry no branches on it.
+template <typename IOE, typename OPE, int NB, bool HEADS, int SIDE>
+__device__ __forceinline__ void split_matrix_waves(const ChunkBwdArgs &p, unsigned char *smem, int tid, int64_t b) {
+    constexpr int side = SIDE;
     const int w = tid >> 6, l = tid & 63, r = l & 15, g = l >> 4;
     const int ch = 16 * w + r;       // this lane's own-side channel
     const int T = (int)p.T;                              // the launcher admits T < 2^24 only
@@ -828,8 +830,12 @@ __global__ __launch_bounds__(SP_THREADS) void lfw_bwd_chunk_kernel(ChunkBwdArgs 
     const int64_t b = (int)blockIdx.x - side * rows_padded;
     if (b >= p.B) return;
     // both branches execute exactly 2 + (number of stages) workgroup barriers
-    if (tid < 256)
-        split_matrix_waves<IOE, OPE, NB, HEADS>(p, smem, tid, b, side);
+    if (tid < 256) {
+        if (side == 0)
+            split_matrix_waves<IOE, OPE, NB, HEADS, 0>(p, smem, tid, b);
+        else
+            split_matrix_waves<IOE, OPE, NB, HEADS, 1>(p, smem, tid, b);
+    }
     else
         split_prep_waves<IOE, OPE, NB, HEADS>(p, smem, tid - 256, b, side);
 }
