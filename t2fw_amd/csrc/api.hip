@@ -151,7 +151,7 @@ static int lfw_forward_rows(const void *x, const void *f, const void *q, const v
     a.C = ckpt ? C : 1;
     a.NC = ckpt ? t2fw_lfw_num_ckpt(T, C) : 1;
 
-    if (chunk_shape_ok(D, K, dtype, flags) && (ckpt == nullptr || C % 32 == 0 || C == 16) && T * heads < CHUNK_MAX_T &&
+    if (chunk_shape_ok(D, K, dtype, flags) && (ckpt == nullptr || C % 32 == 0) && T * heads < CHUNK_MAX_T &&
         aligned16({x, f, q, k, f_key, s0, out, next_state, ckpt})) {
         if (workspace == nullptr || workspace_bytes < row_flag_bytes(B))
             return fail(T2FW_ERR_WORKSPACE, "workspace of %zu bytes needed, %zu given", row_flag_bytes(B),
@@ -234,7 +234,7 @@ static int lfw_backward_rows(const void *g_out, const void *g_state, const void 
     a.heads = (int32_t)heads;
     a.NC = t2fw_lfw_num_ckpt(T, C);
 
-    if (chunk_shape_ok(D, K, dtype, flags) && (C == 16 || C == 32 || C == 64) && T * heads < CHUNK_MAX_T &&
+    if (chunk_shape_ok(D, K, dtype, flags) && (C == 32 || C == 64) && T * heads < CHUNK_MAX_T &&
         aligned16({g_out, g_state, x, f, q, k, f_key, ckpt, d_x, d_f, d_q, d_k, d_f_key, d_s0})) {
         if (workspace == nullptr || workspace_bytes < row_flag_bytes(B))
             return fail(T2FW_ERR_WORKSPACE, "workspace of %zu bytes needed, %zu given", row_flag_bytes(B),
@@ -246,7 +246,7 @@ static int lfw_backward_rows(const void *g_out, const void *g_state, const void 
         c.B = B; c.T = T; c.NC = a.NC; c.C = C;
         c.heads = (int32_t)heads;
         const int op = (dtype == T2FW_F16 && (flags & T2FW_FLAG_FP16_OPERANDS)) ? 1 : 0;
-        if ((rc = (C == 16 || (flags & 8)) ? chunk_backward(c, dtype, op, st) : chunk_backward_pair(c, dtype, op, st))) return rc;
+        if ((rc = chunk_backward(c, dtype, op, st))) return rc;
         a.row_select = c.row_flags;      // rows the chunked form could not take
         if (flags & T2FW_FLAG_NO_FIXUP) return T2FW_OK;
     }

@@ -27,7 +27,7 @@ struct ChunkFwdArgs {
     void *out, *next_state, *ckpt;     // ckpt may be null
     int32_t *row_flags;                // [2 * chunk_rows_padded(B)]: set to 1 for rows the exact kernels must redo
     int64_t B, T, NC;
-    int32_t C;                         // checkpoint interval: 16 (every block) or a multiple of 32
+    int32_t C;                         // checkpoint interval, multiple of 32
     int32_t heads;                     // 1: rows are [T, 64] slabs; H > 1: row b is head b % H of a [B / H, T, H, 64] tensor
 };
 
@@ -48,8 +48,6 @@ __host__ __device__ inline int64_t chunk_rows_padded(int64_t B) { return (B + 7)
 int chunk_forward(const ChunkFwdArgs &a, int dtype, int op, bool split, hipStream_t stream);
 // two workgroups per batch row (one per side of the state)
 int chunk_backward(const ChunkBwdArgs &a, int dtype, int op, hipStream_t stream);
-// the same with stages of two blocks (checkpoint intervals 32 and 64)
-int chunk_backward_pair(const ChunkBwdArgs &a, int dtype, int op, hipStream_t stream);
 constexpr int64_t CHUNK_MAX_T = 1 << 24;      // the kernels address a batch row with 32-bit offsets: T * heads must stay below this
 
 #if defined(__HIPCC__)

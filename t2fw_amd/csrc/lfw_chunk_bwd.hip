@@ -32,13 +32,26 @@
 //
 // A workgroup has 12 waves.  Matrix wave w (of 4) holds, in fp32 accumulators, the slab of S and
 // of Gb for own channels 16w..16w+15 (all other channels), so that every contraction is local to
-// a wave.  Chunks are visited last to first; inside a chunk a forward sweep ("R" stages, two
-// blocks per stage) recomputes the block-start states from the checkpoint and keeps them as
-// 16-bit MFMA operands in registers, then the blocks are visited last to first ("B" stages).
-// Eight prep waves (B stages: 4 roles x 2 token halves; R stages: 2 blocks x 2 sides x 2 token
-// halves) build the operand tiles of the next stage in double-buffered LDS; one barrier per
-// stage.  Raw inputs go from global memory straight to the prep waves' registers two stages
-// ahead, and the matrix waves store the gradients themselves.
+// a wave.  Chunks (one per checkpoint) are visited last to first.  A chunk needs a forward sweep
+// over its blocks ("R" work: the block-start states, recomputed from the checkpoint and kept as
+// 16-bit MFMA operands in registers) before its blocks can be visited last to first ("B" work:
+// gradients and the adjoint).  R work is light for the matrix waves and heavy for the prep waves, B
+// work the other way round, and with one workgroup barrier per stage a stage is as long as the
+// slower of the two; so a stage here carries the B work of a pair of blocks of chunk c AND the R
+// work of a pair of blocks of chunk c - 1, which no dependence forbids (R needs only the checkpoint):
+//   prologue     R pairs of the last chunk
+//   transition   c -> c - 1, for k = 0 .. NB/2 - 1:  B pair NB/2 - 1 - k of chunk c, R pair k of chunk c - 1
+//   epilogue     B pairs of chunk 0
+// The states recomputed for chunk c - 1 go to the registers of the pair of chunk c that the same
+// stage has just finished with (the two pairs are swapped into place after the transition).
+//
+// Eight prep waves build the operand tiles of the next stage in double-buffered LDS: (block of the
+// pair, own / other side, token half) for the B and for the R part.  In the B part one lane builds
+// the prefix-scaled AND the suffix-scaled operands of its side from one set of gate conversions and
+// one 16-step product.  Raw inputs go from global memory straight to registers, one set per part,
+// refilled in place one stage ahead after their contents have been converted (the refill's address
+// depends on the converted values, so the compiler cannot hoist the loads above the conversions);
+// the matrix waves store the gradients themselves.
 //
 // Replaces lfw_cuda_bwd_kernel and the six einsums of the reference
 // (t2fw/csrc/lfw_kernel.cu:61-102, t2fw/csrc/lfw.cpp:84-93).
@@ -51,102 +64,89 @@ namespace {
 
 using namespace bwd;
 
-constexpr int SP_THREADS = 768;
+constexpr int BW_THREADS = 768;
 constexpr int CC = 20;   // channel-major 16-token tiles: row stride in elements
 
-// ---- LDS layout of one stage buffer (bytes) ----------------------------------------------
+// ---- LDS layout: a stage buffer holds the B tiles of two blocks, then the R tiles of two blocks -----
 constexpr int TM_TILE = CH_L * TS * 2;       // token-major 16-bit tile [16][TS], channels permuted (tm_pos)
 constexpr int CM_TILE = CH_N * CC * 2;       // channel-major 16-bit tile [64][CC]
 constexpr int CF_TILE = CH_N * CC * 4;       // channel-major fp32 tile [64][CC]
 enum { TM_AOS = 0, TM_VOT, TM_VOH, TM_NUM };
-// B stages use the named tiles; an R stage covers two blocks j = 0, 1 and uses tiles 2j (VOH) and 2j+1 (VH)
 enum { CM_AOS = 0, CM_VOH, CM_AS, CM_VT, CM_VH, CM_NUM };
-enum { F_RG = 0, F_IP, F_PP, F_NUM };        // 1/own gate, 1/own prefix, own prefix
+enum { F_RG = 0, F_IP, F_NUM };              // 1/own gate, 1/own prefix (the prefix itself is its reciprocal)
 constexpr int OFF_TM = 0;
 constexpr int OFF_CM = OFF_TM + TM_NUM * TM_TILE;
 constexpr int OFF_CF = OFF_CM + CM_NUM * CM_TILE;
-// 16-step gate products, [block j of an R stage][other side, own side][64] f32 (B stages: j = 0)
-constexpr int OFF_LV = OFF_CF + F_NUM * CF_TILE;
-constexpr int STAGE_BYTES = OFF_LV + 4 * CH_N * 4;
-constexpr int SP_SMEM = 2 * STAGE_BYTES;
-static_assert(SP_SMEM <= 160 * 1024, "backward stage buffers exceed the LDS of one CU");
-static_assert(STAGE_BYTES % 16 == 0, "stage buffers must keep 16-byte alignment");
-
-__device__ __forceinline__ float *lv_vec(unsigned char *stage, int j, int own) {
-    return reinterpret_cast<float *>(stage + OFF_LV) + (2 * j + own) * CH_N;
-}
-__device__ __forceinline__ const float *lv_vec(const unsigned char *stage, int j, int own) {
-    return reinterpret_cast<const float *>(stage + OFF_LV) + (2 * j + own) * CH_N;
-}
+constexpr int OFF_LV = OFF_CF + F_NUM * CF_TILE;      // 16-step gate products [other side, own side][64] f32
+constexpr int BLOCK_BYTES = OFF_LV + 2 * CH_N * 4;
+// R tiles of one block: VOH, VH (channel-major) and the gate products
+constexpr int ROFF_VOH = 0, ROFF_VH = CM_TILE, ROFF_LV = 2 * CM_TILE;
+constexpr int RBLOCK_BYTES = ROFF_LV + 2 * CH_N * 4;
+constexpr int OFF_RPART = 2 * BLOCK_BYTES;
+constexpr int STAGE_BYTES = OFF_RPART + 2 * RBLOCK_BYTES;
+// after the two stage buffers: per matrix wave, room to park its fp32 state slab (64 lanes x 16 floats)
+// while the B part of a stage needs the registers
+constexpr int OFF_PARK = 2 * STAGE_BYTES;
+constexpr int BW_SMEM = OFF_PARK + 4 * 64 * 16 * 4;
+static_assert(BW_SMEM <= 160 * 1024, "backward stage buffers exceed the LDS of one CU");
+static_assert(BLOCK_BYTES % 16 == 0 && RBLOCK_BYTES % 16 == 0, "tile regions must keep 16-byte alignment");
 
 // ---- stage schedule ----------------------------------------------------------------------
-// Chunks are visited from the last one down; a chunk with nb blocks takes ceil(nb/2) "R"
-// stages of two blocks each (forward in time), then nb "B" stages (blocks nb-1..0).
-// A stage is one int: (first token of its first block) * 2 + (1 for a B stage).
-// NB = 1 means a checkpoint per block (C = 16): the state at every block start comes from memory, so
-// only the last block of the sequence takes an R stage (for the state at the end of the sequence).
-template <int NB> struct SplitSchedule {
-    static constexpr unsigned PER_CHUNK = NB == 1 ? 1 : NB / 2 + NB;
-    int NC, C, total, nb_last, st_last;
-    __device__ SplitSchedule(int64_t T, int64_t NC_, int C_) {
+// The last chunk of a sequence may have fewer pairs of blocks than a full one, its last pair one
+// block, its last block fewer than 16 tokens.
+template <int NB> struct StageSchedule {
+    static constexpr int MP = NB / 2;                    // pairs of a full chunk
+    int NC, C, nb_last, m_last, m0, n_trans, total;
+    __device__ StageSchedule(int64_t T, int64_t NC_, int C_) {
         NC = (int)NC_;
         C = C_;
         const int len_last = (int)(T - (NC_ - 1) * C_);
         nb_last = (len_last + CH_L - 1) / CH_L;
-        st_last = (nb_last + 1) / 2 + nb_last;
-        total = st_last + (NC - 1) * (int)PER_CHUNK;
+        m_last = (nb_last + 1) / 2;
+        m0 = NC == 1 ? m_last : MP;                      // pairs of chunk 0
+        n_trans = (NC - 1) * MP;
+        total = m_last + n_trans + m0;
+    }
+    // stage s -> first tokens of the pairs of blocks of its B and R parts (wave-uniform)
+    struct Desc {
+        int tok_b, tok_r;
+        bool has_b, has_r;
+    };
+    __device__ Desc at(int s) const {
+        Desc d;
+        d.tok_b = 0;
+        d.tok_r = 0;
+        if (s < m_last) {
+            d.has_b = false;
+            d.has_r = true;
+            d.tok_r = (NC - 1) * C + s * 2 * CH_L;
+        } else if (s - m_last < n_trans) {
+            const unsigned s2 = (unsigned)(s - m_last);
+            const int c = NC - 1 - (int)(s2 / (unsigned)MP), k = (int)(s2 % (unsigned)MP), pb = MP - 1 - k;
+            d.has_b = 2 * pb < (c == NC - 1 ? nb_last : NB);
+            d.tok_b = c * C + pb * 2 * CH_L;
+            d.has_r = true;
+            d.tok_r = (c - 1) * C + k * 2 * CH_L;
+        } else {
+            const int k = s - m_last - n_trans;
+            d.has_b = true;
+            d.has_r = false;
+            d.tok_b = (m0 - 1 - k) * 2 * CH_L;
+        }
+        return d;
     }
 };
-
-// The same schedule as a forward iterator: cur() is SplitSchedule::at of the stage it stands on;
-// advancing past the last stage leaves it there.  The stages of a chunk are one byte each in a
-// 64-bit table, (block << 1) | (1 for a B stage), so that a step costs a few scalar instructions.
-template <int NB> struct StageIter {
-    static __host__ __device__ constexpr uint64_t table_of(int nb) {
-        uint64_t t = 0;
-        const int nr = (nb + 1) / 2;
-        for (int l = 0; l < nr + nb; ++l) {
-            const uint64_t e = l < nr ? (uint64_t)(2 * l) << 1 : ((uint64_t)(nb - 1 - (l - nr)) << 1) | 1u;
-            t |= e << (8 * l);
-        }
-        return t;
-    }
-    uint64_t table;     // of the chunk it stands in
-    int base2;          // (first token of that chunk) * 2
-    int local, count;   // stage inside the chunk, stages of the chunk
-    int C2, left;       // 2 * C; stages after the current one
-    __device__ StageIter(const SplitSchedule<NB> &sc)
-        : base2((sc.NC - 1) * sc.C * 2), local(0), count(sc.st_last), C2(2 * sc.C), left(sc.total - 1) {
-        table = sc.nb_last == 1 ? table_of(1) : sc.nb_last == 2 ? table_of(2) : sc.nb_last == 3 ? table_of(3) : table_of(4);
-    }
-    __device__ void advance() {
-        if (left > 0) {
-            --left;
-            ++local;
-            if (local == count) {
-                base2 -= C2;
-                local = 0;
-                count = (int)SplitSchedule<NB>::PER_CHUNK;
-                table = NB == 1 ? (uint64_t)1 /* one B stage, block 0 */ : table_of(NB);
-            }
-        }
-    }
-    __device__ int cur() const {
-        const int e = (int)(table >> (8 * local)) & 0xff;       // (block << 1) | bmode
-        return base2 + (e >> 1) * (2 * CH_L) + (e & 1);
-    }
-};
-static_assert(SplitSchedule<4>::PER_CHUNK <= 8, "a chunk's stages must fit the 64-bit table");
 
 // ---- raw inputs --------------------------------------------------------------------------
-// A prep thread works on one channel and eight tokens; it needs the gate at those tokens, the
-// gate at the block's other eight tokens and one value (or adjoint) array at its own tokens:
-// 24 two-byte loads, coalesced over the wave's 64 channels.  They go straight to registers,
-// two stages ahead of their use: the block's first token of an array is a scalar base, the
-// lane's channel and token half a constant vector offset, the token inside the half an
-// immediate one (for rows that are heads of a [B, T, H, 64] tensor see TokenMap).
+// A prep lane works on one channel and eight tokens of one block; it needs the gate at those
+// tokens and at the block's other eight, the value array of its side at its own tokens and, for the
+// B part (ADJ), the adjoint array as well.
 struct RawSet {
-    u16 gown[8], goth[8], val[8];
+    u16 gown[8], goth[8], val[8], adj[8];
+};
+struct RawF {
+    float gown[8], val[8], adj[8], poth;
+    u32 bad;
 };
 
 // Where the sixteen tokens of a block are, seen from a prep lane.  Consecutive tokens are ts elements
@@ -163,15 +163,13 @@ template <bool HEADS> struct TokenMap {
         shift_own = 8u * (u32)h * ts;
         shift_oth = 8u * (u32)(1 - h) * ts;
 #pragma unroll
-        for (int t = 0; t < 8; ++t) {
-            tok_off[t] = 2u * ((u32)c + (u32)t * ts);
-        }
+        for (int t = 0; t < 8; ++t) tok_off[t] = 2u * ((u32)c + (u32)t * ts);
     }
 };
 
-// gate, val: wave-uniform addresses of the block's first token
-template <bool HEADS>
-__device__ __forceinline__ void raw_issue(RawSet &r, const u16 *gate, const u16 *val, TokenMap<HEADS> &m) {
+// gate, val, adj: wave-uniform addresses of the block's first token; all sixteen tokens exist
+template <bool HEADS, bool ADJ>
+__device__ __forceinline__ void raw_issue(RawSet &r, const u16 *gate, const u16 *val, const u16 *adj, TokenMap<HEADS> &m) {
     if constexpr (!HEADS) {
         auto at = [&](const u16 *base, u32 voff, int t) -> u16 {
             return *reinterpret_cast<const u16 *>(reinterpret_cast<const unsigned char *>(base + t * CH_N) + voff);
@@ -182,48 +180,47 @@ __device__ __forceinline__ void raw_issue(RawSet &r, const u16 *gate, const u16 
         for (int t = 0; t < 8; ++t) r.gown[t] = at(gate, m.voff_own, t);
 #pragma unroll
         for (int t = 0; t < 8; ++t) r.val[t] = at(val, m.voff_own, t);
-    } else {
-        // The offsets are made opaque at every use: they then stay in eight 32-bit registers (no
-        // re-derivation from the channel, no widened copies hoisted out of the loops), which is the
-        // form the scalar-base addressing mode of the loads takes.
+        if constexpr (ADJ) {
 #pragma unroll
-        for (int t = 0; t < 8; ++t) asm volatile("" : "+v"(m.tok_off[t]));
+            for (int t = 0; t < 8; ++t) r.adj[t] = at(adj, m.voff_own, t);
+        }
+    } else {
         auto at = [&](const u16 *base, int t) -> u16 {
             return *reinterpret_cast<const u16 *>(reinterpret_cast<const unsigned char *>(base) + m.tok_off[t]);
         };
-        const u16 *const go = gate + m.shift_own, *const gx = gate + m.shift_oth, *const vo = val + m.shift_own;
+        const u16 *const go = gate + m.shift_own, *const gx = gate + m.shift_oth;
+        const u16 *const vo = val + m.shift_own, *const ao = adj + m.shift_own;
 #pragma unroll
         for (int t = 0; t < 8; ++t) r.goth[t] = at(gx, t);
 #pragma unroll
         for (int t = 0; t < 8; ++t) r.gown[t] = at(go, t);
 #pragma unroll
         for (int t = 0; t < 8; ++t) r.val[t] = at(vo, t);
+        if constexpr (ADJ) {
+#pragma unroll
+            for (int t = 0; t < 8; ++t) r.adj[t] = at(ao, t);
+        }
     }
 }
 
-// The same for a block that reaches past the end of the sequence (T % 16 != 0, last chunk only):
-// tokens past the end are read from the last one, with the same number of loads, and replaced by
-// raw_patch_tail when the set is taken.  row_gate, row_val: token 0 of the batch row.
-__device__ __forceinline__ void raw_issue_tail(RawSet &r, const u16 *row_gate, const u16 *row_val, int tok_own,
-                                               int tok_oth, int T, int c, u32 ts) {
-    auto at = [&](const u16 *base, int tok) -> u16 { return base[(u32)min(tok, T - 1) * ts + c]; };
+// The same for a block that reaches past the end of the sequence (or lies past it): tokens past the
+// end are read from the last one, with the same number of loads, and replaced when the set is taken.
+// row_*: token 0 of the batch row.
+template <bool ADJ>
+__device__ __forceinline__ void raw_issue_any(RawSet &r, const u16 *row_gate, const u16 *row_val, const u16 *row_adj,
+                                              int tok_own, int tok_oth, int T, u32 cbytes, u32 ts) {
+    auto at = [&](const u16 *base, int tok) -> u16 {
+        return *reinterpret_cast<const u16 *>(reinterpret_cast<const unsigned char *>(base + (u32)min(tok, T - 1) * ts) + cbytes);
+    };
 #pragma unroll
     for (int t = 0; t < 8; ++t) r.goth[t] = at(row_gate, tok_oth + t);
 #pragma unroll
     for (int t = 0; t < 8; ++t) r.gown[t] = at(row_gate, tok_own + t);
 #pragma unroll
     for (int t = 0; t < 8; ++t) r.val[t] = at(row_val, tok_own + t);
-}
-
-// tokens past the end act as identity: gate 1, everything else 0
-template <typename IOE> __device__ __forceinline__ void raw_patch_tail(RawSet &r, int tok_own, int tok_oth, int T) {
+    if constexpr (ADJ) {
 #pragma unroll
-    for (int t = 0; t < 8; ++t) {
-        if (tok_oth + t >= T) r.goth[t] = IOE::ONE_BITS;
-        if (tok_own + t >= T) {
-            r.gown[t] = IOE::ONE_BITS;
-            r.val[t] = 0;
-        }
+        for (int t = 0; t < 8; ++t) r.adj[t] = at(row_adj, tok_own + t);
     }
 }
 
@@ -237,6 +234,34 @@ template <typename IOE> __device__ __forceinline__ u32 gate_check8(const u16 (&g
     return (mx >= IOE::ONE_BITS) ? 1u : 0u;
 }
 
+
+// Registers -> floats, with the gate range check (gates must lie in (0, 1]) and the product of the
+// other half's gates.  ANY: tokens at or past T act as identity (gate 1, everything else 0).
+template <typename IOE, bool ANY, bool ADJ>
+__device__ __forceinline__ RawF raw_take(const RawSet &r, int tok_own, int tok_oth, int T) {
+    RawF f;
+    // the loads complete in order: one wait for the last of them covers the whole set
+    if constexpr (ADJ)
+        asm volatile("" ::"v"(r.adj[7]));
+    else
+        asm volatile("" ::"v"(r.val[7]));
+    float po = 1.0f;
+    u16 mx = 0;
+#pragma unroll
+    for (int t = 0; t < 8; ++t) {
+        const bool own = !ANY || tok_own + t < T;
+        const u16 m1 = own ? (u16)(r.gown[t] - 1) : (u16)0;      // 0 < bits <= bits(1.0)
+        mx = m1 > mx ? m1 : mx;
+        f.gown[t] = own ? IOE::to_f32(r.gown[t]) : 1.0f;
+        f.val[t] = own ? IOE::to_f32(r.val[t]) : 0.0f;
+        if constexpr (ADJ) f.adj[t] = own ? IOE::to_f32(r.adj[t]) : 0.0f;
+        if (!ANY || tok_oth + t < T) po *= IOE::to_f32(r.goth[t]);
+    }
+    f.poth = po;
+    f.bad = (mx >= IOE::ONE_BITS) ? 1u : 0u;
+    return f;
+}
+
 // eight tokens of one channel as four packed pairs
 struct Packed8 {
     u32 p[4];
@@ -248,8 +273,9 @@ template <typename OPE> __device__ __forceinline__ Packed8 pack8(const float (&v
     return r;
 }
 
-__device__ __forceinline__ void write_tm8(unsigned char *stage, int tile, int c, int t0, const Packed8 &v) {
-    u16 *tm = reinterpret_cast<u16 *>(stage + OFF_TM + tile * TM_TILE) + t0 * TS + tm_pos(c);
+
+__device__ __forceinline__ void write_tm8(unsigned char *blk, int tile, int c, int t0, const Packed8 &v) {
+    u16 *tm = reinterpret_cast<u16 *>(blk + OFF_TM + tile * TM_TILE) + t0 * TS + tm_pos(c);
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
         tm[(2 * i) * TS] = (u16)(v.p[i] & 0xffffu);
@@ -257,279 +283,205 @@ __device__ __forceinline__ void write_tm8(unsigned char *stage, int tile, int c,
     }
 }
 
-__device__ __forceinline__ void write_cm8(unsigned char *stage, int tile, int c, int t0, const Packed8 &v) {
-    uint2 *cm = reinterpret_cast<uint2 *>(stage + OFF_CM + tile * CM_TILE + (c * CC + t0) * 2);
+__device__ __forceinline__ void write_cm8(unsigned char *blk, int tile, int c, int t0, const Packed8 &v) {
+    uint2 *cm = reinterpret_cast<uint2 *>(blk + OFF_CM + tile * CM_TILE + (c * CC + t0) * 2);
     cm[0] = make_uint2(v.p[0], v.p[1]);
     cm[1] = make_uint2(v.p[2], v.p[3]);
 }
 
-__device__ __forceinline__ void write_cf8(unsigned char *stage, int tile, int c, int t0, const float (&v)[8]) {
-    float4 *cf = reinterpret_cast<float4 *>(stage + OFF_CF + tile * CF_TILE + (c * CC + t0) * 4);
+__device__ __forceinline__ void write_cf8(unsigned char *blk, int tile, int c, int t0, const float (&v)[8]) {
+    float4 *cf = reinterpret_cast<float4 *>(blk + OFF_CF + tile * CF_TILE + (c * CC + t0) * 4);
     cf[0] = make_float4(v[0], v[1], v[2], v[3]);
     cf[1] = make_float4(v[4], v[5], v[6], v[7]);
 }
 
-template <typename IOE> __device__ __forceinline__ float product8(const u16 (&g)[8]) {
-    float p = IOE::mul2(g[0], g[1]);
-#pragma unroll
-    for (int t = 2; t < 8; ++t) p = IOE::mul(g[t], p);
-    return p;
+__device__ __forceinline__ float *lv_vec(unsigned char *blk, int own) {
+    return reinterpret_cast<float *>(blk + OFF_LV) + own * CH_N;
+}
+__device__ __forceinline__ const float *lv_vec(const unsigned char *blk, int own) {
+    return reinterpret_cast<const float *>(blk + OFF_LV) + own * CH_N;
 }
 
-// Gate-suffix scalings of one half block: hat = v * prod_{r>t} gate_r, til = hat / total,
-// inv = 1 / prod_{r<=t} gate_r; returns the 16-step product.
-template <typename IOE, typename OPE>
-__device__ __forceinline__ float suffix_scale(const RawSet &r, int h, bool check, float (&hat)[8], float (&til)[8],
-                                              float (&inv)[8], u32 &bad) {
-    const float poth = product8<IOE>(r.goth);
-    const float tot = product8<IOE>(r.gown) * poth;
-    if (check) bad |= gate_check8<IOE>(r.gown);
+// Gate scalings of one half block (tokens 8h..8h+7) of one channel: pre = prod_{r<=t} gate_r from the
+// block start, inv = 1 / pre, hat = v * prod_{r>t} gate_r (scaled to the block end), til = hat / total
+// (scaled to the block start); returns the 16-step product.
+template <typename OPE>
+__device__ __forceinline__ float scale_half(const RawF &f, int h, float (&pre)[8], float (&hat)[8], float (&til)[8],
+                                            float (&inv)[8], u32 &bad) {
+    float run = h ? f.poth : 1.0f;
+#pragma unroll
+    for (int t = 0; t < 8; ++t) {
+        run *= f.gown[t];
+        pre[t] = run;
+    }
+    const float tot = h ? run : run * f.poth;
     bad |= (tot >= OPE::MIN_PRODUCT) ? 0u : 1u;
     const float itot = __builtin_amdgcn_rcpf(tot);
-    float sfx = h ? 1.0f : poth;
+    float sfx = h ? 1.0f : f.poth;
 #pragma unroll
     for (int t = 7; t >= 0; --t) {
         inv[t] = sfx * itot;
-        hat[t] = IOE::mul(r.val[t], sfx);
+        hat[t] = f.val[t] * sfx;
         til[t] = hat[t] * itot;
-        sfx = IOE::mul(r.gown[t], sfx);
+        sfx *= f.gown[t];
     }
     return tot;
 }
 
-// B stage, one prep wave: one role, tokens 8h..8h+7 of the block, channel c.
-//   role 0: other gate prefix -> AOS (token- and channel-major)
-//   role 1: other gate suffix -> VOH (both layouts), VOT (token-major), L_other
-//   role 2: own gate prefix   -> AS, 1/gate, prefix (side 1)
-//   role 3: own gate suffix   -> VH, VT, 1/prefix, L_own
-template <typename IOE, typename OPE>
-__device__ __forceinline__ void prep_b(const RawSet &r, unsigned char *stage, int role, int h, int c, bool want_pp,
-                                       u32 &bad) {
-    const bool other = role < 2;
+// R part, one prep lane (tokens 8h..8h+7 of one block, channel c, own or other side): the
+// suffix-scaled values (VH | VOH, channel-major) and the 16-step gate product.
+template <typename OPE>
+__device__ __forceinline__ void prep_lane_r(const RawF &f, unsigned char *rblk, int own, int h, int c, u32 &bad) {
+    float pre[8], hat[8], til[8], inv[8];
+    const float tot = scale_half<OPE>(f, h, pre, hat, til, inv, bad);
+    if (h == 0) reinterpret_cast<float *>(rblk + ROFF_LV)[own * CH_N + c] = tot;
+    const Packed8 hp = pack8<OPE>(hat);
+    uint2 *cm = reinterpret_cast<uint2 *>(rblk + (own ? ROFF_VH : ROFF_VOH) + (c * CC + 8 * h) * 2);
+    cm[0] = make_uint2(hp.p[0], hp.p[1]);
+    cm[1] = make_uint2(hp.p[2], hp.p[3]);
+}
+
+// B part, one prep lane.
+//   other side: AOS (token- and channel-major), VOH (both), VOT (token-major), L_other
+//   own side  : AS, VH, VT (channel-major), 1/gate, 1/prefix, L_own
+template <typename OPE>
+__device__ __forceinline__ void prep_lane_b(const RawF &f, unsigned char *blk, int own, int h, int c, u32 &bad) {
     const int t0 = 8 * h;
-    if ((role & 1) == 0) {
-        const float base = h ? product8<IOE>(r.goth) : 1.0f;
-        float run = base;
-        float pre[8], v[8];
+    float pre[8], hat[8], til[8], inv[8];
+    const float tot = scale_half<OPE>(f, h, pre, hat, til, inv, bad);
+    bad |= f.bad;                        // every block's gates are range-checked in its B part
+    if (h == 0) lv_vec(blk, own)[c] = tot;
+    float v[8];
 #pragma unroll
-        for (int t = 0; t < 8; ++t) {
-            run = IOE::mul(r.gown[t], run);
-            pre[t] = run;
-            v[t] = IOE::mul(r.val[t], run);
-        }
-        const Packed8 vp = pack8<OPE>(v);
-        if (other) {
-            write_tm8(stage, TM_AOS, c, t0, vp);
-            write_cm8(stage, CM_AOS, c, t0, vp);
-        } else {
-            // 1/gate_t = prefix_{t-1} / prefix_t from one reciprocal and the running products
-            float ipre = __builtin_amdgcn_rcpf(pre[7]);
-            float rg[8];
-#pragma unroll
-            for (int t = 7; t >= 1; --t) {
-                rg[t] = pre[t - 1] * ipre;
-                ipre = IOE::mul(r.gown[t], ipre);
-            }
-            rg[0] = base * ipre;
-            write_cm8(stage, CM_AS, c, t0, vp);
-            write_cf8(stage, F_RG, c, t0, rg);
-            if (want_pp) write_cf8(stage, F_PP, c, t0, pre);
-        }
+    for (int t = 0; t < 8; ++t) v[t] = f.adj[t] * pre[t];
+    const Packed8 vp = pack8<OPE>(v), hp = pack8<OPE>(hat), tp = pack8<OPE>(til);
+    if (!own) {
+        write_tm8(blk, TM_AOS, c, t0, vp);
+        write_cm8(blk, CM_AOS, c, t0, vp);
+        write_cm8(blk, CM_VOH, c, t0, hp);
+        write_tm8(blk, TM_VOH, c, t0, hp);
+        write_tm8(blk, TM_VOT, c, t0, tp);
     } else {
-        float hat[8], til[8], inv[8];
-        const float tot = suffix_scale<IOE, OPE>(r, h, true, hat, til, inv, bad);
-        if (h == 0) lv_vec(stage, 0, other ? 0 : 1)[c] = tot;
-        const Packed8 hp = pack8<OPE>(hat), tp = pack8<OPE>(til);
-        if (other) {
-            write_cm8(stage, CM_VOH, c, t0, hp);
-            write_tm8(stage, TM_VOH, c, t0, hp);
-            write_tm8(stage, TM_VOT, c, t0, tp);
-        } else {
-            write_cm8(stage, CM_VH, c, t0, hp);
-            write_cm8(stage, CM_VT, c, t0, tp);
-            write_cf8(stage, F_IP, c, t0, inv);
-        }
+        float rg[8];                     // 1/gate_t = prefix_{t-1} / prefix_t
+        rg[0] = (h ? f.poth : 1.0f) * inv[0];
+#pragma unroll
+        for (int t = 1; t < 8; ++t) rg[t] = pre[t - 1] * inv[t];
+        write_cm8(blk, CM_AS, c, t0, vp);
+        write_cm8(blk, CM_VH, c, t0, hp);
+        write_cm8(blk, CM_VT, c, t0, tp);
+        write_cf8(blk, F_RG, c, t0, rg);
+        write_cf8(blk, F_IP, c, t0, inv);
     }
 }
 
-// R stage, one prep wave: block j of the pair, own or other side, tokens 8h..8h+7, channel c:
-// the suffix-scaled values (channel-major) and the 16-step gate product.  (Every block's gates
-// are range-checked in its B stage.)
-template <typename IOE, typename OPE>
-__device__ __forceinline__ void prep_r(const RawSet &r, unsigned char *stage, int j, int own, int h, int c, u32 &bad) {
-    float hat[8], til[8], inv[8];
-    const float tot = suffix_scale<IOE, OPE>(r, h, false, hat, til, inv, bad);
-    if (h == 0) lv_vec(stage, j, own)[c] = tot;
-    write_cm8(stage, 2 * j + own, c, 8 * h, pack8<OPE>(hat));
-}
-
 template <typename IOE, typename OPE, int NB, bool HEADS>
-__device__ __forceinline__ void split_prep_waves(const ChunkBwdArgs &p, unsigned char *smem, int tid, int64_t b,
-                                                 int side) {
+__device__ __forceinline__ void bwd_prep_waves(const ChunkBwdArgs &p, unsigned char *smem, int tid, int64_t b,
+                                                int side) {
     const int pw = __builtin_amdgcn_readfirstlane(tid >> 6), c = tid & 63;
-    // B stages: SIMD-balanced assignment of (role, token half); roles 1 and 3 are the heavier ones
-    const int h = pw >> 2;
-    const int role = (h ? (pw ^ 1) : pw) & 3;
-    // R stages: (block of the pair, side, token half)
-    const int rj = (pw >> 1) & 1, rown = pw & 1;
+    // (block of the pair, own / other side, token half); each SIMD gets an own-side and an other-side wave
+    const int jb = (pw >> 1) & 1, own = pw & 1, h = pw >> 2;
     const int T = (int)p.T;                              // the launcher admits T * heads < 2^24 only
     const int64_t row_off = row_first_token(b, p.T, HEADS ? p.heads : 1) * CH_N;
-    // this batch row of: other gate, other value, own gate, own value, other adjoint, own adjoint
     const u16 *const x = reinterpret_cast<const u16 *>(p.x) + row_off, *const f = reinterpret_cast<const u16 *>(p.f) + row_off;
     const u16 *const g = reinterpret_cast<const u16 *>(p.g_out) + row_off, *const k = reinterpret_cast<const u16 *>(p.k) + row_off;
     const u16 *const fk = reinterpret_cast<const u16 *>(p.f_key) + row_off, *const q = reinterpret_cast<const u16 *>(p.q) + row_off;
-    const u16 *const GO = side == 0 ? fk : f, *const VO = side == 0 ? k : x, *const GW = side == 0 ? f : fk;
-    const u16 *const VW = side == 0 ? x : k, *const AO = side == 0 ? q : g, *const AW = side == 0 ? g : q;
-    // the two arrays this wave reads in B stages and in R stages
-    const u16 *const b_gate = role < 2 ? GO : GW;
-    const u16 *const b_val = role == 0 ? AO : role == 1 ? VO : role == 2 ? AW : VW;
-    const u16 *const r_gate = rown ? GW : GO;
-    const u16 *const r_val = rown ? VW : VO;
-    const SplitSchedule<NB> sched(p.T, p.NC, p.C);
-    u32 bad = 0;
-
+    // this wave's side of the state: value side = (x, f, g_out), key side = (k, f_key, q)
+    const bool value_side = (side == 0) == (own == 1);
+    const u16 *const gate = value_side ? f : fk, *const val = value_side ? x : k, *const adj = value_side ? g : q;
+    const StageSchedule<NB> sched(p.T, p.NC, p.C);
     TokenMap<HEADS> tmap(HEADS ? (u32)p.heads * CH_N : (u32)CH_N, h, c);
     const u32 ts = tmap.ts;                              // elements between consecutive tokens
-    // first token of the block this wave works on in stage st (R stages cover a pair of blocks)
-    auto block_tok = [&](int st) -> int { return (st >> 1) + ((st & 1) ? 0 : rj * CH_L); };
-    auto issue = [&](RawSet &r, int st) {          // raw inputs of stage st (wave-uniform) -> registers
-        const bool bmode = st & 1;
-        const int tok = block_tok(st);
-        const u16 *const gate = bmode ? b_gate : r_gate, *const val = bmode ? b_val : r_val;
-        if (tok + CH_L <= T)
-            raw_issue<HEADS>(r, gate + (u32)tok * ts, val + (u32)tok * ts, tmap);
-        else        // the block reaches past the end (or, second block of the last R pair, lies past it)
-            raw_issue_tail(r, gate, val, tok + 8 * h, tok + 8 * (1 - h), T, c, ts);
-    };
-    // Three register sets rotate: the tiles of stage s are built from `cur`, which was loaded two
-    // stages ago, while `refill` (used up in the stage before) takes the raw inputs of stage s + 2.
-    // The loads are unconditional (past the end: the last stage again), so that the number of loads
-    // in flight is the same on every path and the waits for them can be exact.
-    StageIter<NB> it_load(sched);
-    int st_cur = 0, st_next = 0;                   // descriptors of stages s and s + 1
+    u32 bad = 0;
     PHASE_BEGIN();
-    auto prepare = [&](const RawSet &cur, RawSet &refill, int s) {
-        const int st = st_cur;
-        it_load.advance();
-        const int st_new = it_load.cur();
-        issue(refill, st_new);
-        st_cur = st_next;
-        st_next = st_new;
-        // the loads complete in order: one wait for the last of `cur` covers the whole set
-        asm volatile("" ::"v"(cur.val[7]));
-        RawSet raw = cur;
-        const int tok = block_tok(st);
-        if (tok + CH_L > T) raw_patch_tail<IOE>(raw, tok + 8 * h, tok + 8 * (1 - h), T);
-        unsigned char *stage = smem + (s & 1) * STAGE_BYTES;
-        if (st & 1)
-            prep_b<IOE, OPE>(raw, stage, role, h, c, side == 1, bad);
+
+    // Raw inputs of a part of a stage -> registers; tok: first token of the part's pair of blocks.
+    // ANY: the block may reach past the end of the sequence or lie past it; the loads then go through
+    // clamped per-token addresses, which is correct for every block but slow.
+    auto issue = [&](RawSet &r, int tok, auto any_c, auto adj_c) {
+        constexpr bool ADJ = decltype(adj_c)::value;
+        tok += jb * CH_L;                                // this wave's block of the pair
+        if constexpr (decltype(any_c)::value)
+            raw_issue_any<ADJ>(r, gate, val, adj, tok + 8 * h, tok + 8 * (1 - h), T, 2u * (u32)c, ts);
         else
-            prep_r<IOE, OPE>(raw, stage, rj, rown, h, c, bad);
+            raw_issue<HEADS, ADJ>(r, gate + (u32)tok * ts, val + (u32)tok * ts, adj + (u32)tok * ts, tmap);
+    };
+    // The loads that refill a set must come after the conversion of its contents, or they need
+    // registers (and a wait) of their own: their addresses are tied to the converted values.
+    auto tie = [&](const RawF &fl, auto adj_c) {
+        asm volatile(""
+                     : "+v"(tmap.voff_own), "+v"(tmap.voff_oth)
+                     : "v"(fl.gown[0]), "v"(fl.gown[1]), "v"(fl.gown[2]), "v"(fl.gown[3]), "v"(fl.gown[4]), "v"(fl.gown[5]),
+                       "v"(fl.gown[6]), "v"(fl.gown[7]), "v"(fl.val[0]), "v"(fl.val[1]), "v"(fl.val[2]), "v"(fl.val[3]),
+                       "v"(fl.val[4]), "v"(fl.val[5]), "v"(fl.val[6]), "v"(fl.val[7]), "v"(fl.poth), "v"(fl.bad));
+        if constexpr (decltype(adj_c)::value) {
+            asm volatile(""
+                         : "+v"(tmap.voff_own), "+v"(tmap.voff_oth)
+                         : "v"(fl.adj[0]), "v"(fl.adj[1]), "v"(fl.adj[2]), "v"(fl.adj[3]), "v"(fl.adj[4]), "v"(fl.adj[5]),
+                           "v"(fl.adj[6]), "v"(fl.adj[7]));
+        }
+        if constexpr (HEADS) {
+#pragma unroll
+            for (int t = 0; t < 8; ++t) asm volatile("" : "+v"(tmap.tok_off[t]) : "v"(tmap.voff_own));
+        }
+    };
+    // One stage: this wave's tiles of the B part from setB and of the R part from setR; each set takes
+    // the raw inputs of the next stage as soon as its contents are converted.  A part that the stage
+    // does not have still loads (from the start of the row): the number of loads in flight is the
+    // same on every path, so the waits for them are exact.
+    RawSet setB, setR;
+    using Desc = typename StageSchedule<NB>::Desc;
+    auto stage = [&](int s, const Desc cur, auto any_cur, auto any_next) {
+        constexpr bool ANY = decltype(any_cur)::value;
+        const Desc nxt = sched.at(min(s + 1, sched.total - 1));
+        unsigned char *const buf = smem + (s & 1) * STAGE_BYTES;
+        {
+            const int tok = cur.tok_b + jb * CH_L;
+            const RawF fl = raw_take<IOE, ANY, true>(setB, tok + 8 * h, tok + 8 * (1 - h), T);
+            tie(fl, std::true_type{});
+            issue(setB, nxt.tok_b, any_next, std::true_type{});
+            if (cur.has_b) prep_lane_b<OPE>(fl, buf + jb * BLOCK_BYTES, own, h, c, bad);
+        }
+        {
+            const int tok = cur.tok_r + jb * CH_L;
+            const RawF fl = raw_take<IOE, ANY, false>(setR, tok + 8 * h, tok + 8 * (1 - h), T);
+            tie(fl, std::false_type{});
+            issue(setR, nxt.tok_r, any_next, std::false_type{});
+            if (cur.has_r) prep_lane_r<OPE>(fl, buf + OFF_RPART + jb * RBLOCK_BYTES, own, h, c, bad);
+        }
         PHASE_MARK(2);
         __syncthreads();
         PHASE_MARK(3);
     };
-
-    // Stages are done in triples (sets A, B, C in turn) with no exit inside a triple, so that the
-    // order of the loads in flight is the same on every path.  First the stages of the last chunk of
-    // the sequence (it may be short), with the general iterator; its first (count % 3) stages are
-    // peeled off, with the sets assigned so that the triples start on A.
-    RawSet setA, setB, setC;
-    int s = 0;
-    // (with a checkpoint per block, also as many of the following blocks as make the rest a multiple of three)
-    const int n_last = sched.st_last + (NB == 1 ? (sched.NC - 1) % 3 : 0);
-    const int rem = n_last % 3;
-    st_cur = it_load.cur();
-    it_load.advance();
-    st_next = it_load.cur();
-    if (rem == 0) {
-        issue(setA, st_cur);
-        issue(setB, st_next);
-    } else if (rem == 1) {
-        issue(setC, st_cur);
-        issue(setA, st_next);
-        prepare(setC, setB, 0);
-        s = 1;
-    } else {
-        issue(setB, st_cur);
-        issue(setC, st_next);
-        prepare(setB, setA, 0);
-        prepare(setC, setB, 1);
-        s = 2;
-    }
-    for (; s < n_last; s += 3) {
-        prepare(setA, setC, s);
-        prepare(setB, setA, s + 1);
-        prepare(setC, setB, s + 2);
-    }
-
-    if constexpr (NB != 1) {
-        // Then the full chunks, last to first.  Inside a chunk the kind of every stage and its block are
-        // compile-time constants (position POS of PER), which leaves a pointer bump per stage for the
-        // scalar unit; PER is a multiple of three, so every chunk starts on set A.  The refill of
-        // position POS + 2 reaches into the chunk below for the last two positions (below the first
-        // chunk: that chunk again, never used).
-        constexpr int PER = (int)SplitSchedule<NB>::PER_CHUNK, NR = NB / 2;
-        static_assert(PER % 3 == 0, "a chunk must take a whole number of register-set triples");
-        const u16 *const r_gate_w = r_gate + (u32)(rj * CH_L) * ts, *const r_val_w = r_val + (u32)(rj * CH_L) * ts;
-        auto issue_at = [&](RawSet &r, int chunk_tok, auto pos_c) {
-            constexpr int POS = decltype(pos_c)::value;
-            if constexpr (POS < NR) {
-                const u32 e = (u32)(chunk_tok + 2 * POS * CH_L) * ts;
-                raw_issue<HEADS>(r, r_gate_w + e, r_val_w + e, tmap);
-            } else {
-                const u32 e = (u32)(chunk_tok + (NB - 1 - (POS - NR)) * CH_L) * ts;
-                raw_issue<HEADS>(r, b_gate + e, b_val + e, tmap);
-            }
-        };
-        auto prepare_at = [&](const RawSet &cur, RawSet &refill, int chunk_tok, int below_tok, auto pos_c) {
-            constexpr int POS = decltype(pos_c)::value;
-            if constexpr (POS + 2 < PER)
-                issue_at(refill, chunk_tok, std::integral_constant<int, (POS + 2) % PER>{});
-            else
-                issue_at(refill, below_tok, std::integral_constant<int, (POS + 2) % PER>{});
-            // the loads complete in order: one wait for the last of `cur` covers the whole set
-            asm volatile("" ::"v"(cur.val[7]));
-            unsigned char *stage = smem + (s & 1) * STAGE_BYTES;
-            if constexpr (POS >= NR)
-                prep_b<IOE, OPE>(cur, stage, role, h, c, side == 1, bad);
-            else
-                prep_r<IOE, OPE>(cur, stage, rj, rown, h, c, bad);
-            ++s;
-            PHASE_MARK(POS >= NR ? 2 : 0);
-            __syncthreads();
-            PHASE_MARK(POS >= NR ? 3 : 1);
-        };
-        for (int chunk_tok = (sched.NC - 2) * p.C; chunk_tok >= 0; chunk_tok -= p.C) {
-            const int below_tok = max(chunk_tok - p.C, 0);
-            prepare_at(setA, setC, chunk_tok, below_tok, std::integral_constant<int, 0>{});
-            prepare_at(setB, setA, chunk_tok, below_tok, std::integral_constant<int, 1>{});
-            prepare_at(setC, setB, chunk_tok, below_tok, std::integral_constant<int, 2>{});
-            if constexpr (PER == 6) {
-                prepare_at(setA, setC, chunk_tok, below_tok, std::integral_constant<int, 3>{});
-                prepare_at(setB, setA, chunk_tok, below_tok, std::integral_constant<int, 4>{});
-                prepare_at(setC, setB, chunk_tok, below_tok, std::integral_constant<int, 5>{});
-            }
+    // Blocks can be partial or missing only in the last chunk, i.e. in the prologue and the first
+    // transition: those stages go through the general loader unless that chunk is full.  Parts that a
+    // stage does not have load from the start of the row, which the fast loader may do as soon as the
+    // row has more than one chunk (or one full one).
+    const bool last_full = p.T % p.C == 0;
+    const int n1 = last_full ? 0 : sched.m_last + min(sched.NC - 1, 1) * StageSchedule<NB>::MP;
+    const int n2 = (sched.NC > 1 || last_full) ? sched.total : sched.m_last + sched.n_trans;
+    {
+        const Desc d0 = sched.at(0);
+        if (n1 > 0) {
+            issue(setB, d0.tok_b, std::true_type{}, std::true_type{});
+            issue(setR, d0.tok_r, std::true_type{}, std::false_type{});
+        } else {
+            issue(setB, d0.tok_b, std::false_type{}, std::true_type{});
+            issue(setR, d0.tok_r, std::false_type{}, std::false_type{});
         }
-    } else {
-        // A checkpoint per block: what is left are B stages of full blocks, a multiple of three of
-        // them, last to first; set A holds the highest one, set B the one below it.
-        auto prepare_block = [&](const RawSet &cur, RawSet &refill, int refill_tok) {
-            const u32 e = (u32)max(refill_tok, 0) * ts;      // below the first block: that block again, never used
-            raw_issue<HEADS>(refill, b_gate + e, b_val + e, tmap);
-            // the loads complete in order: one wait for the last of `cur` covers the whole set
-            asm volatile("" ::"v"(cur.val[7]));
-            prep_b<IOE, OPE>(cur, smem + (s & 1) * STAGE_BYTES, role, h, c, side == 1, bad);
-            ++s;
-            PHASE_MARK(2);
-            __syncthreads();
-            PHASE_MARK(3);
-        };
-        const int nblocks = (sched.NC - 1) / 3 * 3;
-        for (int tok = (nblocks - 1) * CH_L; tok >= 0; tok -= 3 * CH_L) {
-            prepare_block(setA, setC, tok - 2 * CH_L);
-            prepare_block(setB, setA, tok - 3 * CH_L);
-            prepare_block(setC, setB, tok - 4 * CH_L);
+    }
+    for (int s = 0; s < sched.total; ++s) {
+        const Desc cur = sched.at(s);
+        const bool any_cur = s < n1 || s >= n2, any_next = s + 1 < n1 || s + 1 >= n2;
+        if (any_cur) {
+            if (any_next)
+                stage(s, cur, std::true_type{}, std::true_type{});
+            else
+                stage(s, cur, std::true_type{}, std::false_type{});
+        } else {
+            if (any_next)
+                stage(s, cur, std::false_type{}, std::true_type{});
+            else
+                stage(s, cur, std::false_type{}, std::false_type{});
         }
     }
     // Both workgroups of a row see all four gates' blocks and reach the same verdict, so either
@@ -538,19 +490,16 @@ __device__ __forceinline__ void split_prep_waves(const ChunkBwdArgs &p, unsigned
     PHASE_END(4 + (tid >> 6));
 }
 
-// SIDE is a template parameter here: the stores at the end of a stage (and the state loads) then
-// carry no branches on it.
 template <typename IOE, typename OPE, int NB, bool HEADS, int SIDE>
-__device__ __forceinline__ void split_matrix_waves(const ChunkBwdArgs &p, unsigned char *smem, int tid, int64_t b) {
+__device__ __forceinline__ void bwd_matrix_waves(const ChunkBwdArgs &p, unsigned char *smem, int tid, int64_t b) {
     constexpr int side = SIDE;
     const int w = tid >> 6, l = tid & 63, r = l & 15, g = l >> 4;
     const int ch = 16 * w + r;       // this lane's own-side channel
-    const int T = (int)p.T;                              // the launcher admits T < 2^24 only
+    const int T = (int)p.T;                              // the launcher admits T * heads < 2^24 only
     const int64_t NC = p.NC;
     const int C = p.C;
     const u16 *ckpt = reinterpret_cast<const u16 *>(p.ckpt) + b * NC * (CH_N * CH_N);
     const int nb_last = (int)((p.T - (NC - 1) * C + CH_L - 1) / CH_L);
-    // this batch row of the gradients this side writes
     const int64_t row_off = row_first_token(b, p.T, HEADS ? p.heads : 1) * CH_N;
     const u32 ts = HEADS ? (u32)p.heads * CH_N : (u32)CH_N;       // elements between consecutive tokens
     u16 *const d_val = reinterpret_cast<u16 *>(side == 0 ? p.d_x : p.d_k) + row_off;
@@ -586,59 +535,6 @@ __device__ __forceinline__ void split_matrix_waves(const ChunkBwdArgs &p, unsign
     load_state(reinterpret_cast<const u16 *>(p.g_state) + b * (CH_N * CH_N), pf);
     take_state(pf, G);
     load_state(ckpt + (NC - 1) * (CH_N * CH_N), pf);
-    // A checkpoint per block (NB = 1): the block-start state of every block but the last comes
-    // straight from memory: raw loads (side 0: four 8-byte loads, side 1: sixteen 2-byte loads of a
-    // column) issued at the start of the stage above and put together at its end; `top` keeps the raw
-    // state of the latest block whose start is a multiple of four blocks (for the anchor).
-    u32 ahead[NB == 1 ? 16 : 1];
-    uint2 below[4] = {};             // raw start state of the block below the current one
-    uint2 top[4] = {pf[0], pf[1], pf[2], pf[3]};
-    auto fetch_ahead = [&](const u16 *m) {
-        if (side == 0) {
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const uint2 v = ld2(m + ch * CH_N + 16 * j + 4 * g);
-                ahead[(2 * j) % (NB == 1 ? 16 : 1)] = v.x;
-                ahead[(2 * j + 1) % (NB == 1 ? 16 : 1)] = v.y;
-            }
-#pragma unroll
-            for (int j = 8; j < (NB == 1 ? 16 : 1); ++j) ahead[j] = 0;
-        } else {
-#pragma unroll
-            for (int j = 0; j < 4; ++j)
-#pragma unroll
-                for (int i = 0; i < 4; ++i) ahead[(4 * j + i) % (NB == 1 ? 16 : 1)] = m[(16 * j + 4 * g + i) * CH_N + ch];
-        }
-    };
-    auto take_ahead = [&](uint2 (&dst)[4]) {
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            constexpr int M = NB == 1 ? 16 : 1;
-            if (side == 0)
-                dst[j] = make_uint2(ahead[(2 * j) % M], ahead[(2 * j + 1) % M]);
-            else
-                dst[j] = make_uint2(ahead[(4 * j) % M] | (ahead[(4 * j + 1) % M] << 16),
-                                    ahead[(4 * j + 2) % M] | (ahead[(4 * j + 3) % M] << 16));
-        }
-    };
-    // raw state (I/O type, four values per 32-bit pair) -> the two MFMA operands
-    auto to_operands = [&](const uint2 (&raw)[4], uint4 &lo, uint4 &hi) {
-        if constexpr (std::is_same<IOE, OPE>::value) {
-            lo = cat(raw[0], raw[1]);
-            hi = cat(raw[2], raw[3]);
-        } else {
-            uint2 o[4];
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                float t[4];
-                unpack4<IOE>(raw[j], t);
-                const floatx4 v = {t[0], t[1], t[2], t[3]};
-                o[j] = pack4v<OPE>(v);
-            }
-            lo = cat(o[0], o[1]);
-            hi = cat(o[2], o[3]);
-        }
-    };
     float carry = 0.f;
     int s = 0;
     if (tid == 0) {      // both flag slots of the row (the backward kernels report in the first)
@@ -647,168 +543,219 @@ __device__ __forceinline__ void split_matrix_waves(const ChunkBwdArgs &p, unsign
     }
     PHASE_BEGIN();
 
-    // every stage starts with the workgroup barrier that publishes its operand tiles
-    for (int64_t chunk = NC - 1; chunk >= 0; --chunk) {
-        const bool last = chunk == NC - 1;
-        const int nb = last ? nb_last : NB;
-        const bool recompute = NB != 1 || last;              // this chunk has R stages
-        if (recompute) {
-            take_state(pf, S);
-            if (NB != 1 && chunk > 0) load_state(ckpt + (chunk - 1) * (CH_N * CH_N), pf);
-        }
-        // ---- R stages: block-start states, forward in time, two blocks per stage
+    // R part of a stage: the states at the start of blocks i2 and i2 + 1 of a chunk with nbc blocks
+    // (S runs forward over them), as MFMA operands into d0 and d1
+    auto r_pair = [&](const unsigned char *stage, int nbc, int i2, uint4 (&d0)[2], uint4 (&d1)[2]) {
 #pragma unroll
-        for (int i2 = 0; i2 < NB; i2 += 2) {
-            if (i2 < nb && recompute) {
-                __syncthreads();
-                PHASE_MARK(3);
-                const unsigned char *stage = smem + (s & 1) * STAGE_BYTES;
-#pragma unroll
-                for (int jb = 0; jb < 2; ++jb) {
-                    const int i = (i2 + jb) % NB;           // (i2 + jb < NB wherever the branch below is taken)
-                    if (i2 + jb < nb) {
-                        const u16 *VOHc = reinterpret_cast<const u16 *>(stage + OFF_CM + (2 * jb) * CM_TILE);
-                        const u16 *VHc = reinterpret_cast<const u16 *>(stage + OFF_CM + (2 * jb + 1) * CM_TILE);
-                        const float *LX = lv_vec(stage, jb, 0), *LO = lv_vec(stage, jb, 1);
-                        {
-                            const uint2 a0 = pack4v<OPE>(S[0]), a1 = pack4v<OPE>(S[1]), a2 = pack4v<OPE>(S[2]),
-                                        a3 = pack4v<OPE>(S[3]);
-                            sv[i][0] = cat(a0, a1);
-                            sv[i][1] = cat(a2, a3);
-                        }
-                        const float lo = LO[ch];
-                        const uint2 vhc = ld2(VHc + ch * CC + 4 * g);
-#pragma unroll
-                        for (int j = 0; j < 4; ++j) {
-                            const float4 lx = *reinterpret_cast<const float4 *>(LX + 16 * j + 4 * g);
-                            S[j][0] *= lo * lx.x; S[j][1] *= lo * lx.y; S[j][2] *= lo * lx.z; S[j][3] *= lo * lx.w;
-                            S[j] = OPE::mfma16(ld2(VOHc + (16 * j + r) * CC + 4 * g), vhc, S[j]);
-                        }
-                    }
+        for (int jb = 0; jb < 2; ++jb) {
+            if (i2 + jb < nbc) {
+                const unsigned char *rblk = stage + OFF_RPART + jb * RBLOCK_BYTES;
+                const u16 *VOHc = reinterpret_cast<const u16 *>(rblk + ROFF_VOH);
+                const u16 *VHc = reinterpret_cast<const u16 *>(rblk + ROFF_VH);
+                const float *LX = reinterpret_cast<const float *>(rblk + ROFF_LV), *LO = LX + CH_N;
+                {
+                    const uint2 a0 = pack4v<OPE>(S[0]), a1 = pack4v<OPE>(S[1]), a2 = pack4v<OPE>(S[2]),
+                                a3 = pack4v<OPE>(S[3]);
+                    uint4(&d)[2] = jb ? d1 : d0;
+                    d[0] = cat(a0, a1);
+                    d[1] = cat(a2, a3);
                 }
-                PHASE_MARK(0);
-                ++s;
-            }
-        }
-        // ---- re-anchor the running sum of the gate gradient: sum over the other side of Gb * S_end
-        // (with a checkpoint per block: every fourth block, S_end = the start state of the block above)
-        if (NB == 1 && !last && (chunk & 3) == 3) take_state(top, S);
-        if (recompute || (chunk & 3) == 3) {
-            float us = 0.f;
-#pragma unroll
-            for (int j = 0; j < 4; ++j)
-#pragma unroll
-                for (int i = 0; i < 4; ++i) us += G[j][i] * S[j][i];
-            carry = row_sums(us).all;
-        }
-        // ---- B stages: blocks last to first
-#pragma unroll
-        for (int i = NB - 1; i >= 0; --i) {
-            if (i < nb) {
-                __syncthreads();
-                PHASE_MARK(2);
-                const unsigned char *stage = smem + (s & 1) * STAGE_BYTES;
-                const u16 *AOS = reinterpret_cast<const u16 *>(stage + OFF_TM + TM_AOS * TM_TILE);
-                const u16 *VOT = reinterpret_cast<const u16 *>(stage + OFF_TM + TM_VOT * TM_TILE);
-                const u16 *VOH = reinterpret_cast<const u16 *>(stage + OFF_TM + TM_VOH * TM_TILE);
-                const u16 *AOSc = reinterpret_cast<const u16 *>(stage + OFF_CM + CM_AOS * CM_TILE);
-                const u16 *ASc = reinterpret_cast<const u16 *>(stage + OFF_CM + CM_AS * CM_TILE);
-                const u16 *VTc = reinterpret_cast<const u16 *>(stage + OFF_CM + CM_VT * CM_TILE);
-                const float *LX = lv_vec(stage, 0, 0), *LO = lv_vec(stage, 0, 1);
-                const floatx4 zero = {0.f, 0.f, 0.f, 0.f};
-                // the state at the start of this block, as MFMA operands
-                uint4 sb0 = sv[i][0], sb1 = sv[i][1];
-                if constexpr (NB == 1) {
-                    if (!last) {
-                        to_operands(below, sb0, sb1);
-                        if ((chunk & 3) == 0) {
-#pragma unroll
-                            for (int j = 0; j < 4; ++j) top[j] = below[j];
-                        }
-                    }
-                    if (chunk > 0) fetch_ahead(ckpt + (chunk - 1) * (CH_N * CH_N));
-                }
-                // the 16x16 token-token product, in both orientations (full contraction over 64 channels)
-                const int ro = r * TS + 8 * g;
-                const uint4 vot_lo = ld4(VOT + ro), vot_hi = ld4(VOT + ro + 32);
-                const uint4 aos_lo = ld4(AOS + ro), aos_hi = ld4(AOS + ro + 32);
-                floatx4 pt1 = OPE::mfma32(vot_hi, aos_hi, OPE::mfma32(vot_lo, aos_lo, zero));   // P[t=r][s=4g+i]
-                floatx4 pt2 = OPE::mfma32(aos_hi, vot_hi, OPE::mfma32(aos_lo, vot_lo, zero));   // P[r'=4g+i][t=r]
-                float pd[4];     // diagonal for this lane's tokens 4g+i
-#pragma unroll
-                for (int ii = 0; ii < 4; ++ii) pd[ii] = __shfl(pt1[ii], 20 * g + ii, 64);
-#pragma unroll
-                for (int ii = 0; ii < 4; ++ii) {
-                    pt1[ii] = (4 * g + ii < r) ? pt1[ii] : 0.f;
-                    pt2[ii] = (4 * g + ii > r) ? pt2[ii] : 0.f;
-                }
-                const uint2 pa_o = pack4v<OPE>(pt1), pa_v = pack4v<OPE>(pt2);
-                const uint2 vtc = ld2(VTc + ch * CC + 4 * g), asc = ld2(ASc + ch * CC + 4 * g);
                 const float lo = LO[ch];
-                const int po = r * TS + 16 * g;
-                // o' uses the block-start state
-                floatx4 oa = OPE::mfma32(ld4(AOS + po + 8), sb1, OPE::mfma32(ld4(AOS + po), sb0, zero));
-                oa += OPE::mfma16(pa_o, vtc, zero);
-                // v' uses the adjoint entering the block, scaled to the block end on the own side
-                floatx4 ga[4];
-#pragma unroll
-                for (int j = 0; j < 4; ++j) ga[j] = G[j] * lo;
-                const uint4 gp0 = cat(pack4v<OPE>(ga[0]), pack4v<OPE>(ga[1]));
-                const uint4 gp1 = cat(pack4v<OPE>(ga[2]), pack4v<OPE>(ga[3]));
-                floatx4 va = OPE::mfma32(ld4(VOH + po + 8), gp1, OPE::mfma32(ld4(VOH + po), gp0, zero));
-                va += OPE::mfma16(pa_v, asc, zero);
-                // adjoint of the previous block
+                const uint2 vhc = ld2(VHc + ch * CC + 4 * g);
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
                     const float4 lx = *reinterpret_cast<const float4 *>(LX + 16 * j + 4 * g);
-                    ga[j][0] *= lx.x; ga[j][1] *= lx.y; ga[j][2] *= lx.z; ga[j][3] *= lx.w;
-                    G[j] = OPE::mfma16(ld2(AOSc + (16 * j + r) * CC + 4 * g), asc, ga[j]);
+                    S[j][0] *= lo * lx.x; S[j][1] *= lo * lx.y; S[j][2] *= lo * lx.z; S[j][3] *= lo * lx.w;
+                    S[j] = OPE::mfma16(ld2(VOHc + (16 * j + r) * CC + 4 * g), vhc, S[j]);
                 }
-                // ---- gradients for tokens 4g+i, channel ch
-                {
-                    float asv[4], vtv[4], du[4];
-                    unpack4<OPE>(asc, asv);
-                    unpack4<OPE>(vtc, vtv);
-#pragma unroll
-                    for (int ii = 0; ii < 4; ++ii) du[ii] = oa[ii] * asv[ii] - va[ii] * vtv[ii];
-                    reverse_running_sum_swap(du, carry, g);
-                    const float *cf = reinterpret_cast<const float *>(stage + OFF_CF) + ch * CC + 4 * g;
-                    const float4 rg = *reinterpret_cast<const float4 *>(cf + F_RG * (CF_TILE / 4));
-                    const float4 ip = *reinterpret_cast<const float4 *>(cf + F_IP * (CF_TILE / 4));
-                    const float rgv[4] = {rg.x, rg.y, rg.z, rg.w}, ipv[4] = {ip.x, ip.y, ip.z, ip.w};
-                    // 16 lanes write 32 contiguous bytes of a token row; the four waves complete the row.
-                    // Only the last block of the sequence can reach past its end.
-                    const int tg = (int)chunk * C + i * CH_L + 4 * g;         // this lane's first token
-                    const u32 go = (u32)tg * ts + (u32)ch;
-                    float ppv[4] = {0.f, 0.f, 0.f, 0.f};
-                    if (side == 1) {
-                        const float4 pp = *reinterpret_cast<const float4 *>(cf + F_PP * (CF_TILE / 4));
-                        ppv[0] = pp.x; ppv[1] = pp.y; ppv[2] = pp.z; ppv[3] = pp.w;
-                    }
-                    // The state of the block below has had this stage's arithmetic to arrive; it is taken
-                    // before the stores are issued, so that the wait for it never includes them.
-                    if constexpr (NB == 1) {
-                        if (chunk > 0) take_ahead(below);
-                    }
-                    // one address per array; the four tokens are immediate offsets from it (folded rows)
-                    u16 *const pv = d_val + go, *const pg = d_gate + go, *const pa = d_adj + go;
-                    auto store = [&](int ii) {
-                        pv[ii * ts] = cvt1<IOE>(ipv[ii] * (va[ii] + asv[ii] * pd[ii]));
-                        pg[ii * ts] = cvt1<IOE>(du[ii] * rgv[ii]);
-                        if (side == 1) pa[ii * ts] = cvt1<IOE>(ppv[ii] * (oa[ii] + vtv[ii] * pd[ii]));
-                    };
-                    if ((int)chunk * C + (i + 1) * CH_L <= T) {
-#pragma unroll
-                        for (int ii = 0; ii < 4; ++ii) store(ii);
-                    } else {
-#pragma unroll
-                        for (int ii = 0; ii < 4; ++ii)
-                            if (tg + ii < T) store(ii);
-                    }
-                }
-                PHASE_MARK(1);
-                ++s;
             }
+        }
+    };
+    // B part of a stage: blocks i2 + 1 and i2 (in that order) of chunk `chunk`, which has nb blocks
+    auto b_pair = [&](const unsigned char *stage, int64_t chunk, int nb, auto i2_c) {
+        constexpr int i2 = decltype(i2_c)::value;
+#pragma unroll
+        for (int jb = 1; jb >= 0; --jb) {
+            const int i = i2 + jb;
+            // the blocks are kept apart in the instruction schedule: interleaved, their temporaries
+            // do not fit the register file next to the states
+            __builtin_amdgcn_sched_barrier(0);
+            if (i < nb) {
+            const unsigned char *blk = stage + jb * BLOCK_BYTES;
+            const u16 *AOS = reinterpret_cast<const u16 *>(blk + OFF_TM + TM_AOS * TM_TILE);
+            const u16 *VOT = reinterpret_cast<const u16 *>(blk + OFF_TM + TM_VOT * TM_TILE);
+            const u16 *VOH = reinterpret_cast<const u16 *>(blk + OFF_TM + TM_VOH * TM_TILE);
+            const u16 *AOSc = reinterpret_cast<const u16 *>(blk + OFF_CM + CM_AOS * CM_TILE);
+            const u16 *ASc = reinterpret_cast<const u16 *>(blk + OFF_CM + CM_AS * CM_TILE);
+            const u16 *VTc = reinterpret_cast<const u16 *>(blk + OFF_CM + CM_VT * CM_TILE);
+            const float *LX = lv_vec(blk, 0), *LO = lv_vec(blk, 1);
+            const floatx4 zero = {0.f, 0.f, 0.f, 0.f};
+            const uint4 sb0 = sv[i][0], sb1 = sv[i][1];      // the state at the start of this block
+            // the 16x16 token-token product, in both orientations (full contraction over 64 channels)
+            const int ro = r * TS + 8 * g;
+            const uint4 vot_lo = ld4(VOT + ro), vot_hi = ld4(VOT + ro + 32);
+            const uint4 aos_lo = ld4(AOS + ro), aos_hi = ld4(AOS + ro + 32);
+            floatx4 pt1 = OPE::mfma32(vot_hi, aos_hi, OPE::mfma32(vot_lo, aos_lo, zero));   // P[t=r][s=4g+i]
+            floatx4 pt2 = OPE::mfma32(aos_hi, vot_hi, OPE::mfma32(aos_lo, vot_lo, zero));   // P[r'=4g+i][t=r]
+            float pd[4];     // diagonal for this lane's tokens 4g+i
+        #pragma unroll
+            for (int ii = 0; ii < 4; ++ii) pd[ii] = __shfl(pt1[ii], 20 * g + ii, 64);
+        #pragma unroll
+            for (int ii = 0; ii < 4; ++ii) {
+                pt1[ii] = (4 * g + ii < r) ? pt1[ii] : 0.f;
+                pt2[ii] = (4 * g + ii > r) ? pt2[ii] : 0.f;
+            }
+            const uint2 pa_o = pack4v<OPE>(pt1), pa_v = pack4v<OPE>(pt2);
+            const uint2 vtc = ld2(VTc + ch * CC + 4 * g), asc = ld2(ASc + ch * CC + 4 * g);
+            const float lo = LO[ch];
+            const int po = r * TS + 16 * g;
+            // o' uses the block-start state
+            floatx4 oa = OPE::mfma32(ld4(AOS + po + 8), sb1, OPE::mfma32(ld4(AOS + po), sb0, zero));
+            oa += OPE::mfma16(pa_o, vtc, zero);
+            // v' uses the adjoint entering the block, scaled to the block end on the own side
+            floatx4 ga[4];
+        #pragma unroll
+            for (int j = 0; j < 4; ++j) ga[j] = G[j] * lo;
+            const uint4 gp0 = cat(pack4v<OPE>(ga[0]), pack4v<OPE>(ga[1]));
+            const uint4 gp1 = cat(pack4v<OPE>(ga[2]), pack4v<OPE>(ga[3]));
+            floatx4 va = OPE::mfma32(ld4(VOH + po + 8), gp1, OPE::mfma32(ld4(VOH + po), gp0, zero));
+            va += OPE::mfma16(pa_v, asc, zero);
+            // adjoint of the previous block
+        #pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const float4 lx = *reinterpret_cast<const float4 *>(LX + 16 * j + 4 * g);
+                ga[j][0] *= lx.x; ga[j][1] *= lx.y; ga[j][2] *= lx.z; ga[j][3] *= lx.w;
+                G[j] = OPE::mfma16(ld2(AOSc + (16 * j + r) * CC + 4 * g), asc, ga[j]);
+            }
+            // ---- gradients for tokens 4g+i, channel ch
+            {
+                float asv[4], vtv[4], du[4];
+                unpack4<OPE>(asc, asv);
+                unpack4<OPE>(vtc, vtv);
+        #pragma unroll
+                for (int ii = 0; ii < 4; ++ii) du[ii] = oa[ii] * asv[ii] - va[ii] * vtv[ii];
+                reverse_running_sum_swap(du, carry, g);
+                const float *cf = reinterpret_cast<const float *>(blk + OFF_CF) + ch * CC + 4 * g;
+                const float4 rg = *reinterpret_cast<const float4 *>(cf + F_RG * (CF_TILE / 4));
+                const float4 ip = *reinterpret_cast<const float4 *>(cf + F_IP * (CF_TILE / 4));
+                const float rgv[4] = {rg.x, rg.y, rg.z, rg.w}, ipv[4] = {ip.x, ip.y, ip.z, ip.w};
+                // 16 lanes write 32 contiguous bytes of a token row; the four waves complete the row.
+                // Only the last block of the sequence can reach past its end.
+                const int tg = (int)chunk * C + i * CH_L + 4 * g;         // this lane's first token
+                const u32 go = (u32)tg * ts + (u32)ch;
+                float ppv[4] = {0.f, 0.f, 0.f, 0.f};        // own prefix = 1 / (1 / prefix)
+            if (side == 1) {
+#pragma unroll
+                for (int ii = 0; ii < 4; ++ii) ppv[ii] = __builtin_amdgcn_rcpf(ipv[ii]);
+            }
+            // one address per array; the four tokens are immediate offsets from it (folded rows)
+                u16 *const pv = d_val + go, *const pg = d_gate + go, *const pa = d_adj + go;
+                auto store = [&](int ii) {
+                    pv[ii * ts] = cvt1<IOE>(ipv[ii] * (va[ii] + asv[ii] * pd[ii]));
+                    pg[ii * ts] = cvt1<IOE>(du[ii] * rgv[ii]);
+                    if (side == 1) pa[ii * ts] = cvt1<IOE>(ppv[ii] * (oa[ii] + vtv[ii] * pd[ii]));
+                };
+                if ((int)chunk * C + (i + 1) * CH_L <= T) {
+        #pragma unroll
+                    for (int ii = 0; ii < 4; ++ii) store(ii);
+                } else {
+        #pragma unroll
+                    for (int ii = 0; ii < 4; ++ii)
+                        if (tg + ii < T) store(ii);
+                }
+            }
+            }
+        }
+    };
+    // re-anchor the running sum of the gate gradient: sum over the other side of Gb * S_end
+    auto anchor = [&]() {
+        float us = 0.f;
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) us += G[j][i] * S[j][i];
+        carry = row_sums(us).all;
+    };
+    constexpr int MP = NB / 2;
+
+    // every stage starts with the workgroup barrier that publishes its operand tiles
+    // ---- prologue: R pairs of the last chunk
+    take_state(pf, S);
+    if (NC > 1) load_state(ckpt + (NC - 2) * (CH_N * CH_N), pf);
+#pragma unroll
+    for (int k = 0; k < MP; ++k) {
+        if (2 * k < nb_last) {
+            __syncthreads();
+            PHASE_MARK(3);
+            r_pair(smem + (s & 1) * STAGE_BYTES, nb_last, 2 * k, sv[2 * k], sv[2 * k + 1]);
+            PHASE_MARK(0);
+            ++s;
+        }
+    }
+    anchor();
+    // ---- transitions: B pairs of chunk c, last to first, each with an R pair of chunk c - 1
+    // (the running state S of the R work is kept out of the registers while a B part runs: as the raw
+    // checkpoint before the chunk's first R pair, parked in LDS between its R pairs)
+    float4 *const park = reinterpret_cast<float4 *>(smem + OFF_PARK) + tid * 4;
+    for (int64_t chunk = NC - 1; chunk >= 1; --chunk) {
+        const int nb = chunk == NC - 1 ? nb_last : NB;
+        {
+            __syncthreads();
+            PHASE_MARK(2);
+            const unsigned char *stage = smem + (s & 1) * STAGE_BYTES;
+            b_pair(stage, chunk, nb, std::integral_constant<int, NB - 2>{});
+            take_state(pf, S);
+            if (chunk > 1) load_state(ckpt + (chunk - 2) * (CH_N * CH_N), pf);
+            // the registers of the pair just done take the first pair of the chunk below
+            r_pair(stage, NB, 0, sv[NB - 2], sv[NB - 1]);
+            if constexpr (MP == 2) {
+#pragma unroll
+                for (int j = 0; j < 4; ++j) park[j] = make_float4(S[j][0], S[j][1], S[j][2], S[j][3]);
+            }
+            PHASE_MARK(1);
+            ++s;
+        }
+        if constexpr (MP == 2) {
+            __syncthreads();
+            PHASE_MARK(2);
+            const unsigned char *stage = smem + (s & 1) * STAGE_BYTES;
+            b_pair(stage, chunk, nb, std::integral_constant<int, 0>{});
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const float4 v = park[j];
+                S[j][0] = v.x; S[j][1] = v.y; S[j][2] = v.z; S[j][3] = v.w;
+            }
+            r_pair(stage, NB, 2, sv[0], sv[1]);
+            PHASE_MARK(1);
+            ++s;
+            // ... which leaves the two pairs in each other's place
+#pragma unroll
+            for (int i = 0; i < 2; ++i)
+#pragma unroll
+                for (int e = 0; e < 2; ++e) {
+                    const uint4 t = sv[i][e];
+                    sv[i][e] = sv[(i + 2) % NB][e];
+                    sv[(i + 2) % NB][e] = t;
+                }
+        }
+        anchor();
+    }
+    // ---- epilogue: B pairs of chunk 0
+    {
+        const int nb = NC == 1 ? nb_last : NB;
+        if (NB - 2 < nb && MP == 2) {
+            __syncthreads();
+            PHASE_MARK(2);
+            b_pair(smem + (s & 1) * STAGE_BYTES, 0, nb, std::integral_constant<int, NB - 2>{});
+            PHASE_MARK(1);
+            ++s;
+        }
+        {
+            __syncthreads();
+            PHASE_MARK(2);
+            b_pair(smem + (s & 1) * STAGE_BYTES, 0, nb, std::integral_constant<int, 0>{});
+            PHASE_MARK(1);
+            ++s;
         }
     }
     // d_s0 = adjoint after the first block (value side only: rows of [d][k] are contiguous there)
@@ -821,7 +768,7 @@ __device__ __forceinline__ void split_matrix_waves(const ChunkBwdArgs &p, unsign
 }
 
 template <typename IOE, typename OPE, int NB, bool HEADS>
-__global__ __launch_bounds__(SP_THREADS) void lfw_bwd_chunk_kernel(ChunkBwdArgs p, int rows_padded) {
+__global__ __launch_bounds__(BW_THREADS) void lfw_bwd_chunk_kernel(ChunkBwdArgs p, int rows_padded) {
     extern __shared__ __align__(16) unsigned char smem[];
     const int tid = threadIdx.x;
     // blockIdx = side * rows_padded + row with rows_padded a multiple of 8: the two workgroups of a
@@ -829,37 +776,36 @@ __global__ __launch_bounds__(SP_THREADS) void lfw_bwd_chunk_kernel(ChunkBwdArgs 
     const int side = (int)blockIdx.x >= rows_padded ? 1 : 0;
     const int64_t b = (int)blockIdx.x - side * rows_padded;
     if (b >= p.B) return;
-    // both branches execute exactly 2 + (number of stages) workgroup barriers
+    // both branches execute one workgroup barrier per stage
     if (tid < 256) {
         if (side == 0)
-            split_matrix_waves<IOE, OPE, NB, HEADS, 0>(p, smem, tid, b);
+            bwd_matrix_waves<IOE, OPE, NB, HEADS, 0>(p, smem, tid, b);
         else
-            split_matrix_waves<IOE, OPE, NB, HEADS, 1>(p, smem, tid, b);
+            bwd_matrix_waves<IOE, OPE, NB, HEADS, 1>(p, smem, tid, b);
+    } else {
+        bwd_prep_waves<IOE, OPE, NB, HEADS>(p, smem, tid - 256, b, side);
     }
-    else
-        split_prep_waves<IOE, OPE, NB, HEADS>(p, smem, tid - 256, b, side);
 }
 
 template <typename IOE, typename OPE, int NB, bool HEADS> int launch(const ChunkBwdArgs &a, hipStream_t stream) {
     auto kern = lfw_bwd_chunk_kernel<IOE, OPE, NB, HEADS>;
     // more than 64 KB of dynamic LDS has to be enabled per function (and per device)
     int rc = check_hip(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, SP_SMEM),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, BW_SMEM),
                        "hipFuncSetAttribute(backward chunk kernel)");
     if (rc) return rc;
     if (a.B > 0x1fffffffLL) return fail(T2FW_ERR_UNSUPPORTED, "B=%lld is too large", (long long)a.B);
     if (a.heads < 1 || a.T * a.heads >= CHUNK_MAX_T)
         return fail(T2FW_ERR_UNSUPPORTED, "T=%lld with %d heads is too long for 32-bit row offsets", (long long)a.T, a.heads);
     const int rows_padded = (int)((a.B + 7) / 8 * 8);
-    hipLaunchKernelGGL(kern, dim3(2u * (unsigned)rows_padded), dim3(SP_THREADS), SP_SMEM, stream, a, rows_padded);
+    hipLaunchKernelGGL(kern, dim3(2u * (unsigned)rows_padded), dim3(BW_THREADS), BW_SMEM, stream, a, rows_padded);
     return check_hip(hipGetLastError(), "lfw_bwd_chunk_kernel launch");
 }
 
 template <typename IOE, typename OPE> int by_nb(const ChunkBwdArgs &a, hipStream_t stream) {
-    if (a.C == 16) return a.heads == 1 ? launch<IOE, OPE, 1, false>(a, stream) : launch<IOE, OPE, 1, true>(a, stream);
     if (a.C == 64) return a.heads == 1 ? launch<IOE, OPE, 4, false>(a, stream) : launch<IOE, OPE, 4, true>(a, stream);
     if (a.C == 32) return a.heads == 1 ? launch<IOE, OPE, 2, false>(a, stream) : launch<IOE, OPE, 2, true>(a, stream);
-    return fail(T2FW_ERR_UNSUPPORTED, "the chunked backward kernel takes checkpoint intervals 16, 32 or 64");
+    return fail(T2FW_ERR_UNSUPPORTED, "the chunked backward kernel takes checkpoint intervals 32 or 64");
 }
 
 }  // namespace

@@ -389,9 +389,8 @@ __device__ __forceinline__ void fwd_matrix_waves(const ChunkFwdArgs &p, unsigned
     // One step (two blocks).  FULL: all 32 tokens exist, which leaves the body without a branch
     // around its stores, so that the LDS reads of the whole step can be scheduled ahead of the
     // matrix products that use them.
-    // BLK: a checkpoint per block (inside the step) instead of one every C tokens (at its start).
-    auto step = [&](int n, auto full_c, auto blk_c) {
-        constexpr bool FULL = decltype(full_c)::value, BLK = decltype(blk_c)::value;
+    auto step = [&](int n, auto full_c) {
+        constexpr bool FULL = decltype(full_c)::value;
         __syncthreads();        // the operand tiles of step n are in LDS
         PHASE_MARK(3);
         const unsigned char *ops = smem + (n & 1) * OPS_BYTES;
@@ -403,7 +402,7 @@ __device__ __forceinline__ void fwd_matrix_waves(const ChunkFwdArgs &p, unsigned
         const float *AS = reinterpret_cast<const float *>(ops + OFF_AS);
         const float *BL = reinterpret_cast<const float *>(ops + OFF_BL);
         const float *AL = reinterpret_cast<const float *>(ops + OFF_AL);
-        if (!BLK && ckpt != nullptr) {          // checkpoint interval is a multiple of the step
+        if (ckpt != nullptr) {          // checkpoint interval is a multiple of the step
             if (until_ckpt == 0) {
                 store_state<IOE>(S, ckpt + (b * p.NC + chunk) * (CH_N * CH_N), d, g);
                 until_ckpt = p.C;
@@ -414,9 +413,6 @@ __device__ __forceinline__ void fwd_matrix_waves(const ChunkFwdArgs &p, unsigned
 #pragma unroll
         for (int hh = 0; hh < 2; ++hh) {
             const int tok0 = CH_L * hh;
-            // a checkpoint per block: the state at the start of every block that has a token
-            if (BLK && (FULL || n * CH_STEP + tok0 < T))
-                store_state<IOE>(S, ckpt + (b * p.NC + 2 * n + hh) * (CH_N * CH_N), d, g);
             // P^T[s,t] = kt_s . qs_t, kept for s <= t, as the A operand of the intra product
             const u16 *krow = KT + (tok0 + r) * TS + 8 * g;
             const u16 *qrow = QT + (tok0 + r) * TS + 8 * g;
@@ -463,13 +459,8 @@ __device__ __forceinline__ void fwd_matrix_waves(const ChunkFwdArgs &p, unsigned
         }
     };
     const int nfull = T / CH_STEP;
-    if (ckpt != nullptr && p.C == CH_L) {
-        for (int n = 0; n < nfull; ++n) step(n, std::true_type{}, std::true_type{});
-        if (nfull * CH_STEP < T) step(nfull, std::false_type{}, std::true_type{});
-    } else {
-        for (int n = 0; n < nfull; ++n) step(n, std::true_type{}, std::false_type{});
-        if (nfull * CH_STEP < T) step(nfull, std::false_type{}, std::false_type{});
-    }
+    for (int n = 0; n < nfull; ++n) step(n, std::true_type{});
+    if (nfull * CH_STEP < T) step(nfull, std::false_type{});
     store_state<IOE>(S, reinterpret_cast<u16 *>(p.next_state) + b * (CH_N * CH_N), d, g);
     PHASE_END(tid >> 6);
 }
