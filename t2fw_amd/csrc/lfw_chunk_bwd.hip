@@ -581,89 +581,89 @@ __device__ __forceinline__ void bwd_matrix_waves(const ChunkBwdArgs &p, unsigned
             // do not fit the register file next to the states
             __builtin_amdgcn_sched_barrier(0);
             if (i < nb) {
-            const unsigned char *blk = stage + jb * BLOCK_BYTES;
-            const u16 *AOS = reinterpret_cast<const u16 *>(blk + OFF_TM + TM_AOS * TM_TILE);
-            const u16 *VOT = reinterpret_cast<const u16 *>(blk + OFF_TM + TM_VOT * TM_TILE);
-            const u16 *VOH = reinterpret_cast<const u16 *>(blk + OFF_TM + TM_VOH * TM_TILE);
-            const u16 *AOSc = reinterpret_cast<const u16 *>(blk + OFF_CM + CM_AOS * CM_TILE);
-            const u16 *ASc = reinterpret_cast<const u16 *>(blk + OFF_CM + CM_AS * CM_TILE);
-            const u16 *VTc = reinterpret_cast<const u16 *>(blk + OFF_CM + CM_VT * CM_TILE);
-            const float *LX = lv_vec(blk, 0), *LO = lv_vec(blk, 1);
-            const floatx4 zero = {0.f, 0.f, 0.f, 0.f};
-            const uint4 sb0 = sv[i][0], sb1 = sv[i][1];      // the state at the start of this block
-            // the 16x16 token-token product, in both orientations (full contraction over 64 channels)
-            const int ro = r * TS + 8 * g;
-            const uint4 vot_lo = ld4(VOT + ro), vot_hi = ld4(VOT + ro + 32);
-            const uint4 aos_lo = ld4(AOS + ro), aos_hi = ld4(AOS + ro + 32);
-            floatx4 pt1 = OPE::mfma32(vot_hi, aos_hi, OPE::mfma32(vot_lo, aos_lo, zero));   // P[t=r][s=4g+i]
-            floatx4 pt2 = OPE::mfma32(aos_hi, vot_hi, OPE::mfma32(aos_lo, vot_lo, zero));   // P[r'=4g+i][t=r]
-            float pd[4];     // diagonal for this lane's tokens 4g+i
-        #pragma unroll
-            for (int ii = 0; ii < 4; ++ii) pd[ii] = __shfl(pt1[ii], 20 * g + ii, 64);
-        #pragma unroll
-            for (int ii = 0; ii < 4; ++ii) {
-                pt1[ii] = (4 * g + ii < r) ? pt1[ii] : 0.f;
-                pt2[ii] = (4 * g + ii > r) ? pt2[ii] : 0.f;
-            }
-            const uint2 pa_o = pack4v<OPE>(pt1), pa_v = pack4v<OPE>(pt2);
-            const uint2 vtc = ld2(VTc + ch * CC + 4 * g), asc = ld2(ASc + ch * CC + 4 * g);
-            const float lo = LO[ch];
-            const int po = r * TS + 16 * g;
-            // o' uses the block-start state
-            floatx4 oa = OPE::mfma32(ld4(AOS + po + 8), sb1, OPE::mfma32(ld4(AOS + po), sb0, zero));
-            oa += OPE::mfma16(pa_o, vtc, zero);
-            // v' uses the adjoint entering the block, scaled to the block end on the own side
-            floatx4 ga[4];
-        #pragma unroll
-            for (int j = 0; j < 4; ++j) ga[j] = G[j] * lo;
-            const uint4 gp0 = cat(pack4v<OPE>(ga[0]), pack4v<OPE>(ga[1]));
-            const uint4 gp1 = cat(pack4v<OPE>(ga[2]), pack4v<OPE>(ga[3]));
-            floatx4 va = OPE::mfma32(ld4(VOH + po + 8), gp1, OPE::mfma32(ld4(VOH + po), gp0, zero));
-            va += OPE::mfma16(pa_v, asc, zero);
-            // adjoint of the previous block
-        #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const float4 lx = *reinterpret_cast<const float4 *>(LX + 16 * j + 4 * g);
-                ga[j][0] *= lx.x; ga[j][1] *= lx.y; ga[j][2] *= lx.z; ga[j][3] *= lx.w;
-                G[j] = OPE::mfma16(ld2(AOSc + (16 * j + r) * CC + 4 * g), asc, ga[j]);
-            }
-            // ---- gradients for tokens 4g+i, channel ch
-            {
-                float asv[4], vtv[4], du[4];
-                unpack4<OPE>(asc, asv);
-                unpack4<OPE>(vtc, vtv);
-        #pragma unroll
-                for (int ii = 0; ii < 4; ++ii) du[ii] = oa[ii] * asv[ii] - va[ii] * vtv[ii];
-                reverse_running_sum_swap(du, carry, g);
-                const float *cf = reinterpret_cast<const float *>(blk + OFF_CF) + ch * CC + 4 * g;
-                const float4 rg = *reinterpret_cast<const float4 *>(cf + F_RG * (CF_TILE / 4));
-                const float4 ip = *reinterpret_cast<const float4 *>(cf + F_IP * (CF_TILE / 4));
-                const float rgv[4] = {rg.x, rg.y, rg.z, rg.w}, ipv[4] = {ip.x, ip.y, ip.z, ip.w};
-                // 16 lanes write 32 contiguous bytes of a token row; the four waves complete the row.
-                // Only the last block of the sequence can reach past its end.
-                const int tg = (int)chunk * C + i * CH_L + 4 * g;         // this lane's first token
-                const u32 go = (u32)tg * ts + (u32)ch;
-                float ppv[4] = {0.f, 0.f, 0.f, 0.f};        // own prefix = 1 / (1 / prefix)
-            if (side == 1) {
+                const unsigned char *blk = stage + jb * BLOCK_BYTES;
+                const u16 *AOS = reinterpret_cast<const u16 *>(blk + OFF_TM + TM_AOS * TM_TILE);
+                const u16 *VOT = reinterpret_cast<const u16 *>(blk + OFF_TM + TM_VOT * TM_TILE);
+                const u16 *VOH = reinterpret_cast<const u16 *>(blk + OFF_TM + TM_VOH * TM_TILE);
+                const u16 *AOSc = reinterpret_cast<const u16 *>(blk + OFF_CM + CM_AOS * CM_TILE);
+                const u16 *ASc = reinterpret_cast<const u16 *>(blk + OFF_CM + CM_AS * CM_TILE);
+                const u16 *VTc = reinterpret_cast<const u16 *>(blk + OFF_CM + CM_VT * CM_TILE);
+                const float *LX = lv_vec(blk, 0), *LO = lv_vec(blk, 1);
+                const floatx4 zero = {0.f, 0.f, 0.f, 0.f};
+                const uint4 sb0 = sv[i][0], sb1 = sv[i][1];      // the state at the start of this block
+                // the 16x16 token-token product, in both orientations (full contraction over 64 channels)
+                const int ro = r * TS + 8 * g;
+                const uint4 vot_lo = ld4(VOT + ro), vot_hi = ld4(VOT + ro + 32);
+                const uint4 aos_lo = ld4(AOS + ro), aos_hi = ld4(AOS + ro + 32);
+                floatx4 pt1 = OPE::mfma32(vot_hi, aos_hi, OPE::mfma32(vot_lo, aos_lo, zero));   // P[t=r][s=4g+i]
+                floatx4 pt2 = OPE::mfma32(aos_hi, vot_hi, OPE::mfma32(aos_lo, vot_lo, zero));   // P[r'=4g+i][t=r]
+                float pd[4];     // diagonal for this lane's tokens 4g+i
 #pragma unroll
-                for (int ii = 0; ii < 4; ++ii) ppv[ii] = __builtin_amdgcn_rcpf(ipv[ii]);
-            }
-            // one address per array; the four tokens are immediate offsets from it (folded rows)
-                u16 *const pv = d_val + go, *const pg = d_gate + go, *const pa = d_adj + go;
-                auto store = [&](int ii) {
-                    pv[ii * ts] = cvt1<IOE>(ipv[ii] * (va[ii] + asv[ii] * pd[ii]));
-                    pg[ii * ts] = cvt1<IOE>(du[ii] * rgv[ii]);
-                    if (side == 1) pa[ii * ts] = cvt1<IOE>(ppv[ii] * (oa[ii] + vtv[ii] * pd[ii]));
-                };
-                if ((int)chunk * C + (i + 1) * CH_L <= T) {
-        #pragma unroll
-                    for (int ii = 0; ii < 4; ++ii) store(ii);
-                } else {
-        #pragma unroll
-                    for (int ii = 0; ii < 4; ++ii)
-                        if (tg + ii < T) store(ii);
+                for (int ii = 0; ii < 4; ++ii) pd[ii] = __shfl(pt1[ii], 20 * g + ii, 64);
+#pragma unroll
+                for (int ii = 0; ii < 4; ++ii) {
+                    pt1[ii] = (4 * g + ii < r) ? pt1[ii] : 0.f;
+                    pt2[ii] = (4 * g + ii > r) ? pt2[ii] : 0.f;
                 }
-            }
+                const uint2 pa_o = pack4v<OPE>(pt1), pa_v = pack4v<OPE>(pt2);
+                const uint2 vtc = ld2(VTc + ch * CC + 4 * g), asc = ld2(ASc + ch * CC + 4 * g);
+                const float lo = LO[ch];
+                const int po = r * TS + 16 * g;
+                // o' uses the block-start state
+                floatx4 oa = OPE::mfma32(ld4(AOS + po + 8), sb1, OPE::mfma32(ld4(AOS + po), sb0, zero));
+                oa += OPE::mfma16(pa_o, vtc, zero);
+                // v' uses the adjoint entering the block, scaled to the block end on the own side
+                floatx4 ga[4];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) ga[j] = G[j] * lo;
+                const uint4 gp0 = cat(pack4v<OPE>(ga[0]), pack4v<OPE>(ga[1]));
+                const uint4 gp1 = cat(pack4v<OPE>(ga[2]), pack4v<OPE>(ga[3]));
+                floatx4 va = OPE::mfma32(ld4(VOH + po + 8), gp1, OPE::mfma32(ld4(VOH + po), gp0, zero));
+                va += OPE::mfma16(pa_v, asc, zero);
+                // adjoint of the previous block
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const float4 lx = *reinterpret_cast<const float4 *>(LX + 16 * j + 4 * g);
+                    ga[j][0] *= lx.x; ga[j][1] *= lx.y; ga[j][2] *= lx.z; ga[j][3] *= lx.w;
+                    G[j] = OPE::mfma16(ld2(AOSc + (16 * j + r) * CC + 4 * g), asc, ga[j]);
+                }
+                // ---- gradients for tokens 4g+i, channel ch
+                {
+                    float asv[4], vtv[4], du[4];
+                    unpack4<OPE>(asc, asv);
+                    unpack4<OPE>(vtc, vtv);
+#pragma unroll
+                    for (int ii = 0; ii < 4; ++ii) du[ii] = oa[ii] * asv[ii] - va[ii] * vtv[ii];
+                    reverse_running_sum_swap(du, carry, g);
+                    const float *cf = reinterpret_cast<const float *>(blk + OFF_CF) + ch * CC + 4 * g;
+                    const float4 rg = *reinterpret_cast<const float4 *>(cf + F_RG * (CF_TILE / 4));
+                    const float4 ip = *reinterpret_cast<const float4 *>(cf + F_IP * (CF_TILE / 4));
+                    const float rgv[4] = {rg.x, rg.y, rg.z, rg.w}, ipv[4] = {ip.x, ip.y, ip.z, ip.w};
+                    // 16 lanes write 32 contiguous bytes of a token row; the four waves complete the row.
+                    // Only the last block of the sequence can reach past its end.
+                    const int tg = (int)chunk * C + i * CH_L + 4 * g;         // this lane's first token
+                    const u32 go = (u32)tg * ts + (u32)ch;
+                    float ppv[4] = {0.f, 0.f, 0.f, 0.f};        // own prefix = 1 / (1 / prefix)
+                    if (side == 1) {
+#pragma unroll
+                        for (int ii = 0; ii < 4; ++ii) ppv[ii] = __builtin_amdgcn_rcpf(ipv[ii]);
+                    }
+                    // one address per array; the four tokens are immediate offsets from it (folded rows)
+                    u16 *const pv = d_val + go, *const pg = d_gate + go, *const pa = d_adj + go;
+                    auto store = [&](int ii) {
+                        pv[ii * ts] = cvt1<IOE>(ipv[ii] * (va[ii] + asv[ii] * pd[ii]));
+                        pg[ii * ts] = cvt1<IOE>(du[ii] * rgv[ii]);
+                        if (side == 1) pa[ii * ts] = cvt1<IOE>(ppv[ii] * (oa[ii] + vtv[ii] * pd[ii]));
+                    };
+                    if ((int)chunk * C + (i + 1) * CH_L <= T) {
+#pragma unroll
+                        for (int ii = 0; ii < 4; ++ii) store(ii);
+                    } else {
+#pragma unroll
+                        for (int ii = 0; ii < 4; ++ii)
+                            if (tg + ii < T) store(ii);
+                    }
+                }
             }
         }
     };
