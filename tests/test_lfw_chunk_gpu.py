@@ -80,10 +80,15 @@ def test_config_like_inputs(dtype, gate_mean, state_std, B, T, C):
 @pytest.mark.parametrize("dtype,B,T,C", [(torch.bfloat16, 3, 112, 64), (torch.float16, 2, 48, 32),
                                          (torch.float16, 3, 16, 64), (torch.bfloat16, 2, 80, 64),
                                          (torch.float16, 2, 77, 32), (torch.float16, 3, 15, 64),
-                                         (torch.bfloat16, 2, 65, 64), (torch.float16, 2, 113, 64)])
+                                         (torch.bfloat16, 2, 65, 64), (torch.float16, 2, 113, 64),
+                                         (torch.float16, 2, 64, 64), (torch.bfloat16, 2, 32, 32),
+                                         (torch.float16, 1, 128, 64), (torch.float16, 2, 64, 32),
+                                         (torch.float16, 2, 192, 64), (torch.bfloat16, 1, 160, 64),
+                                         (torch.float16, 2, 161, 64), (torch.float16, 1, 31, 32)])
 def test_short_and_ragged_last_chunks(dtype, B, T, C):
-    """Last chunks of 1..4 blocks, with and without a partial last block (the backward handles the
-    last chunk of a sequence with a general schedule and the full chunks with a fixed one)."""
+    """Last chunks of 1..4 blocks, with and without a partial last block, one chunk only, and
+    sequences of whole chunks (the backward reads the last chunk of a sequence through a general
+    loader unless it is full, and pairs the work of neighbouring chunks in its stages)."""
     x, f, q, k, fk, s, go, gs = make_config_inputs(B, T, 64, 64, dtype, seed=100 + T, gate_mean=2.5, state_std=0.3)
     check_against_oracle((x, f, q, k, fk, s), go, gs, C, dtype, expect_flagged=0)
 
