@@ -47,7 +47,9 @@ constexpr int OFF_AS = OFF_XH + CH_N * CS * 2;             // a_t channel-major 
 constexpr int OFF_BL = OFF_AS + CH_N * CS * 4;             // b_L [2][64] f32
 constexpr int OFF_AL = OFF_BL + 2 * CH_N * 4;              // a_L [2][64] f32
 constexpr int OPS_BYTES = OFF_AL + 2 * CH_N * 4;
-constexpr int FWD_SMEM = 2 * OPS_BYTES;
+// Two stages of two steps each: a workgroup barrier every 64 tokens, the prep waves one stage ahead.
+constexpr int FWD_SMEM = 4 * OPS_BYTES;
+static_assert(FWD_SMEM <= 160 * 1024, "forward operand buffers exceed the LDS of one CU");
 static_assert(OPS_BYTES % 16 == 0, "operand buffers must keep 16-byte alignment");
 
 // ---- raw inputs --------------------------------------------------------------------------
@@ -243,7 +245,7 @@ __device__ __forceinline__ void fwd_prep_side(const ChunkFwdArgs &p, unsigned ch
 
     // this wave's share of the operand tiles of step n
     auto build = [&](const RawF<NV> &f, int n) {
-        unsigned char *ops = smem + (n & 1) * OPS_BYTES;
+        unsigned char *ops = smem + (n & 3) * OPS_BYTES;
         float pre[8], hat[8], til[8];
         const float tot = scale_half<OPE, NV>(f, h, pre, hat, til, bad);
         const int tok0 = CH_L * hh + 8 * h;
@@ -306,7 +308,14 @@ __device__ __forceinline__ void fwd_prep_side(const ChunkFwdArgs &p, unsigned ch
 
     // Full steps alternate between two register sets.  The loop always does a whole pair (set A,
     // then set B) with no exit in between, so that the order of the loads in flight is the same on
-    // every path into it; an odd count peels the first step off.
+    // every path into it; an odd count peels the first step off.  A stage is two steps: the barrier
+    // that publishes the tiles comes after every odd step and after the last one.
+    const int nsteps = nfull + (nfull * CH_STEP < T ? 1 : 0);
+    auto publish = [&](int n) {
+        PHASE_MARK(0);
+        if ((n & 1) || n == nsteps - 1) __syncthreads();
+        PHASE_MARK(3);
+    };
     PHASE_BEGIN();
     if (nfull > 0) {
         RawSet<NV> setA, setB;
@@ -315,9 +324,7 @@ __device__ __forceinline__ void fwd_prep_side(const ChunkFwdArgs &p, unsigned ch
             issue(setB, 0, lane_bytes);
             issue(setA, 1, lane_bytes);
             prepare(setB, 0);
-            PHASE_MARK(0);
-            __syncthreads();
-            PHASE_MARK(3);
+            publish(0);
             n = 1;
         } else {
             issue(setA, 0, lane_bytes);
@@ -325,13 +332,9 @@ __device__ __forceinline__ void fwd_prep_side(const ChunkFwdArgs &p, unsigned ch
         }
         for (; n < nfull; n += 2) {
             prepare(setA, n);
-            PHASE_MARK(0);
-            __syncthreads();
-            PHASE_MARK(3);
+            publish(n);
             prepare(setB, n + 1);
-            PHASE_MARK(0);
-            __syncthreads();
-            PHASE_MARK(3);
+            publish(n + 1);
         }
     }
     if (nfull * CH_STEP < T) {      // the partial step at the end
@@ -339,7 +342,7 @@ __device__ __forceinline__ void fwd_prep_side(const ChunkFwdArgs &p, unsigned ch
         const int t_own = nfull * CH_STEP + off_own, t_oth = nfull * CH_STEP + off_oth;
         raw_issue_tail<NV>(r, gate, val0, val1, t_own, t_oth, T, lane_bytes, ts);
         build(raw_take_tail<IOE, NV>(r, t_own, t_oth, T), nfull);
-        __syncthreads();
+        publish(nfull);
     }
     if (bad) p.row_flags[flag_slot] = 1;
     PHASE_END(4 + (tid >> 6));
@@ -389,11 +392,14 @@ __device__ __forceinline__ void fwd_matrix_waves(const ChunkFwdArgs &p, unsigned
     // One step (two blocks).  FULL: all 32 tokens exist, which leaves the body without a branch
     // around its stores, so that the LDS reads of the whole step can be scheduled ahead of the
     // matrix products that use them.
-    auto step = [&](int n, auto full_c) {
+    // BAR: the step is the first of its stage and starts with the workgroup barrier.
+    auto step = [&](int n, auto full_c, auto bar_c) {
         constexpr bool FULL = decltype(full_c)::value;
-        __syncthreads();        // the operand tiles of step n are in LDS
-        PHASE_MARK(3);
-        const unsigned char *ops = smem + (n & 1) * OPS_BYTES;
+        if constexpr (decltype(bar_c)::value) {
+            __syncthreads();        // the operand tiles of steps n and n + 1 are in LDS
+            PHASE_MARK(3);
+        }
+        const unsigned char *ops = smem + (n & 3) * OPS_BYTES;
         const u16 *QT = reinterpret_cast<const u16 *>(ops + OFF_QT);
         const u16 *KT = reinterpret_cast<const u16 *>(ops + OFF_KT);
         const u16 *KH = reinterpret_cast<const u16 *>(ops + OFF_KH);
@@ -459,8 +465,18 @@ __device__ __forceinline__ void fwd_matrix_waves(const ChunkFwdArgs &p, unsigned
         }
     };
     const int nfull = T / CH_STEP;
-    for (int n = 0; n < nfull; ++n) step(n, std::true_type{});
-    if (nfull * CH_STEP < T) step(nfull, std::false_type{});
+    int n = 0;
+    for (; n + 1 < nfull; n += 2) {
+        step(n, std::true_type{}, std::true_type{});
+        step(n + 1, std::true_type{}, std::false_type{});
+    }
+    if (n < nfull) step(n, std::true_type{}, std::true_type{});
+    if (nfull * CH_STEP < T) {
+        if (nfull & 1)
+            step(nfull, std::false_type{}, std::false_type{});
+        else
+            step(nfull, std::false_type{}, std::true_type{});
+    }
     store_state<IOE>(S, reinterpret_cast<u16 *>(p.next_state) + b * (CH_N * CH_N), d, g);
     PHASE_END(tid >> 6);
 }
@@ -470,7 +486,7 @@ __global__ __launch_bounds__(FWD_THREADS) void lfw_fwd_chunk_kernel(ChunkFwdArgs
     extern __shared__ __align__(16) unsigned char smem[];
     const int tid = threadIdx.x;
     const int64_t b = blockIdx.x;
-    // every wave executes exactly (number of steps) workgroup barriers
+    // every wave executes exactly ceil(number of steps / 2) workgroup barriers
     if (tid < 256) {
         fwd_matrix_waves<IOE, OPE, HEADS>(p, smem, tid, b, 0, b, true);
     } else {
