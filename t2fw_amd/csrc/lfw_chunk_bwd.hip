@@ -577,9 +577,6 @@ __device__ __forceinline__ void bwd_matrix_waves(const ChunkBwdArgs &p, unsigned
 #pragma unroll
         for (int jb = 1; jb >= 0; --jb) {
             const int i = i2 + jb;
-            // the blocks are kept apart in the instruction schedule: interleaved, their temporaries
-            // do not fit the register file next to the states
-            __builtin_amdgcn_sched_barrier(0);
             if (i < nb) {
                 const unsigned char *blk = stage + jb * BLOCK_BYTES;
                 const u16 *AOS = reinterpret_cast<const u16 *>(blk + OFF_TM + TM_AOS * TM_TILE);
