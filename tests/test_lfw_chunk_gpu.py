@@ -237,3 +237,16 @@ def test_long_context_bf16_slice():
     x, f, q, k, fk, s, go, gs = make_config_inputs(B, T, 64, 64, torch.bfloat16, seed=4, gate_mean=3.0,
                                                     state_std=0.1)
     check_against_oracle((x, f, q, k, fk, s), go, gs, 64, torch.bfloat16, expect_flagged=0)
+
+
+@pytest.mark.parametrize("seed", range(24))
+def test_random_lengths_and_intervals(seed):
+    """seeded random (T, C, B, dtype): every combination of chunk count, pairs in the last chunk and
+    tokens in the last block that the stage schedule of the backward distinguishes"""
+    g = torch.Generator().manual_seed(1000 + seed)
+    C = (32, 64)[int(torch.randint(0, 2, (1,), generator=g))]
+    T = int(torch.randint(1, 5 * C + 1, (1,), generator=g))
+    B = int(torch.randint(1, 4, (1,), generator=g))
+    dtype = (torch.float16, torch.bfloat16)[int(torch.randint(0, 2, (1,), generator=g))]
+    x, f, q, k, fk, s, go, gs = make_config_inputs(B, T, 64, 64, dtype, seed=seed, gate_mean=2.5, state_std=0.3)
+    check_against_oracle((x, f, q, k, fk, s), go, gs, C, dtype, expect_flagged=0)
