@@ -13,7 +13,8 @@ value      = B*T*steps / wall time of the timed region, in Mtokens/s (token = on
              outputs; `autograd_api` repeats it through LFWFunction.apply + backward.
 roofline   = algorithmic bytes of the dominant kernel / its mean duration measured with
              events on the launch stream (the call is repeated with the flag that skips the
-             exact-kernel fix-up launch, so that the events bracket that one kernel), against
+             exact redo of flagged rows, for the backward a launch of its own, so that the
+             events bracket that one kernel), against
              8 TB/s.  `traffic` comes from profiles/traffic_<workload>.json (rocprofv3 counters).
 copy256    = calibration workload for those counters: a 256 MiB device-to-device copy.
 cpu_baseline = the TorchScript restatement of the reference loop (oracle/), fp32,
@@ -170,8 +171,8 @@ def main():
         return (sum(e[0].elapsed_time(e[1]) for e in ev) / nrep, sum(e[1].elapsed_time(e[2]) for e in ev) / nrep)
 
     fwd_avg, bwd_avg = timed_calls(flags)
-    # the matrix-core kernel alone: the same calls without the exact-kernel fix-up launch that
-    # follows it (no row of this workload is flagged, so the results are the same)
+    # the matrix-core kernel alone: the same calls without the exact-kernel launch that follows
+    # the backward (no row of this workload is flagged, so the results are the same)
     fwd_kern, bwd_kern = (fwd_avg, bwd_avg) if args.force_scan else timed_calls(flags | _lib.FLAG_NO_FIXUP)
     fwd_bytes, bwd_bytes = algorithmic_bytes(B, T, D, K, es, C, backward)
     if backward and bwd_kern >= fwd_kern:

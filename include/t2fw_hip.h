@@ -75,12 +75,13 @@ extern "C" {
 #define T2FW_FLAG_FP16_OPERANDS 2 /* fp16 tensors: fp16 (not bf16) matrix-core operands;
                                      more mantissa, but rows whose 16-step gate products
                                      fall below 2^-8 take the exact scan path          */
-#define T2FW_FLAG_NO_FIXUP 4      /* matrix-core path: do not launch the exact kernels for the
-                                     rows it flagged; the caller reads the flags from the
-                                     workspace (int32 [2][B rounded up to 8], nonzero in either
-                                     slot = that row's results are not valid) and redoes those
-                                     rows with T2FW_FLAG_FORCE_SCAN, or knows its gates are in
-                                     range.  Saves one launch per call.                         */
+#define T2FW_FLAG_NO_FIXUP 4      /* matrix-core path: do not redo what it flagged with the exact
+                                     recurrence (the forward redoes it inside its kernel, the
+                                     backward with one more launch); the caller reads the flags
+                                     from the workspace (int32 [2][B rounded up to 8], nonzero in
+                                     either slot = that row's results are not valid) and redoes
+                                     those rows with T2FW_FLAG_FORCE_SCAN, or knows its gates are
+                                     in range.  Saves the backward's extra launch.              */
 
 int t2fw_abi_version(void);
 const char *t2fw_last_error(void);

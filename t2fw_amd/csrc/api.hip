@@ -144,8 +144,6 @@ static int lfw_forward_rows(const void *x, const void *f, const void *q, const v
     ScanFwdArgs a{};
     a.x = x; a.f = f; a.q = q; a.k = k; a.f_key = f_key; a.s0 = s0;
     a.out = out; a.next_state = next_state; a.ckpt = ckpt;
-    a.row_select = nullptr;
-    a.row_select2 = nullptr;
     a.B = B; a.T = T; a.D = D; a.K = K;
     a.heads = (int32_t)heads;
     a.C = ckpt ? C : 1;
@@ -162,15 +160,13 @@ static int lfw_forward_rows(const void *x, const void *f, const void *q, const v
         c.row_flags = static_cast<int32_t *>(workspace);
         c.B = B; c.T = T; c.NC = a.NC; c.C = a.C;
         c.heads = (int32_t)heads;
+        c.redo = (flags & T2FW_FLAG_NO_FIXUP) ? 0 : 1;       // flagged rows are redone inside the kernel
         const int op = (dtype == T2FW_F16 && (flags & T2FW_FLAG_FP16_OPERANDS)) ? 1 : 0;
         // two workgroups per batch row while that still fits the device in one wave of workgroups
         const int cus = compute_units();
         if (cus < 0) return fail(T2FW_ERR_HIP, "could not read the device's compute-unit count");
         const bool split = 2 * chunk_rows_padded(B) <= cus;
-        if ((rc = chunk_forward(c, dtype, op, split, st))) return rc;
-        a.row_select = c.row_flags;      // rows the chunked form could not take
-        a.row_select2 = split ? c.row_flags + chunk_rows_padded(B) : nullptr;
-        if (flags & T2FW_FLAG_NO_FIXUP) return T2FW_OK;
+        return chunk_forward(c, dtype, op, split, st);
     }
     return scan_forward(a, dtype, st);
 }

@@ -12,7 +12,11 @@
 // Only the intra-block terms use an inverse (1/b_L, 1/a_L over 16 steps); everything that
 // crosses block boundaries is scaled by factors <= 1, so the form holds for any gates in
 // (0, 1] whose 16-step products stay above 2^-100.  Rows that violate this (or have gates
-// outside (0, 1]) are flagged and recomputed by the exact scan kernels.
+// outside (0, 1]) are flagged and recomputed with the exact scan: by the forward kernel itself,
+// per workgroup (a whole row, or the 32 value channels a workgroup of the split launch owns:
+// value channels are independent recurrences, so the other 32 keep their chunked results unless
+// their own or the key-side gates are flagged too), and by a launch of the exact backward kernel
+// after the chunked backward.
 //
 // All contractions run on MFMA with 16-bit operands (type OP) and fp32 accumulation; the
 // state itself is carried in fp32 accumulator registers for the whole sequence.
@@ -25,10 +29,13 @@ namespace t2fw {
 struct ChunkFwdArgs {
     const void *x, *f, *q, *k, *f_key, *s0;
     void *out, *next_state, *ckpt;     // ckpt may be null
-    int32_t *row_flags;                // [2 * chunk_rows_padded(B)]: set to 1 for rows the exact kernels must redo
+    int32_t *row_flags;                // [2 * chunk_rows_padded(B)]: set to 1 for rows the chunked form cannot take
     int64_t B, T, NC;
     int32_t C;                         // checkpoint interval, multiple of 32
     int32_t heads;                     // 1: rows are [T, 64] slabs; H > 1: row b is head b % H of a [B / H, T, H, 64] tensor
+    // rows the chunked form cannot take are redone in place with the exact scan (0: only reported);
+    // launch geometry of that scan for a 64 x 64 state (set by chunk_forward)
+    int32_t redo, scan_kg, scan_tb, scan_ntiles;
 };
 
 struct ChunkBwdArgs {
@@ -73,6 +80,7 @@ typedef unsigned int u32;
 // by the compiler's wait states.
 // 16-bit element types as raw bits + conversions ---------------------------------------
 struct Bf16 {
+    using io_type = __hip_bfloat16;      // the same tensor element as the exact kernels see it
     static constexpr u16 ONE_BITS = 0x3F80;
     // smallest 16-step gate product accepted with operands of this type: the inverse
     // 1/product scales the intra-block operands and must stay far from overflow
@@ -96,6 +104,7 @@ struct Bf16 {
 };
 
 struct Fp16 {
+    using io_type = __half;
     static constexpr u16 ONE_BITS = 0x3C00;
     static constexpr float MIN_PRODUCT = 0.00390625f;               // 2^-8
     static __device__ __forceinline__ float to_f32(u16 v) { return (float)__builtin_bit_cast(_Float16, v); }

@@ -15,9 +15,11 @@
 //
 // Replaces lfw_cuda_fwd_kernel + the output einsum of the reference
 // (t2fw/csrc/lfw_kernel.cu:18-59, t2fw/csrc/lfw.cpp:45); semantics t2fw/torch.py:21-31.
+#include <algorithm>
 #include <type_traits>
 
 #include "lfw_chunk.hpp"
+#include "lfw_scan_body.hpp"
 
 // Build-time diagnostic (-DT2FW_PHASE_TIMERS): workgroup 0 accumulates shader-clock ticks
 // per phase into row_flags[64..]; off in the shipped library.
@@ -48,7 +50,8 @@ constexpr int OFF_BL = OFF_AS + CH_N * CS * 4;             // b_L [2][64] f32
 constexpr int OFF_AL = OFF_BL + 2 * CH_N * 4;              // a_L [2][64] f32
 constexpr int OPS_BYTES = OFF_AL + 2 * CH_N * 4;
 // Two stages of two steps each: a workgroup barrier every 64 tokens, the prep waves one stage ahead.
-constexpr int FWD_SMEM = 4 * OPS_BYTES;
+constexpr int OFF_VERDICT = 4 * OPS_BYTES;      // one int: some prep wave of this workgroup flagged the row
+constexpr int FWD_SMEM = OFF_VERDICT + 16;
 static_assert(FWD_SMEM <= 160 * 1024, "forward operand buffers exceed the LDS of one CU");
 static_assert(OPS_BYTES % 16 == 0, "operand buffers must keep 16-byte alignment");
 
@@ -344,7 +347,10 @@ __device__ __forceinline__ void fwd_prep_side(const ChunkFwdArgs &p, unsigned ch
         build(raw_take_tail<IOE, NV>(r, t_own, t_oth, T), nfull);
         publish(nfull);
     }
-    if (bad) p.row_flags[flag_slot] = 1;
+    if (bad) {
+        p.row_flags[flag_slot] = 1;
+        *reinterpret_cast<volatile int *>(smem + OFF_VERDICT) = 1;
+    }
     PHASE_END(4 + (tid >> 6));
 }
 
@@ -387,6 +393,7 @@ __device__ __forceinline__ void fwd_matrix_waves(const ChunkFwdArgs &p, unsigned
     if (tid == 0) {
         p.row_flags[flag_slot] = 0;
         if (clear_other_slot) p.row_flags[chunk_rows_padded(p.B) + b] = 0;
+        *reinterpret_cast<volatile int *>(smem + OFF_VERDICT) = 0;
     }
     PHASE_BEGIN();
     // One step (two blocks).  FULL: all 32 tokens exist, which leaves the body without a branch
@@ -481,6 +488,27 @@ __device__ __forceinline__ void fwd_matrix_waves(const ChunkFwdArgs &p, unsigned
     PHASE_END(tid >> 6);
 }
 
+// End of a workgroup's work on its (part of a) batch row.  A barrier publishes the prep waves'
+// verdict; if the chunked form could not take the row, the workgroup's first SCAN_THREADS threads
+// redo value channels of tiles [tile0, tile1) with the exact scan, in place, and everyone else
+// leaves (a workgroup barrier only waits for the waves that are still there).
+template <typename IOE>
+__device__ __forceinline__ void fwd_redo_if_flagged(const ChunkFwdArgs &p, unsigned char *smem, int tid, int64_t b,
+                                                    int tile0, int tile1) {
+    __syncthreads();
+    if (tid >= SCAN_THREADS || !p.redo) return;
+    if (*reinterpret_cast<volatile int *>(smem + OFF_VERDICT) == 0) return;
+    ScanFwdArgs sa{};
+    sa.x = p.x; sa.f = p.f; sa.q = p.q; sa.k = p.k; sa.f_key = p.f_key; sa.s0 = p.s0;
+    sa.out = p.out; sa.next_state = p.next_state; sa.ckpt = p.ckpt;
+    sa.B = p.B; sa.T = p.T; sa.D = CH_N; sa.K = CH_N; sa.NC = p.NC;
+    sa.C = p.C; sa.kg = p.scan_kg; sa.tb = p.scan_tb; sa.ntiles = p.scan_ntiles; sa.heads = p.heads;
+    for (int tile = tile0; tile < tile1; ++tile) {
+        __syncthreads();        // the tiles of the chunked form, or of the tile before, are no longer read
+        scan::fwd_scan_body<typename IOE::io_type, 4>(sa, b, tile);
+    }
+}
+
 template <typename IOE, typename OPE, bool HEADS>
 __global__ __launch_bounds__(FWD_THREADS) void lfw_fwd_chunk_kernel(ChunkFwdArgs p) {
     extern __shared__ __align__(16) unsigned char smem[];
@@ -498,6 +526,7 @@ __global__ __launch_bounds__(FWD_THREADS) void lfw_fwd_chunk_kernel(ChunkFwdArgs
         else
             fwd_prep_side<IOE, OPE, false, HEADS>(p, smem, tid - 256, b, tid & 63, hh, h, b);
     }
+    fwd_redo_if_flagged<IOE>(p, smem, tid, b, 0, p.scan_ntiles);
 }
 
 // Two workgroups per batch row: blockIdx = half * rows_padded + row with rows_padded a multiple of
@@ -523,6 +552,8 @@ __global__ __launch_bounds__(FWD_THREADS_HALF) void lfw_fwd_chunk_half_kernel(Ch
         const int pw = __builtin_amdgcn_readfirstlane((tid - 384) >> 6);
         fwd_prep_side<IOE, OPE, false, HEADS>(p, smem, tid - 128, b, 32 * half + (tid & 31), pw, (tid >> 5) & 1, slot);
     }
+    // this half's value channels are half of the scan's tiles
+    fwd_redo_if_flagged<IOE>(p, smem, tid, b, half * (p.scan_ntiles / 2), (half + 1) * (p.scan_ntiles / 2));
 }
 
 template <typename IOE, typename OPE, bool HEADS> int launch(const ChunkFwdArgs &a, bool split, hipStream_t stream) {
@@ -551,7 +582,19 @@ template <typename IOE, typename OPE, bool HEADS> int launch(const ChunkFwdArgs 
 
 }  // namespace
 
-int chunk_forward(const ChunkFwdArgs &a, int dtype, int op, bool split, hipStream_t stream) {
+int chunk_forward(const ChunkFwdArgs &args, int dtype, int op, bool split, hipStream_t stream) {
+    ChunkFwdArgs a = args;
+    {   // geometry of the exact scan for a 64 x 64 state, as lfw_scan.hip chooses it
+        const ScanGeom g = scan_geometry(CH_N);
+        a.scan_kg = g.kg;
+        int tb = 32;
+        tb = std::min(tb, scan::PFC * SCAN_THREADS / (g.kg * g.kpl));
+        tb = std::min(tb, scan::PFR * SCAN_THREADS / g.rows);
+        a.scan_tb = tb;
+        a.scan_ntiles = CH_N / g.rows;
+        if (g.kpl != 4 || a.scan_ntiles % 2 != 0)
+            return fail(T2FW_ERR_UNSUPPORTED, "unexpected scan geometry for a 64 x 64 state");
+    }
     if (a.heads == 1) {
         if (dtype == T2FW_F16)
             return op == 1 ? launch<Fp16, Fp16, false>(a, split, stream) : launch<Fp16, Bf16, false>(a, split, stream);

@@ -14,9 +14,7 @@
 //
 // Reference semantics: t2fw/torch.py:21-31 (forward), t2fw/csrc/lfw_kernel.cu:85-100
 // and t2fw/csrc/lfw.cpp:84-93 (backward).
-#include "common.hpp"
-#include "lfw_scan.hpp"
-#include "scan_tile.hpp"
+#include "lfw_scan_body.hpp"
 
 namespace t2fw {
 
@@ -24,300 +22,15 @@ namespace {
 
 using namespace scan;
 
-// ------------------------------------------------------------------------------------
-// forward
-// ------------------------------------------------------------------------------------
-// batch row b, tile of g.rows value channels
+// One workgroup per (batch row, tile).
 template <typename IO, int KPL>
-__device__ __forceinline__ void fwd_scan_body(const ScanFwdArgs &p, int64_t b, int tile) {
-    using Acc = typename AccOf<IO>::type;
-    extern __shared__ __align__(16) unsigned char smem_raw[];
-    const Tile g(p.kg, KPL);
-    const int tb = p.tb;
-    Acc *colL = reinterpret_cast<Acc *>(smem_raw);        // [tb][3][KP]   k, f_key, q
-    Acc *rowL = colL + (size_t)tb * 3 * g.KP;            // [tb][2][rows] x, f
-    Acc *outL = rowL + (size_t)tb * 2 * g.rows;          // [tb][rows]
-
-    const int64_t T = p.T, D = p.D, K = p.K;
-    const int64_t line0 = row_first_token(b, T, p.heads);      // [.., D] line of this row's step 0
-    const int64_t d0 = (int64_t)tile * g.rows;
-    const int64_t d = d0 + g.r;
-    const bool row_ok = d < D;
-
-    const IO *const colp[3] = {(const IO *)p.k, (const IO *)p.f_key, (const IO *)p.q};
-    const IO *const rowp[2] = {(const IO *)p.x, (const IO *)p.f};
-    const IO *s0 = (const IO *)p.s0;
-    IO *out = (IO *)p.out, *next_state = (IO *)p.next_state, *ckpt = (IO *)p.ckpt;
-
-    Acc S[KPL];
-#pragma unroll
-    for (int j = 0; j < KPL; ++j)
-        S[j] = (row_ok && g.k0 + j < K) ? to_acc(s0[(b * D + d) * K + g.k0 + j]) : Acc(0);
-
-    Prefetch<IO, 3, 2> pf;
-    block_load(pf, g, colp, rowp, b, T, 0, (int)(T < tb ? T : tb), K, D, d0, p.heads);
-
-    int until_ckpt = 0;          // steps until the next checkpoint is due
-    int64_t chunk = 0;
-    int n_prev = 0;
-    int64_t t_prev = 0;
-    for (int64_t t0 = 0; t0 < T; t0 += tb) {
-        const int n = (int)(T - t0 < tb ? T - t0 : tb);
-        __syncthreads();                                   // previous block fully consumed
-        // flush the previous block's outputs, then publish this block's inputs
-        for (int idx = threadIdx.x; idx < n_prev * g.rows; idx += SCAN_THREADS) {
-            const int tt = idx / g.rows, rr = idx % g.rows;
-            if (d0 + rr < D) out[(line0 + (t_prev + tt) * p.heads) * D + d0 + rr] = from_acc<IO>(outL[idx]);
-        }
-        block_store<IO, Acc, 3, 2>(pf, g, colL, rowL, tb);
-        __syncthreads();
-        if (t0 + tb < T) {
-            const int64_t tn = t0 + tb;
-            block_load(pf, g, colp, rowp, b, T, tn, (int)(T - tn < tb ? T - tn : tb), K, D, d0, p.heads);
-        }
-        for (int tt = 0; tt < n; ++tt) {
-            if (ckpt != nullptr) {
-                if (until_ckpt == 0) {
-                    if (row_ok) {
-#pragma unroll
-                        for (int j = 0; j < KPL; ++j)
-                            if (g.k0 + j < K)
-                                ckpt[((b * p.NC + chunk) * D + d) * K + g.k0 + j] = from_acc<IO>(S[j]);
-                    }
-                    until_ckpt = p.C;
-                    ++chunk;
-                }
-                --until_ckpt;
-            }
-            const Acc xd = rowL[(tt * 2 + 0) * g.rows + g.r];
-            const Acc fd = rowL[(tt * 2 + 1) * g.rows + g.r];
-            const Acc *ck = colL + (tt * 3 + 0) * g.KP + g.k0;
-            const Acc *cf = colL + (tt * 3 + 1) * g.KP + g.k0;
-            const Acc *cq = colL + (tt * 3 + 2) * g.KP + g.k0;
-            Acc acc = 0;
-#pragma unroll
-            for (int j = 0; j < KPL; ++j) {
-                S[j] = S[j] * (fd * cf[j]) + xd * ck[j];
-                acc += S[j] * cq[j];
-            }
-            acc = group_sum(acc, g.kg);
-            if (g.kgi == 0) outL[tt * g.rows + g.r] = acc;
-        }
-        n_prev = n;
-        t_prev = t0;
-    }
-    __syncthreads();
-    for (int idx = threadIdx.x; idx < n_prev * g.rows; idx += SCAN_THREADS) {
-        const int tt = idx / g.rows, rr = idx % g.rows;
-        if (d0 + rr < D) out[(line0 + (t_prev + tt) * p.heads) * D + d0 + rr] = from_acc<IO>(outL[idx]);
-    }
-    if (row_ok) {
-#pragma unroll
-        for (int j = 0; j < KPL; ++j)
-            if (g.k0 + j < K) next_state[(b * D + d) * K + g.k0 + j] = from_acc<IO>(S[j]);
-    }
+__global__ __launch_bounds__(SCAN_THREADS) void lfw_fwd_scan_kernel(ScanFwdArgs p) {
+    fwd_scan_body<IO, KPL>(p, blockIdx.x / p.ntiles, (int)(blockIdx.x % p.ntiles));
 }
 
 // Normal mode: one workgroup per (batch row, tile).  Fix-up mode (row_select given): one
 // workgroup per batch row that walks the tiles itself, so that the launch, in which nearly all
 // workgroups leave at once, dispatches as few of them as possible.
-template <typename IO, int KPL>
-__global__ __launch_bounds__(SCAN_THREADS) void lfw_fwd_scan_kernel(ScanFwdArgs p) {
-    if (p.row_select == nullptr) {
-        fwd_scan_body<IO, KPL>(p, blockIdx.x / p.ntiles, (int)(blockIdx.x % p.ntiles));
-        return;
-    }
-    const int64_t b = blockIdx.x;
-    if (p.row_select[b] == 0 && !(p.row_select2 && p.row_select2[b] != 0)) return;     // uniform per workgroup
-    for (int tile = 0; tile < p.ntiles; ++tile) {
-        if (tile) __syncthreads();
-        fwd_scan_body<IO, KPL>(p, b, tile);
-    }
-}
-
-// ------------------------------------------------------------------------------------
-// backward, one side.  "rows" are the dimension this launch keeps per lane-group,
-// "cols" the dimension it reduces over:
-//   side 0: rows = D, cols = K : a_r = x,  gate_r = f,     u_r = g_out ; a_c = k, gate_c = f_key, u_c = q
-//           outputs d_a = d_x, d_gate = d_f, plus d_s0
-//   side 1: rows = K, cols = D : a_r = k,  gate_r = f_key, u_r = q     ; a_c = x, gate_c = f,     u_c = g_out
-//           outputs d_a = d_k, d_gate = d_f_key, d_u = d_q
-// State element (row, col) lives at [b, row, col] (side 0) or [b, col, row] (side 1).
-//
-// Per chunk: the states at segment starts are recomputed from the checkpoint and kept
-// in LDS (lane-private slots); then segments are visited last to first, each segment's
-// SEG states are recomputed into registers and the adjoint runs backwards over them.
-// ------------------------------------------------------------------------------------
-template <int KPL> struct SegLen { static constexpr int value = (32 / KPL) < 1 ? 1 : (KPL <= 4 ? 8 : 32 / KPL); };
-
-template <typename IO, int KPL, int SIDE>
-__device__ __forceinline__ void bwd_scan_body(const ScanBwdArgs &p, int64_t b, int tile) {
-    using Acc = typename AccOf<IO>::type;
-    constexpr int SEG = SegLen<KPL>::value;
-    extern __shared__ __align__(16) unsigned char smem_raw[];
-    const Tile g(p.kg, KPL);
-    Acc *colL = reinterpret_cast<Acc *>(smem_raw);        // [SEG][3][KP]   a_c, gate_c, u_c
-    Acc *rowL = colL + (size_t)SEG * 3 * g.KP;           // [SEG][3][rows] a_r, gate_r, u_r
-    Acc *outL = rowL + (size_t)SEG * 3 * g.rows;         // [SEG][3][rows] d_a, d_gate, d_u
-    Acc *subL = outL + (size_t)SEG * 3 * g.rows;         // [nseg_max][KPL][SCAN_THREADS]
-
-    const int64_t T = p.T;
-    const int64_t line0 = row_first_token(b, T, p.heads);      // [.., D|K] line of this row's step 0
-    const int64_t nrows = SIDE == 0 ? p.D : p.K, ncols = SIDE == 0 ? p.K : p.D;
-    const int64_t row0 = (int64_t)tile * g.rows;
-    const int64_t row = row0 + g.r;
-    const bool row_ok = row < nrows;
-    const int64_t DK = p.D * p.K;
-
-    const IO *const colp[3] = {(const IO *)(SIDE == 0 ? p.k : p.x), (const IO *)(SIDE == 0 ? p.f_key : p.f),
-                               (const IO *)(SIDE == 0 ? p.q : p.g_out)};
-    const IO *const rowp[3] = {(const IO *)(SIDE == 0 ? p.x : p.k), (const IO *)(SIDE == 0 ? p.f : p.f_key),
-                               (const IO *)(SIDE == 0 ? p.g_out : p.q)};
-    IO *d_a = (IO *)(SIDE == 0 ? p.d_x : p.d_k);
-    IO *d_gate = (IO *)(SIDE == 0 ? p.d_f : p.d_f_key);
-    IO *d_u = (IO *)p.d_q;   // side 1 only
-    const IO *ckpt = (const IO *)p.ckpt;
-
-    // element offset of (row, col0 + j) inside one [D,K] state
-    auto st_off = [&](int j) -> int64_t {
-        return SIDE == 0 ? row * p.K + (g.k0 + j) : (int64_t)(g.k0 + j) * p.K + row;
-    };
-    auto el_ok = [&](int j) -> bool { return row_ok && g.k0 + j < ncols; };
-
-    Acc G[KPL];
-    {
-        const IO *gs = (const IO *)p.g_state + b * DK;
-#pragma unroll
-        for (int j = 0; j < KPL; ++j) G[j] = el_ok(j) ? to_acc(gs[st_off(j)]) : Acc(0);
-    }
-
-    const int C = p.C;
-    const bool use_sub = p.use_sub != 0;
-    Prefetch<IO, 3, 3> pf;
-
-    for (int64_t c = p.NC - 1; c >= 0; --c) {
-        const int64_t tc0 = c * C;
-        const int len = (int)(T - tc0 < C ? T - tc0 : C);
-        const int nseg = (len + SEG - 1) / SEG;
-        const IO *ck = ckpt + (b * p.NC + c) * DK;
-        Acc S[KPL];
-#pragma unroll
-        for (int j = 0; j < KPL; ++j) S[j] = el_ok(j) ? to_acc(ck[st_off(j)]) : Acc(0);
-
-        // ---- forward sweep: states at segment starts -> subL (all but the last are advanced)
-        if (use_sub) {
-            for (int s = 0; s < nseg; ++s) {
-#pragma unroll
-                for (int j = 0; j < KPL; ++j) subL[((size_t)s * KPL + j) * SCAN_THREADS + threadIdx.x] = S[j];
-                if (s == nseg - 1) break;
-                const int64_t t0 = tc0 + (int64_t)s * SEG;
-                block_load(pf, g, colp, rowp, b, T, t0, SEG, ncols, nrows, row0, p.heads);
-                __syncthreads();
-                block_store<IO, Acc, 3, 3>(pf, g, colL, rowL, SEG);
-                __syncthreads();
-#pragma unroll
-                for (int tt = 0; tt < SEG; ++tt) {
-                    const Acc ar = rowL[(tt * 3 + 0) * g.rows + g.r];
-                    const Acc fr = rowL[(tt * 3 + 1) * g.rows + g.r];
-                    const Acc *ca = colL + (tt * 3 + 0) * g.KP + g.k0;
-                    const Acc *cf = colL + (tt * 3 + 1) * g.KP + g.k0;
-#pragma unroll
-                    for (int j = 0; j < KPL; ++j) S[j] = S[j] * (fr * cf[j]) + ar * ca[j];
-                }
-            }
-        }
-
-        // ---- reverse over segments
-        for (int s = nseg - 1; s >= 0; --s) {
-            const int64_t t0 = tc0 + (int64_t)s * SEG;
-            const int n = (int)(len - s * SEG < SEG ? len - s * SEG : SEG);
-            Acc st[SEG + 1][KPL];
-            if (use_sub) {
-#pragma unroll
-                for (int j = 0; j < KPL; ++j) st[0][j] = subL[((size_t)s * KPL + j) * SCAN_THREADS + threadIdx.x];
-            } else {
-                // no room for segment-start states: replay from the checkpoint
-#pragma unroll
-                for (int j = 0; j < KPL; ++j) st[0][j] = el_ok(j) ? to_acc(ck[st_off(j)]) : Acc(0);
-                for (int s2 = 0; s2 < s; ++s2) {
-                    block_load(pf, g, colp, rowp, b, T, tc0 + (int64_t)s2 * SEG, SEG, ncols, nrows, row0, p.heads);
-                    __syncthreads();
-                    block_store<IO, Acc, 3, 3>(pf, g, colL, rowL, SEG);
-                    __syncthreads();
-#pragma unroll
-                    for (int tt = 0; tt < SEG; ++tt) {
-                        const Acc ar = rowL[(tt * 3 + 0) * g.rows + g.r];
-                        const Acc fr = rowL[(tt * 3 + 1) * g.rows + g.r];
-                        const Acc *ca = colL + (tt * 3 + 0) * g.KP + g.k0;
-                        const Acc *cf = colL + (tt * 3 + 1) * g.KP + g.k0;
-#pragma unroll
-                        for (int j = 0; j < KPL; ++j) st[0][j] = st[0][j] * (fr * cf[j]) + ar * ca[j];
-                    }
-                }
-            }
-            block_load(pf, g, colp, rowp, b, T, t0, n, ncols, nrows, row0, p.heads);
-            __syncthreads();
-            block_store<IO, Acc, 3, 3>(pf, g, colL, rowL, SEG);
-            __syncthreads();
-            // recompute the segment's states into registers
-#pragma unroll
-            for (int tt = 0; tt < SEG; ++tt) {
-                const Acc ar = rowL[(tt * 3 + 0) * g.rows + g.r];
-                const Acc fr = rowL[(tt * 3 + 1) * g.rows + g.r];
-                const Acc *ca = colL + (tt * 3 + 0) * g.KP + g.k0;
-                const Acc *cf = colL + (tt * 3 + 1) * g.KP + g.k0;
-#pragma unroll
-                for (int j = 0; j < KPL; ++j) st[tt + 1][j] = st[tt][j] * (fr * cf[j]) + ar * ca[j];
-            }
-            // adjoint, last step of the segment first
-#pragma unroll
-            for (int tt = SEG - 1; tt >= 0; --tt) {
-                if (tt < n) {
-                    const Acc fr = rowL[(tt * 3 + 1) * g.rows + g.r];
-                    const Acc ur = rowL[(tt * 3 + 2) * g.rows + g.r];
-                    const Acc *ca = colL + (tt * 3 + 0) * g.KP + g.k0;
-                    const Acc *cf = colL + (tt * 3 + 1) * g.KP + g.k0;
-                    const Acc *cu = colL + (tt * 3 + 2) * g.KP + g.k0;
-                    Acc sa = 0, sg = 0, su = 0;
-#pragma unroll
-                    for (int j = 0; j < KPL; ++j) {
-                        G[j] += ur * cu[j];                       // G_t = g_t (x) q_t + ...
-                        sa += G[j] * ca[j];                       // d_x / d_k
-                        sg += (G[j] * st[tt][j]) * cf[j];         // d_f / d_f_key   (uses S_{t-1})
-                        if (SIDE == 1) su += st[tt + 1][j] * cu[j];   // d_q = S_t^T g_t
-                        G[j] *= fr * cf[j];
-                    }
-                    sa = group_sum(sa, g.kg);
-                    sg = group_sum(sg, g.kg);
-                    if (SIDE == 1) su = group_sum(su, g.kg);
-                    if (g.kgi == 0) {
-                        outL[(tt * 3 + 0) * g.rows + g.r] = sa;
-                        outL[(tt * 3 + 1) * g.rows + g.r] = sg;
-                        if (SIDE == 1) outL[(tt * 3 + 2) * g.rows + g.r] = su;
-                    }
-                }
-            }
-            __syncthreads();
-            for (int idx = threadIdx.x; idx < n * g.rows; idx += SCAN_THREADS) {
-                const int tt = idx / g.rows, rr = idx % g.rows;
-                if (row0 + rr < nrows) {
-                    const int64_t o = (line0 + (t0 + tt) * p.heads) * nrows + row0 + rr;
-                    d_a[o] = from_acc<IO>(outL[(tt * 3 + 0) * g.rows + rr]);
-                    d_gate[o] = from_acc<IO>(outL[(tt * 3 + 1) * g.rows + rr]);
-                    if (SIDE == 1) d_u[o] = from_acc<IO>(outL[(tt * 3 + 2) * g.rows + rr]);
-                }
-            }
-        }
-    }
-    if (SIDE == 0) {
-        IO *ds = (IO *)p.d_s0 + b * DK;
-#pragma unroll
-        for (int j = 0; j < KPL; ++j)
-            if (el_ok(j)) ds[st_off(j)] = from_acc<IO>(G[j]);
-    }
-}
-
-// workgroup -> (batch row, tiles): as for the forward kernel
 template <typename IO, int KPL, int SIDE> __device__ __forceinline__ void bwd_scan_rows(const ScanBwdArgs &p) {
     if (p.row_select == nullptr) {
         bwd_scan_body<IO, KPL, SIDE>(p, blockIdx.x / p.ntiles, (int)(blockIdx.x % p.ntiles));
@@ -356,7 +69,7 @@ int launch_fwd(const ScanFwdArgs &a, const ScanGeom &g, hipStream_t stream) {
     const size_t smem = ((size_t)a.tb * 3 * g.kg * g.kpl + (size_t)a.tb * 3 * g.rows) * sizeof(Acc);
     ScanFwdArgs a2 = a;
     a2.ntiles = (int)((a.D + g.rows - 1) / g.rows);
-    const int64_t nblocks = a.row_select != nullptr ? a.B : a.B * a2.ntiles;
+    const int64_t nblocks = a.B * a2.ntiles;
     if (nblocks > 0x7fffffffLL) return fail(T2FW_ERR_UNSUPPORTED, "grid of %lld workgroups is too large", (long long)nblocks);
     dim3 grid((unsigned)nblocks, 1, 1);
     hipLaunchKernelGGL((lfw_fwd_scan_kernel<IO, KPL>), grid, dim3(SCAN_THREADS), smem, stream, a2);

@@ -8,8 +8,6 @@ namespace t2fw {
 struct ScanFwdArgs {
     const void *x, *f, *q, *k, *f_key, *s0;
     void *out, *next_state, *ckpt;      // ckpt may be null
-    const int32_t *row_select;          // null, or per batch row: 0 = skip the row ...
-    const int32_t *row_select2;         // ... unless this second per-row array (may be null) is nonzero there
     int64_t B, T, D, K, NC;
     int32_t C, kg, tb, ntiles;
     int32_t heads;                      // 1, or H: row b is head b % H of [B/H, T, H, D|K] tensors (x, f, q, k, f_key, out)
@@ -18,7 +16,7 @@ struct ScanFwdArgs {
 struct ScanBwdArgs {
     const void *g_out, *g_state, *x, *f, *q, *k, *f_key, *ckpt;
     void *d_x, *d_f, *d_q, *d_k, *d_f_key, *d_s0;
-    const int32_t *row_select;
+    const int32_t *row_select;          // null, or per batch row: 0 = skip the row
     int64_t B, T, D, K, NC;
     int32_t C, kg, use_sub, ntiles;
     int32_t heads;                      // as for the forward (inputs, g_out and the five [.., T, .., D|K] gradients)

@@ -176,15 +176,29 @@ def test_rows_outside_the_gate_range_fall_back_to_the_exact_kernels(kind):
         f[1, 11:26, 3] = 6e-8
     out, nxt, ckpt, grads, flagged = run_abi((x, f, q, k, fk, s), go, gs, 64)
     assert flagged == (1, 1), flagged
-    # flagged rows are recomputed by the exact kernels: tight tolerance there, chunk tolerance elsewhere
+    # The forward at this batch size runs one workgroup per (row, 32 value channels), and each
+    # redoes its own channels with the exact recurrence when their gates (or the key-side gates,
+    # which both see) are outside the range: tight tolerance on those channels, chunk tolerance on
+    # the others.  The backward redoes the whole row from the checkpoints the forward left, so its
+    # value-side results are tight on the same channels and its key-side results (sums over all
+    # value channels) are tight when the whole row was redone.
+    exact = {"zero_gate": slice(0, 32), "zero_gate_upper_channels": slice(32, 64), "negative_gate": slice(0, 32),
+             "nan_free_inf_gate": slice(0, 32)}.get(kind, slice(0, 64))
+    whole = exact == slice(0, 64)
     r_out, r_nxt = c_oracle.lfw_forward(x, f, q, k, fk, s)
     r_grads = c_oracle.lfw_backward(go, gs, x, f, q, k, fk, s)
-    assert_close(out[1:2], r_out[1:2], torch.float16, "outputs[flagged row]")
-    assert_close(nxt[1:2], r_nxt[1:2], torch.float16, "next_state[flagged row]")
+    assert_close(out[1:2, :, exact], r_out[1:2, :, exact], torch.float16, "outputs[flagged row]")
+    assert_close(nxt[1:2, exact], r_nxt[1:2, exact], torch.float16, "next_state[flagged row]")
     for n, g, r in zip(NAMES, grads, r_grads):
-        assert_close(g[1:2], r[1:2], torch.float16, n + "[flagged row]")
+        if n in ("d_x", "d_f"):
+            assert_close(g[1:2, :, exact], r[1:2, :, exact], torch.float16, n + "[flagged row]")
+        elif n == "d_state":
+            assert_close(g[1:2, exact], r[1:2, exact], torch.float16, n + "[flagged row]")
+        elif whole:
+            assert_close(g[1:2], r[1:2], torch.float16, n + "[flagged row]")
         assert_close(g, r, torch.float16, n, tol=TOL_CHUNK_GATE if n in ("d_f", "d_f_key") else TOL_CHUNK)
     assert_close(out, r_out, torch.float16, "outputs", tol=TOL_CHUNK)
+    assert_close(nxt, r_nxt, torch.float16, "next_state", tol=TOL_CHUNK)
 
 
 def test_fp16_operand_flag():
