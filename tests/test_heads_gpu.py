@@ -130,6 +130,17 @@ def test_flagged_rows_are_redone_by_the_exact_kernels_in_place():
     check_heads((x, f, q, k, fk, s), go, gs, B, H, 32, torch.float16, expect_flagged=2)
 
 
+def test_flagged_rows_with_one_workgroup_per_row():
+    B, H, T = 23, 6, 70                # 138 rows: the forward runs one workgroup per row
+    x, f, q, k, fk, s, go, gs = make_config_inputs(B * H, T, 64, 64, torch.bfloat16, seed=19, gate_mean=3.0,
+                                                    state_std=0.3)
+    f, fk = f.clone(), fk.clone()
+    f[137, 69, 33] = 0.0               # last row, last token
+    fk[6, 0, 0] = -1.0                 # batch 1, head 0, first token
+    check_heads((x, f, q, k, fk, s), go, gs, B, H, 64, torch.bfloat16, expect_flagged=2,
+                oracle_rows=[0, 5, 6, 7, 136, 137])
+
+
 @pytest.mark.parametrize("dtype,B,H,T,D,K", [(torch.float32, 2, 3, 77, 33, 17), (torch.float16, 1, 4, 50, 32, 16),
                                              (torch.float64, 2, 2, 40, 5, 9), (torch.bfloat16, 2, 2, 300, 64, 32),
                                              (torch.float32, 1, 2, 70, 64, 64)])

@@ -99,9 +99,10 @@ def test_batch_larger_than_half_the_device():
     B, T = 136, 80
     x, f, q, k, fk, s, go, gs = make_config_inputs(B, T, 64, 64, torch.float16, seed=31, state_std=0.2)
     f = f.clone()
-    f[135, 70, 50] = 1.25               # one row for the exact kernels, in the last workgroup
+    f[135, 70, 50] = 1.25               # rows for the exact recurrence: one in the last workgroup,
+    f[64, 3, 7] = 0.0                   # one whose chunked form divides by zero
     out, nxt, ckpt, grads, flagged = run_abi((x, f, q, k, fk, s), go, gs, 64)
-    assert flagged == (1, 1), flagged
+    assert flagged == (2, 2), flagged
     rows = [0, 63, 64, 127, 128, 135]
     sub = [t[rows] for t in (x, f, q, k, fk, s)]
     r_out, r_nxt = c_oracle.lfw_forward(*sub)
@@ -110,6 +111,12 @@ def test_batch_larger_than_half_the_device():
     assert_close(nxt[rows], r_nxt, torch.float16, "next_state", tol=TOL_CHUNK)
     for n, g, r in zip(NAMES, grads, r_grads):
         assert_close(g[rows], r, torch.float16, n, tol=TOL_CHUNK_GATE if n in ("d_f", "d_f_key") else TOL_CHUNK)
+    # one workgroup per row: a flagged row is redone whole, in both directions
+    for i in (2, 5):
+        assert_close(out[rows[i]], r_out[i], torch.float16, "outputs[flagged row %d]" % rows[i])
+        assert_close(nxt[rows[i]], r_nxt[i], torch.float16, "next_state[flagged row %d]" % rows[i])
+        for n, g, r in zip(NAMES, grads, r_grads):
+            assert_close(g[rows[i]], r[i], torch.float16, "%s[flagged row %d]" % (n, rows[i]))
 
 
 def test_flagged_rows_with_a_partial_last_block():
