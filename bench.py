@@ -5,7 +5,7 @@ A "step" is one forward + backward pass of the decay-rule recurrence over one ba
 synthetic input already resident in HBM, at the headline configuration
 (B*H=96, T=1024, D=K=64, fp16 I/O, checkpoint interval 64).  Prints ONE JSON line.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg3|cfg3_heads|cfg2|cfg4|cfg5|copy256]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg3|cfg3_heads|cfg2|cfg4|cfg5|dfw|copy256]
                     [--no-cpu-baseline]
 
 value      = B*T*steps / wall time of the timed region, in Mtokens/s (token = one
@@ -16,6 +16,8 @@ roofline   = algorithmic bytes of the dominant kernel / its mean duration measur
              exact redo of flagged rows, for the backward a launch of its own, so that the
              events bracket that one kernel), against
              8 TB/s.  `traffic` comes from profiles/traffic_<workload>.json (rocprofv3 counters).
+dfw        = the delta-rule kernels (forward + backward) at cfg3's shape in fp32, the dtype the
+             reference tests them in.
 copy256    = calibration workload for those counters: a 256 MiB device-to-device copy.
 cpu_baseline = the TorchScript restatement of the reference loop (oracle/), fp32,
              forward + autograd backward, timed on this host's cores on a bounded sample.
@@ -62,7 +64,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", default="cfg3", choices=sorted(WORKLOADS) + ["copy256"])
+    ap.add_argument("--workload", default="cfg3", choices=sorted(WORKLOADS) + ["dfw", "copy256"])
     ap.add_argument("--ckpt-interval", type=int, default=64)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--force-scan", action="store_true", help="exact scan kernels only")
@@ -83,6 +85,8 @@ def main():
         return bench_generation(args)
     if args.workload == "copy256":
         return bench_copy(args)
+    if args.workload == "dfw":
+        return bench_dfw(args)
     lib = _lib.load()
     w = WORKLOADS[args.workload]
     B, T, D, K = w["B"], w["T"], w["D"], w["K"]
@@ -284,6 +288,84 @@ def bench_copy(args):
                       "ms_per_step": round(wall / args.steps * 1e3, 5), "higher_is_better": True, "scaling": "weak",
                       "vs_baseline": None, "dtype": "u8", "data": "synthetic",
                       "config": {"workload": "copy256: torch copy_ of 268435456 bytes, device to device"}}))
+
+
+def bench_dfw(args):
+    """Delta rule (t2fw/functional_dfw.py:29-65) forward + backward through the C ABI: B=96, T=1024,
+    D=M=64, fp32, keys built as the reference's test builds them (tests/test_dfw.py:45-46).  A step
+    is one forward and one backward call; the backward call is two launches (value side, then
+    query/key side).  Bytes: forward reads q,k,v,s0 and writes out,delta,final_state; backward
+    reads g_out,g_state,q,k,delta,final_state and writes d_q,d_k,d_v,d_s0."""
+    import torch
+    from t2fw_amd import _lib
+    lib = _lib.load()
+    B, T, D, M = 96, 1024, 64, 64
+    dtype, es = torch.float32, 4
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    code = _lib.DTYPE_CODE[dtype]
+    stream = _lib.current_stream_handle(dev)
+    per_set = (B * T * (3 * D + 2 * M) + B * T * (2 * D + 2 * M)) * es
+    nsets = max(2, min(16, int(1.2e9 // per_set) + 1))
+    sets = []
+    for i in range(nsets):
+        g = torch.Generator().manual_seed(i)
+        v = torch.randn(B, T, D, generator=g)
+        q = torch.randn(B, T, M, generator=g)
+        k = torch.randn(B, T, M, generator=g)
+        k = torch.softmax(k, dim=-1) * torch.sigmoid(k.mean(dim=-1, keepdim=True))
+        s0 = torch.randn(B, D, M, generator=g)
+        go = torch.randn(B, T, D, generator=g)
+        gs = torch.randn(B, D, M, generator=g)
+        d = {n: t.to(dev) for n, t in (("q", q), ("k", k), ("v", v), ("s0", s0), ("go", go), ("gs", gs))}
+        for n, like in (("out", "v"), ("delta", "v"), ("fin", "s0"), ("d_q", "q"), ("d_k", "k"), ("d_v", "v"), ("d_s0", "s0")):
+            d[n] = torch.empty_like(d[like])
+        sets.append(d)
+    P = _lib.ptr
+
+    def fwd(d):
+        _lib.check(lib.t2fw_dfw_forward(P(d["q"]), P(d["k"]), P(d["v"]), P(d["s0"]), P(d["out"]), P(d["fin"]),
+                                        P(d["delta"]), B, T, D, M, code, stream))
+
+    def bwd(d):
+        _lib.check(lib.t2fw_dfw_backward(P(d["go"]), P(d["gs"]), P(d["q"]), P(d["k"]), P(d["delta"]), P(d["fin"]),
+                                         P(d["d_q"]), P(d["d_k"]), P(d["d_v"]), P(d["d_s0"]), B, T, D, M, code, stream))
+
+    for i in range(args.warmup):
+        fwd(sets[i % nsets]); bwd(sets[i % nsets])
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        fwd(sets[i % nsets]); bwd(sets[i % nsets])
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    nrep = min(args.steps, 100)
+    ev = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(nrep)]
+    for i in range(nrep):
+        d = sets[i % nsets]
+        ev[i][0].record(); fwd(d); ev[i][1].record(); bwd(d); ev[i][2].record()
+    torch.cuda.synchronize()
+    fwd_ms = sum(e[0].elapsed_time(e[1]) for e in ev) / nrep
+    bwd_ms = sum(e[1].elapsed_time(e[2]) for e in ev) / nrep
+    tok = B * T
+    fwd_bytes = (tok * (2 * M + 3 * D) + 2 * B * D * M) * es
+    bwd_bytes = (tok * (2 * D + 2 * M + 2 * M + D) + 3 * B * D * M) * es
+    ms_per_step = wall / args.steps * 1e3
+    achieved = bwd_bytes / (bwd_ms * 1e-3) / 1e9
+    line = {
+        "metric": "delta rule fwd+bwd Mtokens/s, B=96 T=1024 D=M=64 fp32", "value": round(tok * args.steps / wall / 1e6, 1),
+        "unit": "Mtokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "dfw: B=%d T=%d D=%d M=%d float32 fwd+bwd" % (B, T, D, M), "input_sets_rotated": nsets},
+        "forward_avg_ms": round(fwd_ms, 5), "backward_avg_ms": round(bwd_ms, 5),
+        "whole_step_algorithmic_GBs": round((fwd_bytes + bwd_bytes) / (ms_per_step * 1e-3) / 1e9, 1),
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None, "kernel": "backward (two launches)",
+                     "algorithmic_bytes": bwd_bytes, "avg_launch_ms": round(bwd_ms, 5)},
+        "cpu_baseline": None,
+    }
+    print(json.dumps(line))
 
 
 def bench_generation(args):

@@ -12,6 +12,8 @@
 // state stays in registers for the whole sequence and inputs are staged through LDS one time
 // block ahead.  The backward pass is two launches: rows along D give d_v and d_state, rows
 // along M give d_q and d_k (and consume d_v), so every reduction is along the lane-shared row.
+#include <type_traits>
+
 #include "common.hpp"
 #include "dfw_scan.hpp"
 #include "scan_tile.hpp"
@@ -59,6 +61,33 @@ __global__ __launch_bounds__(SCAN_THREADS) void dfw_fwd_kernel(DfwFwdArgs p) {
             }
         }
     };
+    // The steps of one staged block.  kgv: lanes per state row, as a compile-time constant for the
+    // common geometry (which leaves the cross-lane sums without branches and the LDS strides as
+    // immediates) or as a run-time value.
+    auto steps = [&](int n, auto kgv) {
+        const int kg = kgv, rows = SCAN_THREADS / kg, KP = kg * KPL;
+#pragma unroll 4
+        for (int tt = 0; tt < n; ++tt) {
+            const Acc vd = rowL[tt * rows + g.r];
+            const Acc *ck = colL + (tt * 2 + 0) * KP + g.k0;
+            const Acc *cq = colL + (tt * 2 + 1) * KP + g.k0;
+            Acc so = 0, sq = 0;
+#pragma unroll
+            for (int j = 0; j < KPL; ++j) {
+                so += S[j] * ck[j];       // old = S k
+                sq += S[j] * cq[j];       // out = S q (state before the update)
+            }
+            so = group_sum(so, kg);
+            sq = group_sum(sq, kg);
+            const Acc dl = vd - so;
+#pragma unroll
+            for (int j = 0; j < KPL; ++j) S[j] += dl * ck[j];
+            if (g.kgi == 0) {
+                outL[(tt * 2 + 0) * rows + g.r] = sq;
+                outL[(tt * 2 + 1) * rows + g.r] = dl;
+            }
+        }
+    };
     for (int64_t t0 = 0; t0 < T; t0 += tb) {
         const int n = (int)(T - t0 < tb ? T - t0 : tb);
         __syncthreads();
@@ -69,26 +98,10 @@ __global__ __launch_bounds__(SCAN_THREADS) void dfw_fwd_kernel(DfwFwdArgs p) {
             const int64_t tn = t0 + tb;
             block_load(pf, g, colp, rowp, b, T, tn, (int)(T - tn < tb ? T - tn : tb), M, D, d0);
         }
-        for (int tt = 0; tt < n; ++tt) {
-            const Acc vd = rowL[tt * g.rows + g.r];
-            const Acc *ck = colL + (tt * 2 + 0) * g.KP + g.k0;
-            const Acc *cq = colL + (tt * 2 + 1) * g.KP + g.k0;
-            Acc so = 0, sq = 0;
-#pragma unroll
-            for (int j = 0; j < KPL; ++j) {
-                so += S[j] * ck[j];       // old = S k
-                sq += S[j] * cq[j];       // out = S q (state before the update)
-            }
-            so = group_sum(so, g.kg);
-            sq = group_sum(sq, g.kg);
-            const Acc dl = vd - so;
-#pragma unroll
-            for (int j = 0; j < KPL; ++j) S[j] += dl * ck[j];
-            if (g.kgi == 0) {
-                outL[(tt * 2 + 0) * g.rows + g.r] = sq;
-                outL[(tt * 2 + 1) * g.rows + g.r] = dl;
-            }
-        }
+        if (g.kg == 16)
+            steps(n, std::integral_constant<int, 16>{});
+        else
+            steps(n, g.kg);
         n_prev = n;
         t_prev = t0;
     }
@@ -167,32 +180,28 @@ __global__ __launch_bounds__(SCAN_THREADS) void dfw_bwd_kernel(DfwBwdArgs p) {
             }
         }
     };
-    for (int64_t blk = nblk - 1; blk >= 0; --blk) {
-        const int64_t t0 = blk * tb;
-        const int n = (int)(T - t0 < tb ? T - t0 : tb);
-        __syncthreads();
-        flush();
-        block_store<IO, Acc, NCA, NRA>(pf, g, colL, rowL, tb);
-        __syncthreads();
-        if (blk > 0) block_load(pf, g, colr, rowr, b, T, t0 - tb, tb, ncols, nrows, row0);
+    // The steps of one staged block, last to first; kgv as in the forward kernel.
+    auto steps = [&](int n, auto kgv) {
+        const int kg = kgv, rows = SCAN_THREADS / kg, KP = kg * KPL;
+#pragma unroll 4
         for (int tt = n - 1; tt >= 0; --tt) {
             if (SIDE == 0) {
-                const Acc gr = rowL[tt * g.rows + g.r];
-                const Acc *ck = colL + (tt * 2 + 0) * g.KP + g.k0;
-                const Acc *cq = colL + (tt * 2 + 1) * g.KP + g.k0;
+                const Acc gr = rowL[tt * rows + g.r];
+                const Acc *ck = colL + (tt * 2 + 0) * KP + g.k0;
+                const Acc *cq = colL + (tt * 2 + 1) * KP + g.k0;
                 Acc dv = 0;
 #pragma unroll
                 for (int j = 0; j < KPL; ++j) dv += G[j] * ck[j];          // dv_t = G_t k_t
-                dv = group_sum(dv, g.kg);
+                dv = group_sum(dv, kg);
 #pragma unroll
                 for (int j = 0; j < KPL; ++j) G[j] += gr * cq[j] - dv * ck[j];
-                if (g.kgi == 0) outL[tt * g.rows + g.r] = dv;
+                if (g.kgi == 0) outL[tt * rows + g.r] = dv;
             } else {
-                const Acc kr = rowL[(tt * 2 + 0) * g.rows + g.r];
-                const Acc qr = rowL[(tt * 2 + 1) * g.rows + g.r];
-                const Acc *cd = colL + (tt * 3 + 0) * g.KP + g.k0;   // delta
-                const Acc *cg = colL + (tt * 3 + 1) * g.KP + g.k0;   // g_out
-                const Acc *cv = colL + (tt * 3 + 2) * g.KP + g.k0;   // d_v
+                const Acc kr = rowL[(tt * 2 + 0) * rows + g.r];
+                const Acc qr = rowL[(tt * 2 + 1) * rows + g.r];
+                const Acc *cd = colL + (tt * 3 + 0) * KP + g.k0;   // delta
+                const Acc *cg = colL + (tt * 3 + 1) * KP + g.k0;   // g_out
+                const Acc *cv = colL + (tt * 3 + 2) * KP + g.k0;   // d_v
                 Acc sk = 0, sq = 0;
 #pragma unroll
                 for (int j = 0; j < KPL; ++j) {
@@ -201,14 +210,27 @@ __global__ __launch_bounds__(SCAN_THREADS) void dfw_bwd_kernel(DfwBwdArgs p) {
                     sk += G[j] * cd[j] - S[j] * cv[j];                // dk = G_t^T delta - S_{t-1}^T dv
                     G[j] += cg[j] * qr - cv[j] * kr;
                 }
-                sk = group_sum(sk, g.kg);
-                sq = group_sum(sq, g.kg);
+                sk = group_sum(sk, kg);
+                sq = group_sum(sq, kg);
                 if (g.kgi == 0) {
-                    outL[(tt * 2 + 0) * g.rows + g.r] = sk;
-                    outL[(tt * 2 + 1) * g.rows + g.r] = sq;
+                    outL[(tt * 2 + 0) * rows + g.r] = sk;
+                    outL[(tt * 2 + 1) * rows + g.r] = sq;
                 }
             }
         }
+    };
+    for (int64_t blk = nblk - 1; blk >= 0; --blk) {
+        const int64_t t0 = blk * tb;
+        const int n = (int)(T - t0 < tb ? T - t0 : tb);
+        __syncthreads();
+        flush();
+        block_store<IO, Acc, NCA, NRA>(pf, g, colL, rowL, tb);
+        __syncthreads();
+        if (blk > 0) block_load(pf, g, colr, rowr, b, T, t0 - tb, tb, ncols, nrows, row0);
+        if (g.kg == 16)
+            steps(n, std::integral_constant<int, 16>{});
+        else
+            steps(n, g.kg);
         n_prev = n;
         t_prev = t0;
     }

@@ -505,7 +505,7 @@ __device__ __forceinline__ void fwd_redo_if_flagged(const ChunkFwdArgs &p, unsig
     sa.C = p.C; sa.kg = p.scan_kg; sa.tb = p.scan_tb; sa.ntiles = p.scan_ntiles; sa.heads = p.heads;
     for (int tile = tile0; tile < tile1; ++tile) {
         __syncthreads();        // the tiles of the chunked form, or of the tile before, are no longer read
-        scan::fwd_scan_body<typename IOE::io_type, 4>(sa, b, tile);
+        scan::fwd_scan_body_kg<typename IOE::io_type, 4, 16>(sa, b, tile);
     }
 }
 
@@ -592,7 +592,7 @@ int chunk_forward(const ChunkFwdArgs &args, int dtype, int op, bool split, hipSt
         tb = std::min(tb, scan::PFR * SCAN_THREADS / g.rows);
         a.scan_tb = tb;
         a.scan_ntiles = CH_N / g.rows;
-        if (g.kpl != 4 || a.scan_ntiles % 2 != 0)
+        if (g.kpl != 4 || g.kg != 16 || a.scan_ntiles % 2 != 0)
             return fail(T2FW_ERR_UNSUPPORTED, "unexpected scan geometry for a 64 x 64 state");
     }
     if (a.heads == 1) {

@@ -16,12 +16,14 @@ namespace scan {
 // ------------------------------------------------------------------------------------
 // forward
 // ------------------------------------------------------------------------------------
-// batch row b, tile of g.rows value channels
-template <typename IO, int KPL>
-__device__ __forceinline__ void fwd_scan_body(const ScanFwdArgs &p, int64_t b, int tile) {
+// batch row b, tile of g.rows value channels.  KG: lanes per state row as a compile-time constant
+// (p.kg must equal it), which leaves the cross-lane sums without branches and the LDS strides as
+// immediates; 0 = take p.kg at run time.
+template <typename IO, int KPL, int KG>
+__device__ __forceinline__ void fwd_scan_body_kg(const ScanFwdArgs &p, int64_t b, int tile) {
     using Acc = typename AccOf<IO>::type;
     extern __shared__ __align__(16) unsigned char smem_raw[];
-    const Tile g(p.kg, KPL);
+    const Tile g(KG > 0 ? KG : p.kg, KPL);
     const int tb = p.tb;
     Acc *colL = reinterpret_cast<Acc *>(smem_raw);        // [tb][3][KP]   k, f_key, q
     Acc *rowL = colL + (size_t)tb * 3 * g.KP;            // [tb][2][rows] x, f
@@ -64,6 +66,7 @@ __device__ __forceinline__ void fwd_scan_body(const ScanFwdArgs &p, int64_t b, i
             const int64_t tn = t0 + tb;
             block_load(pf, g, colp, rowp, b, T, tn, (int)(T - tn < tb ? T - tn : tb), K, D, d0, p.heads);
         }
+#pragma unroll 4
         for (int tt = 0; tt < n; ++tt) {
             if (ckpt != nullptr) {
                 if (until_ckpt == 0) {
@@ -107,6 +110,18 @@ __device__ __forceinline__ void fwd_scan_body(const ScanFwdArgs &p, int64_t b, i
     }
 }
 
+// The common geometry (16 lanes per state row: 16 to 64 columns) runs with constant strides.
+template <typename IO, int KPL>
+__device__ __forceinline__ void fwd_scan_body(const ScanFwdArgs &p, int64_t b, int tile) {
+    if constexpr (KPL <= 4) {          // wider rows are spread over more than 16 lanes
+        if (p.kg == 16) {
+            fwd_scan_body_kg<IO, KPL, 16>(p, b, tile);
+            return;
+        }
+    }
+    fwd_scan_body_kg<IO, KPL, 0>(p, b, tile);
+}
+
 // ------------------------------------------------------------------------------------
 // backward, one side.  "rows" are the dimension this launch keeps per lane-group,
 // "cols" the dimension it reduces over:
@@ -122,12 +137,12 @@ __device__ __forceinline__ void fwd_scan_body(const ScanFwdArgs &p, int64_t b, i
 // ------------------------------------------------------------------------------------
 template <int KPL> struct SegLen { static constexpr int value = (32 / KPL) < 1 ? 1 : (KPL <= 4 ? 8 : 32 / KPL); };
 
-template <typename IO, int KPL, int SIDE>
-__device__ __forceinline__ void bwd_scan_body(const ScanBwdArgs &p, int64_t b, int tile) {
+template <typename IO, int KPL, int SIDE, int KG>
+__device__ __forceinline__ void bwd_scan_body_kg(const ScanBwdArgs &p, int64_t b, int tile) {
     using Acc = typename AccOf<IO>::type;
     constexpr int SEG = SegLen<KPL>::value;
     extern __shared__ __align__(16) unsigned char smem_raw[];
-    const Tile g(p.kg, KPL);
+    const Tile g(KG > 0 ? KG : p.kg, KPL);
     Acc *colL = reinterpret_cast<Acc *>(smem_raw);        // [SEG][3][KP]   a_c, gate_c, u_c
     Acc *rowL = colL + (size_t)SEG * 3 * g.KP;           // [SEG][3][rows] a_r, gate_r, u_r
     Acc *outL = rowL + (size_t)SEG * 3 * g.rows;         // [SEG][3][rows] d_a, d_gate, d_u
@@ -287,6 +302,17 @@ __device__ __forceinline__ void bwd_scan_body(const ScanBwdArgs &p, int64_t b, i
         for (int j = 0; j < KPL; ++j)
             if (el_ok(j)) ds[st_off(j)] = from_acc<IO>(G[j]);
     }
+}
+
+template <typename IO, int KPL, int SIDE>
+__device__ __forceinline__ void bwd_scan_body(const ScanBwdArgs &p, int64_t b, int tile) {
+    if constexpr (KPL <= 4) {
+        if (p.kg == 16) {
+            bwd_scan_body_kg<IO, KPL, SIDE, 16>(p, b, tile);
+            return;
+        }
+    }
+    bwd_scan_body_kg<IO, KPL, SIDE, 0>(p, b, tile);
 }
 
 }  // namespace scan
