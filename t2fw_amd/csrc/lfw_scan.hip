@@ -28,26 +28,26 @@ __global__ __launch_bounds__(SCAN_THREADS) void lfw_fwd_scan_kernel(ScanFwdArgs 
     fwd_scan_body<IO, KPL>(p, blockIdx.x / p.ntiles, (int)(blockIdx.x % p.ntiles));
 }
 
-// Normal mode: one workgroup per (batch row, tile).  Fix-up mode (row_select given): one
-// workgroup per batch row that walks the tiles itself, so that the launch, in which nearly all
-// workgroups leave at once, dispatches as few of them as possible.
+// The rows another kernel has flagged (row_select): one workgroup per batch row that walks the
+// tiles itself, so that the launch, in which nearly all workgroups leave at once, dispatches as
+// few of them as possible.  64 x 64 states only (16 lanes per state row, segment-start buffer).
 template <typename IO, int KPL, int SIDE> __device__ __forceinline__ void bwd_scan_rows(const ScanBwdArgs &p) {
-    if (p.row_select == nullptr) {
-        bwd_scan_body<IO, KPL, SIDE>(p, blockIdx.x / p.ntiles, (int)(blockIdx.x % p.ntiles));
-        return;
-    }
     const int64_t b = blockIdx.x;
     if (p.row_select[b] == 0) return;
     for (int tile = 0; tile < p.ntiles; ++tile) {
         if (tile) __syncthreads();
-        bwd_scan_body<IO, KPL, SIDE>(p, b, tile);
+        bwd_scan_body_kg<IO, KPL, SIDE, 16, 1>(p, b, tile);
     }
 }
 
-template <typename IO, int KPL, int SIDE>
+// One workgroup per (batch row, tile); a kernel per geometry (KG lanes per state row, 0 = any) and
+// per use of the segment-start buffer, so that each is register-allocated on its own: a spill
+// in the loop would wait for the prefetched global loads, which return in order with it.
+template <typename IO, int KPL, int SIDE, int KG, int SUB>
 __global__ __launch_bounds__(SCAN_THREADS) void lfw_bwd_scan_kernel(ScanBwdArgs p) {
-    bwd_scan_rows<IO, KPL, SIDE>(p);
+    bwd_scan_body_kg<IO, KPL, SIDE, KG, SUB>(p, blockIdx.x / p.ntiles, (int)(blockIdx.x % p.ntiles));
 }
+
 
 // Both sides in one launch (blockIdx.y = side) for square states, where the two sides share
 // their geometry.  Used when the kernel only redoes the rows another kernel has flagged:
@@ -90,13 +90,24 @@ int launch_bwd(ScanBwdArgs a, const ScanGeom &g, hipStream_t stream) {
     a.ntiles = (int)((nrows + g.rows - 1) / g.rows);
     const int64_t nblocks = a.row_select != nullptr ? a.B : a.B * a.ntiles;
     if (nblocks > 0x7fffffffLL) return fail(T2FW_ERR_UNSUPPORTED, "grid of %lld workgroups is too large", (long long)nblocks);
-    if (SIDE == 2) {
-        hipLaunchKernelGGL((lfw_bwd_scan_both_kernel<IO, KPL>), dim3((unsigned)nblocks, 2, 1), dim3(SCAN_THREADS), smem,
-                           stream, a);
-        return check_hip(hipGetLastError(), "lfw_bwd_scan_both_kernel launch");
+    if constexpr (SIDE == 2) {
+        // only the chunked kernels select rows: 64 x 64 states of 16-bit elements
+        if constexpr (KPL == 4 && sizeof(IO) == 2) {
+            if (g.kg != 16 || !a.use_sub) return fail(T2FW_ERR_UNSUPPORTED, "unexpected scan geometry for a 64 x 64 state");
+            hipLaunchKernelGGL((lfw_bwd_scan_both_kernel<IO, KPL>), dim3((unsigned)nblocks, 2, 1), dim3(SCAN_THREADS), smem,
+                               stream, a);
+            return check_hip(hipGetLastError(), "lfw_bwd_scan_both_kernel launch");
+        }
+        return fail(T2FW_ERR_UNSUPPORTED, "row selection takes 64 x 64 states of 16-bit elements");
+    } else {
+        dim3 grid((unsigned)nblocks, 1, 1);
+        if (KPL <= 4 && g.kg == 16 && a.use_sub)
+            hipLaunchKernelGGL((lfw_bwd_scan_kernel<IO, KPL, SIDE, (KPL <= 4 ? 16 : 0), 1>), grid, dim3(SCAN_THREADS), smem, stream, a);
+        else if (a.use_sub)
+            hipLaunchKernelGGL((lfw_bwd_scan_kernel<IO, KPL, SIDE, 0, 1>), grid, dim3(SCAN_THREADS), smem, stream, a);
+        else
+            hipLaunchKernelGGL((lfw_bwd_scan_kernel<IO, KPL, SIDE, 0, 0>), grid, dim3(SCAN_THREADS), smem, stream, a);
     }
-    dim3 grid((unsigned)nblocks, 1, 1);
-    hipLaunchKernelGGL((lfw_bwd_scan_kernel<IO, KPL, (SIDE == 2 ? 0 : SIDE)>), grid, dim3(SCAN_THREADS), smem, stream, a);
     return check_hip(hipGetLastError(), "lfw_bwd_scan_kernel launch");
 }
 
@@ -138,8 +149,11 @@ template <typename IO, int SIDE> int bwd_by_kpl(const ScanBwdArgs &a, hipStream_
 }
 
 template <typename IO> int bwd_both(const ScanBwdArgs &a, hipStream_t stream) {
-    // SIDE 2 = both sides in one launch (square states, fix-up mode only)
-    if (a.row_select != nullptr && a.D == a.K) return bwd_by_kpl<IO, 2>(a, stream);
+    // SIDE 2 = both sides in one launch (the rows another kernel has flagged)
+    if (a.row_select != nullptr) {
+        if (a.D != a.K) return fail(T2FW_ERR_UNSUPPORTED, "row selection takes square states");
+        return bwd_by_kpl<IO, 2>(a, stream);
+    }
     int rc = bwd_by_kpl<IO, 0>(a, stream);
     if (rc != T2FW_OK) return rc;
     return bwd_by_kpl<IO, 1>(a, stream);

@@ -137,7 +137,8 @@ __device__ __forceinline__ void fwd_scan_body(const ScanFwdArgs &p, int64_t b, i
 // ------------------------------------------------------------------------------------
 template <int KPL> struct SegLen { static constexpr int value = (32 / KPL) < 1 ? 1 : (KPL <= 4 ? 8 : 32 / KPL); };
 
-template <typename IO, int KPL, int SIDE, int KG>
+// KG as for the forward body; SUB: 1 / 0 = p.use_sub is known to be set / clear, -1 = read it.
+template <typename IO, int KPL, int SIDE, int KG, int SUB = -1>
 __device__ __forceinline__ void bwd_scan_body_kg(const ScanBwdArgs &p, int64_t b, int tile) {
     using Acc = typename AccOf<IO>::type;
     constexpr int SEG = SegLen<KPL>::value;
@@ -179,120 +180,143 @@ __device__ __forceinline__ void bwd_scan_body_kg(const ScanBwdArgs &p, int64_t b
     }
 
     const int C = p.C;
-    const bool use_sub = p.use_sub != 0;
+    const bool use_sub = SUB < 0 ? p.use_sub != 0 : SUB != 0;
     Prefetch<IO, 3, 3> pf;
 
-    for (int64_t c = p.NC - 1; c >= 0; --c) {
-        const int64_t tc0 = c * C;
-        const int len = (int)(T - tc0 < C ? T - tc0 : C);
-        const int nseg = (len + SEG - 1) / SEG;
+    auto load_ckpt = [&](Acc (&S)[KPL], int64_t c) {
         const IO *ck = ckpt + (b * p.NC + c) * DK;
-        Acc S[KPL];
 #pragma unroll
         for (int j = 0; j < KPL; ++j) S[j] = el_ok(j) ? to_acc(ck[st_off(j)]) : Acc(0);
-
-        // ---- forward sweep: states at segment starts -> subL (all but the last are advanced)
-        if (use_sub) {
-            for (int s = 0; s < nseg; ++s) {
+    };
+    // prefetched inputs -> LDS, between two barriers (the LDS of the step before is no longer read)
+    auto stage = [&]() {
+        __syncthreads();
+        block_store<IO, Acc, 3, 3, SEG>(pf, g, colL, rowL, SEG);
+        __syncthreads();
+    };
+    // S over the SEG staged steps
+    auto advance = [&](Acc (&S)[KPL]) {
 #pragma unroll
-                for (int j = 0; j < KPL; ++j) subL[((size_t)s * KPL + j) * SCAN_THREADS + threadIdx.x] = S[j];
-                if (s == nseg - 1) break;
-                const int64_t t0 = tc0 + (int64_t)s * SEG;
-                block_load(pf, g, colp, rowp, b, T, t0, SEG, ncols, nrows, row0, p.heads);
-                __syncthreads();
-                block_store<IO, Acc, 3, 3>(pf, g, colL, rowL, SEG);
-                __syncthreads();
+        for (int tt = 0; tt < SEG; ++tt) {
+            const Acc ar = rowL[(tt * 3 + 0) * g.rows + g.r];
+            const Acc fr = rowL[(tt * 3 + 1) * g.rows + g.r];
+            const Acc *ca = colL + (tt * 3 + 0) * g.KP + g.k0;
+            const Acc *cf = colL + (tt * 3 + 1) * g.KP + g.k0;
 #pragma unroll
-                for (int tt = 0; tt < SEG; ++tt) {
-                    const Acc ar = rowL[(tt * 3 + 0) * g.rows + g.r];
-                    const Acc fr = rowL[(tt * 3 + 1) * g.rows + g.r];
-                    const Acc *ca = colL + (tt * 3 + 0) * g.KP + g.k0;
-                    const Acc *cf = colL + (tt * 3 + 1) * g.KP + g.k0;
+            for (int j = 0; j < KPL; ++j) S[j] = S[j] * (fr * cf[j]) + ar * ca[j];
+        }
+    };
+    // The staged segment [t0, t0 + n): its states recomputed into registers from st[0], the adjoint
+    // backwards over them, the outputs written.
+    auto reverse_segment = [&](Acc (&st)[SEG + 1][KPL], int n, int64_t t0) {
 #pragma unroll
-                    for (int j = 0; j < KPL; ++j) S[j] = S[j] * (fr * cf[j]) + ar * ca[j];
+        for (int tt = 0; tt < SEG; ++tt) {
+            const Acc ar = rowL[(tt * 3 + 0) * g.rows + g.r];
+            const Acc fr = rowL[(tt * 3 + 1) * g.rows + g.r];
+            const Acc *ca = colL + (tt * 3 + 0) * g.KP + g.k0;
+            const Acc *cf = colL + (tt * 3 + 1) * g.KP + g.k0;
+#pragma unroll
+            for (int j = 0; j < KPL; ++j) st[tt + 1][j] = st[tt][j] * (fr * cf[j]) + ar * ca[j];
+        }
+        // adjoint, last step of the segment first
+#pragma unroll
+        for (int tt = SEG - 1; tt >= 0; --tt) {
+            if (tt < n) {
+                const Acc fr = rowL[(tt * 3 + 1) * g.rows + g.r];
+                const Acc ur = rowL[(tt * 3 + 2) * g.rows + g.r];
+                const Acc *ca = colL + (tt * 3 + 0) * g.KP + g.k0;
+                const Acc *cf = colL + (tt * 3 + 1) * g.KP + g.k0;
+                const Acc *cu = colL + (tt * 3 + 2) * g.KP + g.k0;
+                Acc sa = 0, sg = 0, su = 0;
+#pragma unroll
+                for (int j = 0; j < KPL; ++j) {
+                    G[j] += ur * cu[j];                       // G_t = g_t (x) q_t + ...
+                    sa += G[j] * ca[j];                       // d_x / d_k
+                    sg += (G[j] * st[tt][j]) * cf[j];         // d_f / d_f_key   (uses S_{t-1})
+                    if (SIDE == 1) su += st[tt + 1][j] * cu[j];   // d_q = S_t^T g_t
+                    G[j] *= fr * cf[j];
+                }
+                sa = group_sum(sa, g.kg);
+                sg = group_sum(sg, g.kg);
+                if (SIDE == 1) su = group_sum(su, g.kg);
+                if (g.kgi == 0) {
+                    outL[(tt * 3 + 0) * g.rows + g.r] = sa;
+                    outL[(tt * 3 + 1) * g.rows + g.r] = sg;
+                    if (SIDE == 1) outL[(tt * 3 + 2) * g.rows + g.r] = su;
                 }
             }
         }
+        __syncthreads();
+        for (int idx = threadIdx.x; idx < n * g.rows; idx += SCAN_THREADS) {
+            const int tt = idx / g.rows, rr = idx % g.rows;
+            if (row0 + rr < nrows) {
+                const int64_t o = (line0 + (t0 + tt) * p.heads) * nrows + row0 + rr;
+                d_a[o] = from_acc<IO>(outL[(tt * 3 + 0) * g.rows + rr]);
+                d_gate[o] = from_acc<IO>(outL[(tt * 3 + 1) * g.rows + rr]);
+                if (SIDE == 1) d_u[o] = from_acc<IO>(outL[(tt * 3 + 2) * g.rows + rr]);
+            }
+        }
+    };
+    auto chunk_len = [&](int64_t c) -> int { return (int)(T - c * C < C ? T - c * C : C); };
 
-        // ---- reverse over segments
-        for (int s = nseg - 1; s >= 0; --s) {
-            const int64_t t0 = tc0 + (int64_t)s * SEG;
-            const int n = (int)(len - s * SEG < SEG ? len - s * SEG : SEG);
-            Acc st[SEG + 1][KPL];
-            if (use_sub) {
+    if (use_sub) {
+        // A chunk with nseg segments is 2 * nseg - 1 staged jobs: nseg - 1 that advance S to the
+        // segment starts (kept in subL), then the segments last to first.  The global loads of a
+        // job are issued while the job before it computes.
+        auto issue = [&](int64_t c, int q) {
+            const int len = chunk_len(c), nseg = (len + SEG - 1) / SEG;
+            const int sg = q < nseg - 1 ? q : 2 * nseg - 2 - q;
+            const int n = q < nseg - 1 ? SEG : (len - sg * SEG < SEG ? len - sg * SEG : SEG);
+            block_load<SEG>(pf, g, colp, rowp, b, T, c * C + (int64_t)sg * SEG, n, ncols, nrows, row0, p.heads);
+        };
+        Acc Snext[KPL];                      // checkpoint of the chunk that comes next
+        load_ckpt(Snext, p.NC - 1);
+        issue(p.NC - 1, 0);
+        for (int64_t c = p.NC - 1; c >= 0; --c) {
+            const int64_t tc0 = c * C;
+            const int len = chunk_len(c), nseg = (len + SEG - 1) / SEG, njobs = 2 * nseg - 1;
+            Acc S[KPL];
 #pragma unroll
-                for (int j = 0; j < KPL; ++j) st[0][j] = subL[((size_t)s * KPL + j) * SCAN_THREADS + threadIdx.x];
-            } else {
-                // no room for segment-start states: replay from the checkpoint
+            for (int j = 0; j < KPL; ++j) S[j] = Snext[j];
+            if (c > 0) load_ckpt(Snext, c - 1);
 #pragma unroll
-                for (int j = 0; j < KPL; ++j) st[0][j] = el_ok(j) ? to_acc(ck[st_off(j)]) : Acc(0);
+            for (int j = 0; j < KPL; ++j) subL[(size_t)j * SCAN_THREADS + threadIdx.x] = S[j];
+            for (int q = 0; q < njobs; ++q) {
+                stage();
+                if (q + 1 < njobs)
+                    issue(c, q + 1);
+                else if (c > 0)
+                    issue(c - 1, 0);
+                if (q < nseg - 1) {
+                    advance(S);
+#pragma unroll
+                    for (int j = 0; j < KPL; ++j) subL[((size_t)(q + 1) * KPL + j) * SCAN_THREADS + threadIdx.x] = S[j];
+                } else {
+                    const int sg = 2 * nseg - 2 - q;
+                    Acc st[SEG + 1][KPL];
+#pragma unroll
+                    for (int j = 0; j < KPL; ++j) st[0][j] = subL[((size_t)sg * KPL + j) * SCAN_THREADS + threadIdx.x];
+                    reverse_segment(st, len - sg * SEG < SEG ? len - sg * SEG : SEG, tc0 + (int64_t)sg * SEG);
+                }
+            }
+        }
+    } else {
+        // no room for the segment-start states: every segment is replayed from the checkpoint
+        for (int64_t c = p.NC - 1; c >= 0; --c) {
+            const int64_t tc0 = c * C;
+            const int len = chunk_len(c), nseg = (len + SEG - 1) / SEG;
+            for (int s = nseg - 1; s >= 0; --s) {
+                Acc st[SEG + 1][KPL];
+                load_ckpt(st[0], c);
                 for (int s2 = 0; s2 < s; ++s2) {
-                    block_load(pf, g, colp, rowp, b, T, tc0 + (int64_t)s2 * SEG, SEG, ncols, nrows, row0, p.heads);
-                    __syncthreads();
-                    block_store<IO, Acc, 3, 3>(pf, g, colL, rowL, SEG);
-                    __syncthreads();
-#pragma unroll
-                    for (int tt = 0; tt < SEG; ++tt) {
-                        const Acc ar = rowL[(tt * 3 + 0) * g.rows + g.r];
-                        const Acc fr = rowL[(tt * 3 + 1) * g.rows + g.r];
-                        const Acc *ca = colL + (tt * 3 + 0) * g.KP + g.k0;
-                        const Acc *cf = colL + (tt * 3 + 1) * g.KP + g.k0;
-#pragma unroll
-                        for (int j = 0; j < KPL; ++j) st[0][j] = st[0][j] * (fr * cf[j]) + ar * ca[j];
-                    }
+                    block_load<SEG>(pf, g, colp, rowp, b, T, tc0 + (int64_t)s2 * SEG, SEG, ncols, nrows, row0, p.heads);
+                    stage();
+                    advance(st[0]);
                 }
-            }
-            block_load(pf, g, colp, rowp, b, T, t0, n, ncols, nrows, row0, p.heads);
-            __syncthreads();
-            block_store<IO, Acc, 3, 3>(pf, g, colL, rowL, SEG);
-            __syncthreads();
-            // recompute the segment's states into registers
-#pragma unroll
-            for (int tt = 0; tt < SEG; ++tt) {
-                const Acc ar = rowL[(tt * 3 + 0) * g.rows + g.r];
-                const Acc fr = rowL[(tt * 3 + 1) * g.rows + g.r];
-                const Acc *ca = colL + (tt * 3 + 0) * g.KP + g.k0;
-                const Acc *cf = colL + (tt * 3 + 1) * g.KP + g.k0;
-#pragma unroll
-                for (int j = 0; j < KPL; ++j) st[tt + 1][j] = st[tt][j] * (fr * cf[j]) + ar * ca[j];
-            }
-            // adjoint, last step of the segment first
-#pragma unroll
-            for (int tt = SEG - 1; tt >= 0; --tt) {
-                if (tt < n) {
-                    const Acc fr = rowL[(tt * 3 + 1) * g.rows + g.r];
-                    const Acc ur = rowL[(tt * 3 + 2) * g.rows + g.r];
-                    const Acc *ca = colL + (tt * 3 + 0) * g.KP + g.k0;
-                    const Acc *cf = colL + (tt * 3 + 1) * g.KP + g.k0;
-                    const Acc *cu = colL + (tt * 3 + 2) * g.KP + g.k0;
-                    Acc sa = 0, sg = 0, su = 0;
-#pragma unroll
-                    for (int j = 0; j < KPL; ++j) {
-                        G[j] += ur * cu[j];                       // G_t = g_t (x) q_t + ...
-                        sa += G[j] * ca[j];                       // d_x / d_k
-                        sg += (G[j] * st[tt][j]) * cf[j];         // d_f / d_f_key   (uses S_{t-1})
-                        if (SIDE == 1) su += st[tt + 1][j] * cu[j];   // d_q = S_t^T g_t
-                        G[j] *= fr * cf[j];
-                    }
-                    sa = group_sum(sa, g.kg);
-                    sg = group_sum(sg, g.kg);
-                    if (SIDE == 1) su = group_sum(su, g.kg);
-                    if (g.kgi == 0) {
-                        outL[(tt * 3 + 0) * g.rows + g.r] = sa;
-                        outL[(tt * 3 + 1) * g.rows + g.r] = sg;
-                        if (SIDE == 1) outL[(tt * 3 + 2) * g.rows + g.r] = su;
-                    }
-                }
-            }
-            __syncthreads();
-            for (int idx = threadIdx.x; idx < n * g.rows; idx += SCAN_THREADS) {
-                const int tt = idx / g.rows, rr = idx % g.rows;
-                if (row0 + rr < nrows) {
-                    const int64_t o = (line0 + (t0 + tt) * p.heads) * nrows + row0 + rr;
-                    d_a[o] = from_acc<IO>(outL[(tt * 3 + 0) * g.rows + rr]);
-                    d_gate[o] = from_acc<IO>(outL[(tt * 3 + 1) * g.rows + rr]);
-                    if (SIDE == 1) d_u[o] = from_acc<IO>(outL[(tt * 3 + 2) * g.rows + rr]);
-                }
+                const int n = len - s * SEG < SEG ? len - s * SEG : SEG;
+                block_load<SEG>(pf, g, colp, rowp, b, T, tc0 + (int64_t)s * SEG, n, ncols, nrows, row0, p.heads);
+                stage();
+                reverse_segment(st, n, tc0 + (int64_t)s * SEG);
             }
         }
     }
@@ -302,17 +326,6 @@ __device__ __forceinline__ void bwd_scan_body_kg(const ScanBwdArgs &p, int64_t b
         for (int j = 0; j < KPL; ++j)
             if (el_ok(j)) ds[st_off(j)] = from_acc<IO>(G[j]);
     }
-}
-
-template <typename IO, int KPL, int SIDE>
-__device__ __forceinline__ void bwd_scan_body(const ScanBwdArgs &p, int64_t b, int tile) {
-    if constexpr (KPL <= 4) {
-        if (p.kg == 16) {
-            bwd_scan_body_kg<IO, KPL, SIDE, 16>(p, b, tile);
-            return;
-        }
-    }
-    bwd_scan_body_kg<IO, KPL, SIDE, 0>(p, b, tile);
 }
 
 }  // namespace scan

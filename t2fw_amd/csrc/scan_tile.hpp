@@ -42,7 +42,9 @@ template <typename IO, int NCA, int NRA> struct Prefetch {
 // colp[a] are [B,T,ncols] arrays, rowp[a] are [B,T,nrows] arrays (heads = 1), or
 // [B/heads,T,heads,ncols] and [B/heads,T,heads,nrows] with row b = (batch, head); this
 // workgroup needs all columns and rows [row0, row0 + rows).
-template <typename IO, int NCA, int NRA>
+// TMAX: an upper bound of n known at compile time; slots that can only hold later steps are
+// skipped (which removes their loads when the geometry is a compile-time constant too).
+template <int TMAX = 1 << 30, typename IO, int NCA, int NRA>
 __device__ __forceinline__ void block_load(Prefetch<IO, NCA, NRA> &pf, const Tile &g,
                                            const IO *const (&colp)[NCA],
                                            const IO *const (&rowp)[NRA],
@@ -54,6 +56,7 @@ __device__ __forceinline__ void block_load(Prefetch<IO, NCA, NRA> &pf, const Til
     const int64_t cbase = line0 * ncols;
 #pragma unroll
     for (int m = 0; m < PFC; ++m) {
+        if (g.SP * (m >> g.lncc) >= TMAX) continue;
         const int tt = tsub + g.SP * (m >> g.lncc);
         const int c = csub + g.CW * (m & ((1 << g.lncc) - 1));
         const bool ok = tt < n && c < ncols;
@@ -65,6 +68,7 @@ __device__ __forceinline__ void block_load(Prefetch<IO, NCA, NRA> &pf, const Til
     const int64_t rbase = line0 * nrows + row0;
 #pragma unroll
     for (int m = 0; m < PFR; ++m) {
+        if (g.SPR * m >= TMAX) continue;
         const int tt = tsr + g.SPR * m;
         const bool ok = tt < n && row0 + rsub < nrows;
 #pragma unroll
@@ -74,12 +78,13 @@ __device__ __forceinline__ void block_load(Prefetch<IO, NCA, NRA> &pf, const Til
 }
 
 // Write the prefetched block into LDS: colL[(tt*NCA + a)*KP + c], rowL[(tt*NRA + a)*rows + r]
-template <typename IO, typename Acc, int NCA, int NRA>
+template <typename IO, typename Acc, int NCA, int NRA, int TMAX = 1 << 30>
 __device__ __forceinline__ void block_store(const Prefetch<IO, NCA, NRA> &pf, const Tile &g,
                                             Acc *colL, Acc *rowL, int tb) {
     const int csub = threadIdx.x % g.CW, tsub = threadIdx.x / g.CW;
 #pragma unroll
     for (int m = 0; m < PFC; ++m) {
+        if (g.SP * (m >> g.lncc) >= TMAX) continue;
         const int tt = tsub + g.SP * (m >> g.lncc);
         const int c = csub + g.CW * (m & ((1 << g.lncc) - 1));
         if (tt < tb) {
@@ -90,6 +95,7 @@ __device__ __forceinline__ void block_store(const Prefetch<IO, NCA, NRA> &pf, co
     const int rsub = threadIdx.x % g.rows, tsr = threadIdx.x / g.rows;
 #pragma unroll
     for (int m = 0; m < PFR; ++m) {
+        if (g.SPR * m >= TMAX) continue;
         const int tt = tsr + g.SPR * m;
         if (tt < tb) {
 #pragma unroll
