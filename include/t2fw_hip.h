@@ -106,6 +106,24 @@ int t2fw_lfw_forward(const void *x, const void *f, const void *q, const void *k,
                      void *workspace, size_t workspace_bytes, void *stream);
 
 /*
+ * The forward scan for callers that cannot allocate device memory or pass a workspace: code
+ * under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  It has no
+ * counterpart in the reference (whose launcher allocates on every call, lfw_kernel.cu:140).
+ * Same arguments and results as t2fw_lfw_forward, minus the workspace: the scratch lives in a
+ * buffer of T2FW_STATIC_SCRATCH_BYTES bytes built into the library (one copy per GPU, held until
+ * the process ends).  The call allocates and frees nothing.  A shape whose scratch
+ * (t2fw_lfw_workspace_bytes) exceeds the buffer is rejected with T2FW_ERR_WORKSPACE.  All calls
+ * on one GPU share the buffer: calls that overlap in time on one GPU (different streams or
+ * threads) race on it; calls on one stream do not.
+ */
+#define T2FW_STATIC_SCRATCH_BYTES (1 << 20)
+int t2fw_lfw_forward_static(const void *x, const void *f, const void *q, const void *k,
+                            const void *f_key, const void *s0,
+                            void *out, void *next_state, void *ckpt,
+                            int64_t B, int64_t T, int64_t D, int64_t K,
+                            int32_t C, int32_t dtype, int32_t flags, void *stream);
+
+/*
  * Backward pass: recomputes the states inside each chunk from ckpt, runs the
  * reverse-time adjoint scan and writes all six gradients.  Replaces lfw_backward
  * (lfw.cpp:50-96); gradient order as returned there (lfw.cpp:95).

@@ -31,6 +31,7 @@ SIGNATURES = {
     "t2fw_lfw_num_ckpt": (_i64, [_i64, _i32]),
     "t2fw_lfw_workspace_bytes": (_sz, [_i64, _i64, _i64, _i64, _i32, _i32, _i32]),
     "t2fw_lfw_forward": (ctypes.c_int, [_vp] * 9 + [_i64] * 4 + [_i32] * 3 + [_vp, _sz, _vp]),
+    "t2fw_lfw_forward_static": (ctypes.c_int, [_vp] * 9 + [_i64] * 4 + [_i32] * 3 + [_vp]),
     "t2fw_lfw_backward": (ctypes.c_int, [_vp] * 15 + [_i64] * 4 + [_i32] * 3 + [_vp, _sz, _vp]),
     "t2fw_lfw_forward_heads": (ctypes.c_int, [_vp] * 9 + [_i64] * 5 + [_i32] * 3 + [_vp, _sz, _vp]),
     "t2fw_lfw_backward_heads": (ctypes.c_int, [_vp] * 15 + [_i64] * 5 + [_i32] * 3 + [_vp, _sz, _vp]),

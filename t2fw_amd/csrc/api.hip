@@ -9,6 +9,7 @@
 
 #include <cstring>
 #include <initializer_list>
+#include <mutex>
 
 namespace t2fw {
 
@@ -90,6 +91,37 @@ int check_dims(int64_t B, int64_t T, int64_t D, int64_t K) {
 }  // namespace t2fw
 
 using namespace t2fw;
+
+// ---- forward scan for callers that cannot allocate -------------------------------------------
+// The scratch of t2fw_lfw_forward (the row flags of the matrix-core kernels) lives in a file-scope
+// device array instead of a caller's workspace.  Every GPU holds its own copy of the array at its
+// own address; the array's name is only a host-side handle, so the address is looked up once per
+// device with hipGetSymbolAddress and only that pointer is ever handed to a kernel.
+static __device__ __align__(256) unsigned char scratch[T2FW_STATIC_SCRATCH_BYTES];
+
+namespace {
+constexpr int MAX_DEVICES = 64;
+std::mutex g_scratch_mutex;
+void *g_scratch_ptr[MAX_DEVICES] = {};
+
+// device address of `scratch` on the current device (looked up on the first call per device)
+int static_scratch(void **out) {
+    int dev = -1;
+    int rc = check_hip(hipGetDevice(&dev), "hipGetDevice");
+    if (rc) return rc;
+    if (dev < 0 || dev >= MAX_DEVICES) return fail(T2FW_ERR_UNSUPPORTED, "device ordinal %d is out of range", dev);
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (g_scratch_ptr[dev] == nullptr) {
+        void *ptr = nullptr;
+        rc = check_hip(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)), "hipGetSymbolAddress(scratch)");
+        if (rc) return rc;
+        if (ptr == nullptr) return fail(T2FW_ERR_HIP, "hipGetSymbolAddress returned a null address");
+        g_scratch_ptr[dev] = ptr;
+    }
+    *out = g_scratch_ptr[dev];
+    return T2FW_OK;
+}
+}  // namespace
 
 extern "C" {
 
@@ -183,6 +215,24 @@ int t2fw_lfw_forward(const void *x, const void *f, const void *q, const void *k,
                      size_t workspace_bytes, void *stream) {
     return lfw_forward_rows(x, f, q, k, f_key, s0, out, next_state, ckpt, B, T, 1, D, K, C, dtype, flags, workspace,
                             workspace_bytes, stream);
+}
+
+int t2fw_lfw_forward_static(const void *x, const void *f, const void *q, const void *k, const void *f_key,
+                            const void *s0, void *out, void *next_state, void *ckpt, int64_t B, int64_t T,
+                            int64_t D, int64_t K, int32_t C, int32_t dtype, int32_t flags, void *stream) {
+    const size_t need = t2fw_lfw_workspace_bytes(B, T, D, K, C, dtype, flags);
+    if (need > (size_t)T2FW_STATIC_SCRATCH_BYTES)
+        return fail(T2FW_ERR_WORKSPACE,
+                    "t2fw_lfw_forward_static: this shape needs %zu bytes of scratch, the built-in buffer holds %d "
+                    "(use t2fw_lfw_forward with a workspace)", need, T2FW_STATIC_SCRATCH_BYTES);
+    void *ws = nullptr;
+    if (need > 0) {
+        const int rc = static_scratch(&ws);
+        if (rc) return rc;
+    }
+    // the kernels clear the flags of the rows they work on themselves, so what an earlier call left
+    // in the buffer does not matter
+    return lfw_forward_rows(x, f, q, k, f_key, s0, out, next_state, ckpt, B, T, 1, D, K, C, dtype, flags, ws, need, stream);
 }
 
 int t2fw_lfw_forward_heads(const void *x, const void *f, const void *q, const void *k, const void *f_key,
