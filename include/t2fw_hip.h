@@ -50,7 +50,7 @@
 extern "C" {
 #endif
 
-#define T2FW_ABI_VERSION 1
+#define T2FW_ABI_VERSION 2
 
 /* dtype codes (reference dispatch: AT_DISPATCH_FLOATING_TYPES_AND_HALF,
  * lfw_kernel.cu:157 -> fp64/fp32/fp16; bf16 is added here) */
@@ -83,15 +83,23 @@ extern "C" {
                                      those rows with T2FW_FLAG_FORCE_SCAN, or knows its gates are
                                      in range.  Saves the backward's extra launch.              */
 
+#define T2FW_FLAG_BLOCKWISE 8     /* matrix-core path: the block-wise kernels (16-step blocks, one or two
+                                     workgroups per batch row) instead of the chunk-parallel ones    */
+
 int t2fw_abi_version(void);
 const char *t2fw_last_error(void);
 
 /* Number of checkpoints per batch row: ceil(T / C), at least 1. */
 int64_t t2fw_lfw_num_ckpt(int64_t T, int32_t C);
 
-/* Bytes of caller-provided scratch the forward / backward calls need (0 = none). */
+/* Bytes of caller-provided scratch that serve both the forward and the backward call of a
+ * shape (0 = none): row flags, and for the chunk-parallel backward kernels the adjoint entering
+ * every chunk, [B, NC, D, K] bf16. */
 size_t t2fw_lfw_workspace_bytes(int64_t B, int64_t T, int64_t D, int64_t K,
                                 int32_t C, int32_t dtype, int32_t flags);
+/* The same for a caller that only runs the forward call. */
+size_t t2fw_lfw_forward_workspace_bytes(int64_t B, int64_t T, int64_t D, int64_t K,
+                                        int32_t C, int32_t dtype, int32_t flags);
 
 /*
  * Forward scan.  S_t = S_{t-1} * (f_t (x) f_key_t) + x_t (x) k_t ;  out_t = S_t q_t ;

@@ -3,6 +3,7 @@
 #include "common.hpp"
 #include "lfw_scan.hpp"
 #include "lfw_chunk.hpp"
+#include "lfw_par.hpp"
 #include "dfw_scan.hpp"
 #include "gate.hpp"
 #include "lfw_step.hpp"
@@ -75,8 +76,43 @@ int compute_units() {
     return n;
 }
 
-// two flag slots per batch row (kernels that split a row over two workgroups use both)
+// Workspace of the matrix-core kernels:
+//   [0, row_flag_bytes)                 flags of the block-wise kernels, two slots per batch row (kernels
+//                                       that split a row over two workgroups use both)
+//   [row_flag_bytes, 2 * row_flag_bytes)  flags of the chunk-parallel kernels, one slot per row
+//   then, backward only (ParScratch): per-chunk flags [B * NC] int32, per-chunk gate products
+//   [B, NC, PAR_NVEC, 64] fp32, adjoint entering every chunk [B, NC, 64, 64] bf16
 size_t row_flag_bytes(int64_t B) { return (size_t)((2 * chunk_rows_padded(B) * 4 + 255) / 256 * 256); }
+
+// The chunk-parallel kernels take checkpoint intervals 32 and 64 and bf16 matrix-core operands.
+bool par_ok(int32_t C, int32_t flags) {
+    return (C == 32 || C == 64) && (flags & (T2FW_FLAG_BLOCKWISE | T2FW_FLAG_FP16_OPERANDS)) == 0;
+}
+
+struct ParScratch {
+    size_t chunk_flags, vecs, gh, total;       // byte offsets from the start of the workspace
+};
+ParScratch par_scratch(int64_t B, int64_t T, int32_t C) {
+    const int64_t nc = (C < 1 || T <= 0) ? 1 : (T + C - 1) / C;
+    const size_t items = (size_t)(B * nc);
+    ParScratch s;
+    s.chunk_flags = 2 * row_flag_bytes(B);
+    s.vecs = s.chunk_flags + (items * 4 + 255) / 256 * 256;
+    s.gh = s.vecs + items * (size_t)(PAR_NVEC * CH_N * 4);
+    s.total = s.gh + items * (size_t)(CH_N * CH_N * 2);
+    return s;
+}
+
+size_t forward_workspace_bytes(int64_t B, int64_t D, int64_t K, int32_t dtype, int32_t flags) {
+    if (B > 0 && chunk_shape_ok(D, K, dtype, flags)) return 2 * row_flag_bytes(B);
+    return 0;
+}
+
+size_t backward_workspace_bytes(int64_t B, int64_t T, int64_t D, int64_t K, int32_t C, int32_t dtype, int32_t flags) {
+    if (B > 0 && chunk_shape_ok(D, K, dtype, flags))
+        return par_ok(C, flags) ? par_scratch(B, T, C).total : 2 * row_flag_bytes(B);
+    return 0;
+}
 
 int check_dims(int64_t B, int64_t T, int64_t D, int64_t K) {
     if (B < 0 || T < 0) return fail(T2FW_ERR_BAD_SHAPE, "B=%lld and T=%lld must be non-negative", (long long)B, (long long)T);
@@ -123,6 +159,11 @@ int static_scratch(void **out) {
 }
 }  // namespace
 
+#ifdef T2FW_PAR_TIMERS
+static unsigned long long *g_dbg = nullptr;
+extern "C" void t2fw_debug_set_buffer(void *p) { g_dbg = static_cast<unsigned long long *>(p); }
+#endif
+
 extern "C" {
 
 int t2fw_abi_version(void) { return T2FW_ABI_VERSION; }
@@ -136,9 +177,15 @@ int64_t t2fw_lfw_num_ckpt(int64_t T, int32_t C) {
 
 size_t t2fw_lfw_workspace_bytes(int64_t B, int64_t T, int64_t D, int64_t K, int32_t C, int32_t dtype,
                                 int32_t flags) {
+    const size_t fwd = forward_workspace_bytes(B, D, K, dtype, flags);
+    const size_t bwd = backward_workspace_bytes(B, T, D, K, C, dtype, flags);
+    return fwd > bwd ? fwd : bwd;
+}
+
+size_t t2fw_lfw_forward_workspace_bytes(int64_t B, int64_t T, int64_t D, int64_t K, int32_t C, int32_t dtype,
+                                        int32_t flags) {
     (void)T; (void)C;
-    if (B > 0 && chunk_shape_ok(D, K, dtype, flags)) return row_flag_bytes(B);
-    return 0;
+    return forward_workspace_bytes(B, D, K, dtype, flags);
 }
 
 // B batch rows; heads = 1: rows are contiguous [T, D|K] slabs, heads = H > 1: row b is head b % H of
@@ -183,9 +230,9 @@ static int lfw_forward_rows(const void *x, const void *f, const void *q, const v
 
     if (chunk_shape_ok(D, K, dtype, flags) && (ckpt == nullptr || C % 32 == 0) && T * heads < CHUNK_MAX_T &&
         aligned16({x, f, q, k, f_key, s0, out, next_state, ckpt})) {
-        if (workspace == nullptr || workspace_bytes < row_flag_bytes(B))
-            return fail(T2FW_ERR_WORKSPACE, "workspace of %zu bytes needed, %zu given", row_flag_bytes(B),
-                        workspace_bytes);
+        const size_t need = forward_workspace_bytes(B, D, K, dtype, flags);
+        if (workspace == nullptr || workspace_bytes < need)
+            return fail(T2FW_ERR_WORKSPACE, "workspace of %zu bytes needed, %zu given", need, workspace_bytes);
         ChunkFwdArgs c{};
         c.x = x; c.f = f; c.q = q; c.k = k; c.f_key = f_key; c.s0 = s0;
         c.out = out; c.next_state = next_state; c.ckpt = ckpt;
@@ -220,7 +267,7 @@ int t2fw_lfw_forward(const void *x, const void *f, const void *q, const void *k,
 int t2fw_lfw_forward_static(const void *x, const void *f, const void *q, const void *k, const void *f_key,
                             const void *s0, void *out, void *next_state, void *ckpt, int64_t B, int64_t T,
                             int64_t D, int64_t K, int32_t C, int32_t dtype, int32_t flags, void *stream) {
-    const size_t need = t2fw_lfw_workspace_bytes(B, T, D, K, C, dtype, flags);
+    const size_t need = t2fw_lfw_forward_workspace_bytes(B, T, D, K, C, dtype, flags);
     if (need > (size_t)T2FW_STATIC_SCRATCH_BYTES)
         return fail(T2FW_ERR_WORKSPACE,
                     "t2fw_lfw_forward_static: this shape needs %zu bytes of scratch, the built-in buffer holds %d "
@@ -282,15 +329,37 @@ static int lfw_backward_rows(const void *g_out, const void *g_state, const void 
 
     if (chunk_shape_ok(D, K, dtype, flags) && (C == 32 || C == 64) && T * heads < CHUNK_MAX_T &&
         aligned16({g_out, g_state, x, f, q, k, f_key, ckpt, d_x, d_f, d_q, d_k, d_f_key, d_s0})) {
-        if (workspace == nullptr || workspace_bytes < row_flag_bytes(B))
-            return fail(T2FW_ERR_WORKSPACE, "workspace of %zu bytes needed, %zu given", row_flag_bytes(B),
-                        workspace_bytes);
+        const size_t need = backward_workspace_bytes(B, T, D, K, C, dtype, flags);
+        if (workspace == nullptr || workspace_bytes < need)
+            return fail(T2FW_ERR_WORKSPACE, "workspace of %zu bytes needed, %zu given", need, workspace_bytes);
         ChunkBwdArgs c{};
         c.g_out = g_out; c.g_state = g_state; c.x = x; c.f = f; c.q = q; c.k = k; c.f_key = f_key; c.ckpt = ckpt;
         c.d_x = d_x; c.d_f = d_f; c.d_q = d_q; c.d_k = d_k; c.d_f_key = d_f_key; c.d_s0 = d_s0;
         c.row_flags = static_cast<int32_t *>(workspace);
+        c.row_select = nullptr;
         c.B = B; c.T = T; c.NC = a.NC; c.C = C;
         c.heads = (int32_t)heads;
+        if (par_ok(C, flags)) {
+            // chunk-parallel kernels; the rows they flag are redone with the exact scan
+            ParBwdArgs pa{};
+            pa.g_out = g_out; pa.g_state = g_state; pa.x = x; pa.f = f; pa.q = q; pa.k = k; pa.f_key = f_key; pa.ckpt = ckpt;
+            pa.d_x = d_x; pa.d_f = d_f; pa.d_q = d_q; pa.d_k = d_k; pa.d_f_key = d_f_key; pa.d_s0 = d_s0;
+            unsigned char *const ws = static_cast<unsigned char *>(workspace);
+            const ParScratch sc = par_scratch(B, T, C);
+            pa.row_flags = reinterpret_cast<int32_t *>(ws + row_flag_bytes(B));
+            pa.chunk_flags = reinterpret_cast<int32_t *>(ws + sc.chunk_flags);
+            pa.vecs = reinterpret_cast<float *>(ws + sc.vecs);
+            pa.gh = ws + sc.gh;
+            pa.B = B; pa.T = T; pa.NC = a.NC; pa.C = C;
+            pa.heads = (int32_t)heads;
+#ifdef T2FW_PAR_TIMERS
+            pa.dbg = g_dbg;
+#endif
+            if ((rc = par_backward(pa, dtype, st))) return rc;
+            if (flags & T2FW_FLAG_NO_FIXUP) return T2FW_OK;
+            a.row_select = pa.row_flags;
+            return scan_backward(a, dtype, st);
+        }
         const int op = (dtype == T2FW_F16 && (flags & T2FW_FLAG_FP16_OPERANDS)) ? 1 : 0;
         if ((rc = chunk_backward(c, dtype, op, st))) return rc;
         a.row_select = c.row_flags;      // rows the chunked form could not take

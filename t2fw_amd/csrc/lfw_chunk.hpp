@@ -42,6 +42,7 @@ struct ChunkBwdArgs {
     const void *g_out, *g_state, *x, *f, *q, *k, *f_key, *ckpt;
     void *d_x, *d_f, *d_q, *d_k, *d_f_key, *d_s0;
     int32_t *row_flags;                // as for the forward
+    const int32_t *row_select;         // null: every row; else only rows b with row_select[b] != 0 (the others report "not flagged")
     int64_t B, T, NC;
     int32_t C;
     int32_t heads;                     // as for the forward (inputs, g_out and the five [.., T, .., 64] gradients)

@@ -773,6 +773,13 @@ __global__ __launch_bounds__(BW_THREADS) void lfw_bwd_chunk_kernel(ChunkBwdArgs 
     const int side = (int)blockIdx.x >= rows_padded ? 1 : 0;
     const int64_t b = (int)blockIdx.x - side * rows_padded;
     if (b >= p.B) return;
+    if (p.row_select != nullptr && p.row_select[b] == 0) {      // not this kernel's row: nothing to redo after it either
+        if (tid == 0) {
+            p.row_flags[b] = 0;
+            p.row_flags[rows_padded + b] = 0;
+        }
+        return;
+    }
     // both branches execute one workgroup barrier per stage
     if (tid < 256) {
         if (side == 0)

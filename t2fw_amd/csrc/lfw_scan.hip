@@ -28,15 +28,20 @@ __global__ __launch_bounds__(SCAN_THREADS) void lfw_fwd_scan_kernel(ScanFwdArgs 
     fwd_scan_body<IO, KPL>(p, blockIdx.x / p.ntiles, (int)(blockIdx.x % p.ntiles));
 }
 
-// The rows another kernel has flagged (row_select): one workgroup per batch row that walks the
-// tiles itself, so that the launch, in which nearly all workgroups leave at once, dispatches as
-// few of them as possible.  64 x 64 states only (16 lanes per state row, segment-start buffer).
+// The rows another kernel has flagged (row_select): a small grid of workgroups that walk over the
+// batch rows, and over the tiles of a flagged row, themselves, so that the launch, in which
+// normally every workgroup finds nothing to do, dispatches as little as possible.  64 x 64
+// states only (16 lanes per state row, segment-start buffer).
+constexpr int ROW_SELECT_GRID = 32;
 template <typename IO, int KPL, int SIDE> __device__ __forceinline__ void bwd_scan_rows(const ScanBwdArgs &p) {
-    const int64_t b = blockIdx.x;
-    if (p.row_select[b] == 0) return;
-    for (int tile = 0; tile < p.ntiles; ++tile) {
-        if (tile) __syncthreads();
-        bwd_scan_body_kg<IO, KPL, SIDE, 16, 1>(p, b, tile);
+    bool first = true;
+    for (int64_t b = blockIdx.x; b < p.B; b += gridDim.x) {
+        if (p.row_select[b] == 0) continue;          // the same for every thread of the workgroup
+        for (int tile = 0; tile < p.ntiles; ++tile) {
+            if (!first) __syncthreads();
+            first = false;
+            bwd_scan_body_kg<IO, KPL, SIDE, 16, 1>(p, b, tile);
+        }
     }
 }
 
@@ -88,7 +93,7 @@ int launch_bwd(ScanBwdArgs a, const ScanGeom &g, hipStream_t stream) {
     const size_t smem = base + (a.use_sub ? sub : 0);
     a.kg = g.kg;
     a.ntiles = (int)((nrows + g.rows - 1) / g.rows);
-    const int64_t nblocks = a.row_select != nullptr ? a.B : a.B * a.ntiles;
+    const int64_t nblocks = a.row_select != nullptr ? (a.B < ROW_SELECT_GRID ? a.B : ROW_SELECT_GRID) : a.B * a.ntiles;
     if (nblocks > 0x7fffffffLL) return fail(T2FW_ERR_UNSUPPORTED, "grid of %lld workgroups is too large", (long long)nblocks);
     if constexpr (SIDE == 2) {
         // only the chunked kernels select rows: 64 x 64 states of 16-bit elements

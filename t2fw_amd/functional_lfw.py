@@ -25,7 +25,8 @@ def _ckpt_interval():
 
 def _flags():
     """Kernel-path flags (include/t2fw_hip.h): 0 = automatic, 1 = exact scan kernels only,
-    2 = fp16 matrix-core operands for fp16 tensors.  Overridable with T2FW_FLAGS."""
+    2 = fp16 matrix-core operands for fp16 tensors, 8 = block-wise matrix-core kernels.
+    Overridable with T2FW_FLAGS."""
     v = os.environ.get("T2FW_FLAGS")
     return int(v) if v else _lib.FLAG_AUTO
 
@@ -84,7 +85,7 @@ def _lfw_forward(value, forget, query, key, f_key, state, need_grad, heads=False
         if need_grad:
             nc = lib.t2fw_lfw_num_ckpt(T, C)
             ckpt = torch.empty((B * H, nc, D, K), dtype=value.dtype, device=dev)
-        ws_bytes = lib.t2fw_lfw_workspace_bytes(B * H, T, D, K, C, code, flags)
+        ws_bytes = lib.t2fw_lfw_forward_workspace_bytes(B * H, T, D, K, C, code, flags)
         ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev) if ws_bytes else None
         ptrs = (_lib.ptr(value), _lib.ptr(forget), _lib.ptr(query), _lib.ptr(key), _lib.ptr(f_key),
                 _lib.ptr(state), _lib.ptr(outputs), _lib.ptr(next_state), _lib.ptr(ckpt))
