@@ -21,6 +21,9 @@ dfw        = the delta-rule kernels (forward + backward) at cfg3's shape in fp32
 copy256    = calibration workload for those counters: a 256 MiB device-to-device copy.
 cpu_baseline = the TorchScript restatement of the reference loop (oracle/), fp32,
              forward + autograd backward, timed on this host's cores on a bounded sample.
+parity     = computed in the same CPU leg: per tensor, the GPU results of the first three rows of
+             input set 0 against the float64 oracle on the same quantised inputs (max-abs error,
+             max-abs error / max|reference|, mean relative error).
 """
 import argparse
 import json
@@ -76,7 +79,7 @@ def main():
 
     import torch
     from t2fw_amd import _lib
-    from tests.lfw_cases import make_config_inputs
+    from t2fw_amd.synthetic import make_config_inputs
 
     if not torch.cuda.is_available():
         print("bench.py: no GPU visible", file=sys.stderr)
@@ -243,15 +246,19 @@ def main():
         autograd["graph_replay_value"] = round(B * T / autograd["graph_replay_ms_per_step"] / 1e3, 1)
 
     cpu = None
+    parity = None
     if not args.no_cpu_baseline:
         cpu = cpu_baseline(w, backward)
+        if not H:
+            parity = parity_report(sets[0], fwd, bwd if backward else None)
 
     line = {
         "metric": "fwd+bwd Mtokens/s + % HBM roofline, B*H=96 T=1024 d=kdim=64 fp16" if args.workload == "cfg3"
                   else "Mtokens/s (%s)" % args.workload,
         "value": round(mtok, 1), "unit": "Mtokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms_per_step, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": {"float16": "fp16", "bfloat16": "bf16"}[w["dtype"]] + " I/O, fp32 state",
+        "dtype": {"float16": "fp16", "bfloat16": "bf16"}[w["dtype"]] + (
+            " I/O, fp32 state" if args.force_scan else " I/O, bf16 MFMA operands, fp32 accumulate"),
         "data": "synthetic",
         "config": {"workload": "%s: B=%d T=%d D=%d K=%d %s %s, checkpoint interval %d" % (
             args.workload, B, T, D, K, w["dtype"], "fwd+bwd" if backward else "fwd", C),
@@ -262,10 +269,35 @@ def main():
         "autograd_api": autograd,
         "roofline": roofline,
         "cpu_baseline": cpu,
+        "parity": parity,
     }
     if cpu:
         line["speedup_vs_cpu"] = round(mtok / cpu["value"], 1) if cpu["value"] else None
     print(json.dumps(line))
+
+
+def parity_report(d, fwd, bwd, rows=3):
+    """Part of the CPU leg: the GPU results of input set `d` (recomputed here, outside any timed
+    region) against the float64 oracle on the first `rows` batch rows (rows are independent)."""
+    import torch
+    from oracle import c_oracle
+    from t2fw_amd.synthetic import err_stats
+    fwd(d)
+    if bwd is not None:
+        bwd(d)
+    torch.cuda.synchronize()
+    ins = [t[:rows].cpu() for t in d["ins"]]
+    r_out, r_nxt = c_oracle.lfw_forward(*ins)
+    pairs = [("outputs", d["out"][:rows], r_out), ("next_state", d["nxt"][:rows], r_nxt)]
+    if bwd is not None:
+        r_grads = c_oracle.lfw_backward(d["go"][:rows].cpu(), d["gs"][:rows].cpu(), *ins)
+        pairs += [(n, g[:rows], r) for n, g, r in zip(("d_x", "d_f", "d_q", "d_k", "d_f_key", "d_state"), d["grads"], r_grads)]
+    rep = {"reference": "float64 oracle (oracle/lfw_oracle.c) on the same quantised inputs", "rows": rows, "tensors": {}}
+    for name, got, ref in pairs:
+        mx, rel, mean_rel = err_stats(got, torch.as_tensor(ref))
+        rep["tensors"][name] = {"max_abs": float("%.3e" % mx), "max_abs_over_max_ref": float("%.3e" % rel),
+                                "mean_rel": float("%.3e" % mean_rel)}
+    return rep
 
 
 def bench_copy(args):
@@ -373,7 +405,7 @@ def bench_generation(args):
     one call of t2fw_lfw_step over the whole batch; bytes = state read + write + six vectors."""
     import torch
     from t2fw_amd import _lib
-    from tests.lfw_cases import make_config_inputs
+    from t2fw_amd.synthetic import make_config_inputs
     lib = _lib.load()
     w = WORKLOADS["cfg5"]
     B, D, K = w["B"], w["D"], w["K"]
@@ -431,7 +463,7 @@ def cpu_baseline(w, backward):
     Bounded sample: a slice of the batch (rows are independent, so cost is linear in B)."""
     import torch
     from oracle.lfw_ref import lfw_reference_script
-    from tests.lfw_cases import make_config_inputs
+    from t2fw_amd.synthetic import make_config_inputs
     B, T, D, K = w["B"], w["T"], w["D"], w["K"]
     Bs = min(B, 24)
     Ts = min(T, 1024)

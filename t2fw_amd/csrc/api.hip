@@ -159,11 +159,6 @@ int static_scratch(void **out) {
 }
 }  // namespace
 
-#ifdef T2FW_PAR_TIMERS
-static unsigned long long *g_dbg = nullptr;
-extern "C" void t2fw_debug_set_buffer(void *p) { g_dbg = static_cast<unsigned long long *>(p); }
-#endif
-
 extern "C" {
 
 int t2fw_abi_version(void) { return T2FW_ABI_VERSION; }
@@ -352,9 +347,6 @@ static int lfw_backward_rows(const void *g_out, const void *g_state, const void 
             pa.gh = ws + sc.gh;
             pa.B = B; pa.T = T; pa.NC = a.NC; pa.C = C;
             pa.heads = (int32_t)heads;
-#ifdef T2FW_PAR_TIMERS
-            pa.dbg = g_dbg;
-#endif
             if ((rc = par_backward(pa, dtype, st))) return rc;
             if (flags & T2FW_FLAG_NO_FIXUP) return T2FW_OK;
             a.row_select = pa.row_flags;

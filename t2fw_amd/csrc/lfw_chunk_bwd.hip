@@ -392,7 +392,6 @@ __device__ __forceinline__ void bwd_prep_waves(const ChunkBwdArgs &p, unsigned c
     TokenMap<HEADS> tmap(HEADS ? (u32)p.heads * CH_N : (u32)CH_N, h, c);
     const u32 ts = tmap.ts;                              // elements between consecutive tokens
     u32 bad = 0;
-    PHASE_BEGIN();
 
     // Raw inputs of a part of a stage -> registers; tok: first token of the part's pair of blocks.
     // ANY: the block may reach past the end of the sequence or lie past it; the loads then go through
@@ -448,9 +447,7 @@ __device__ __forceinline__ void bwd_prep_waves(const ChunkBwdArgs &p, unsigned c
             issue(setR, nxt.tok_r, any_next, std::false_type{});
             if (cur.has_r) prep_lane_r<OPE>(fl, buf + OFF_RPART + jb * RBLOCK_BYTES, own, h, c, bad);
         }
-        PHASE_MARK(2);
         __syncthreads();
-        PHASE_MARK(3);
     };
     // Blocks can be partial or missing only in the last chunk, i.e. in the prologue and the first
     // transition: those stages go through the general loader unless that chunk is full.  Parts that a
@@ -487,7 +484,6 @@ __device__ __forceinline__ void bwd_prep_waves(const ChunkBwdArgs &p, unsigned c
     // Both workgroups of a row see all four gates' blocks and reach the same verdict, so either
     // order of their writes leaves the same flag.
     if (bad) p.row_flags[b] = 1;
-    PHASE_END(4 + (tid >> 6));
 }
 
 template <typename IOE, typename OPE, int NB, bool HEADS, int SIDE>
@@ -541,7 +537,6 @@ __device__ __forceinline__ void bwd_matrix_waves(const ChunkBwdArgs &p, unsigned
         p.row_flags[b] = 0;
         p.row_flags[chunk_rows_padded(p.B) + b] = 0;
     }
-    PHASE_BEGIN();
 
     // R part of a stage: the states at the start of blocks i2 and i2 + 1 of a chunk with nbc blocks
     // (S runs forward over them), as MFMA operands into d0 and d1
@@ -683,9 +678,7 @@ __device__ __forceinline__ void bwd_matrix_waves(const ChunkBwdArgs &p, unsigned
     for (int k = 0; k < MP; ++k) {
         if (2 * k < nb_last) {
             __syncthreads();
-            PHASE_MARK(3);
             r_pair(smem + (s & 1) * STAGE_BYTES, nb_last, 2 * k, sv[2 * k], sv[2 * k + 1]);
-            PHASE_MARK(0);
             ++s;
         }
     }
@@ -698,7 +691,6 @@ __device__ __forceinline__ void bwd_matrix_waves(const ChunkBwdArgs &p, unsigned
         const int nb = chunk == NC - 1 ? nb_last : NB;
         {
             __syncthreads();
-            PHASE_MARK(2);
             const unsigned char *stage = smem + (s & 1) * STAGE_BYTES;
             b_pair(stage, chunk, nb, std::integral_constant<int, NB - 2>{});
             take_state(pf, S);
@@ -709,12 +701,10 @@ __device__ __forceinline__ void bwd_matrix_waves(const ChunkBwdArgs &p, unsigned
 #pragma unroll
                 for (int j = 0; j < 4; ++j) park[j] = make_float4(S[j][0], S[j][1], S[j][2], S[j][3]);
             }
-            PHASE_MARK(1);
             ++s;
         }
         if constexpr (MP == 2) {
             __syncthreads();
-            PHASE_MARK(2);
             const unsigned char *stage = smem + (s & 1) * STAGE_BYTES;
             b_pair(stage, chunk, nb, std::integral_constant<int, 0>{});
 #pragma unroll
@@ -723,7 +713,6 @@ __device__ __forceinline__ void bwd_matrix_waves(const ChunkBwdArgs &p, unsigned
                 S[j][0] = v.x; S[j][1] = v.y; S[j][2] = v.z; S[j][3] = v.w;
             }
             r_pair(stage, NB, 2, sv[0], sv[1]);
-            PHASE_MARK(1);
             ++s;
             // ... which leaves the two pairs in each other's place
 #pragma unroll
@@ -742,16 +731,12 @@ __device__ __forceinline__ void bwd_matrix_waves(const ChunkBwdArgs &p, unsigned
         const int nb = NC == 1 ? nb_last : NB;
         if (NB - 2 < nb && MP == 2) {
             __syncthreads();
-            PHASE_MARK(2);
             b_pair(smem + (s & 1) * STAGE_BYTES, 0, nb, std::integral_constant<int, NB - 2>{});
-            PHASE_MARK(1);
             ++s;
         }
         {
             __syncthreads();
-            PHASE_MARK(2);
             b_pair(smem + (s & 1) * STAGE_BYTES, 0, nb, std::integral_constant<int, 0>{});
-            PHASE_MARK(1);
             ++s;
         }
     }
@@ -761,7 +746,6 @@ __device__ __forceinline__ void bwd_matrix_waves(const ChunkBwdArgs &p, unsigned
 #pragma unroll
         for (int j = 0; j < 4; ++j) *reinterpret_cast<uint2 *>(ds + ch * CH_N + 16 * j + 4 * g) = pack4v<IOE>(G[j]);
     }
-    PHASE_END(tid >> 6);
 }
 
 template <typename IOE, typename OPE, int NB, bool HEADS>

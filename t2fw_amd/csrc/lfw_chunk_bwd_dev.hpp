@@ -3,20 +3,6 @@
 
 #include "lfw_chunk.hpp"
 
-// Build-time diagnostic (-DT2FW_PHASE_TIMERS): workgroup 0 accumulates shader-clock ticks
-// per phase into row_flags[64..]; off in the shipped library.
-#ifdef T2FW_PHASE_TIMERS
-#define PHASE_BEGIN() unsigned long long ph_t = __builtin_amdgcn_s_memtime(); unsigned long long ph_acc[8] = {0, 0, 0, 0, 0, 0, 0, 0}; int ph_sel = 0
-#define PHASE_MARK(i) { const unsigned long long ph_n = __builtin_amdgcn_s_memtime(); ph_acc[(i) + ph_sel] += ph_n - ph_t; ph_t = ph_n; }
-#define PHASE_END(slot) if (b == 0 && (tid & 63) == 0) { for (int ph_i = 0; ph_i < 8; ++ph_i) p.row_flags[64 + (slot) * 8 + ph_i] = (int)(ph_acc[ph_i] & 0x7fffffff); }
-#define PHASE_SELECT(v) ph_sel = (v)
-#else
-#define PHASE_BEGIN()
-#define PHASE_MARK(i)
-#define PHASE_END(slot)
-#define PHASE_SELECT(v)
-#endif
-
 namespace t2fw {
 namespace bwd {
 

@@ -21,18 +21,6 @@
 #include "lfw_chunk.hpp"
 #include "lfw_scan_body.hpp"
 
-// Build-time diagnostic (-DT2FW_PHASE_TIMERS): workgroup 0 accumulates shader-clock ticks
-// per phase into row_flags[64..]; off in the shipped library.
-#ifdef T2FW_PHASE_TIMERS
-#define PHASE_BEGIN() unsigned long long ph_t = __builtin_amdgcn_s_memtime(); unsigned long long ph_acc[4] = {0, 0, 0, 0}
-#define PHASE_MARK(i) { const unsigned long long ph_n = __builtin_amdgcn_s_memtime(); ph_acc[i] += ph_n - ph_t; ph_t = ph_n; }
-#define PHASE_END(slot) if (b == 0 && (tid & 63) == 0) { for (int ph_i = 0; ph_i < 4; ++ph_i) p.row_flags[64 + (slot) * 8 + ph_i * 2] = (int)(ph_acc[ph_i] & 0x7fffffff); }
-#else
-#define PHASE_BEGIN()
-#define PHASE_MARK(i)
-#define PHASE_END(slot)
-#endif
-
 namespace t2fw {
 namespace {
 
@@ -315,11 +303,8 @@ __device__ __forceinline__ void fwd_prep_side(const ChunkFwdArgs &p, unsigned ch
     // that publishes the tiles comes after every odd step and after the last one.
     const int nsteps = nfull + (nfull * CH_STEP < T ? 1 : 0);
     auto publish = [&](int n) {
-        PHASE_MARK(0);
         if ((n & 1) || n == nsteps - 1) __syncthreads();
-        PHASE_MARK(3);
     };
-    PHASE_BEGIN();
     if (nfull > 0) {
         RawSet<NV> setA, setB;
         int n = 0;
@@ -351,7 +336,6 @@ __device__ __forceinline__ void fwd_prep_side(const ChunkFwdArgs &p, unsigned ch
         p.row_flags[flag_slot] = 1;
         *reinterpret_cast<volatile int *>(smem + OFF_VERDICT) = 1;
     }
-    PHASE_END(4 + (tid >> 6));
 }
 
 template <typename E> __device__ __forceinline__ uint2 pack4(const floatx4 &v) {
@@ -395,7 +379,6 @@ __device__ __forceinline__ void fwd_matrix_waves(const ChunkFwdArgs &p, unsigned
         if (clear_other_slot) p.row_flags[chunk_rows_padded(p.B) + b] = 0;
         *reinterpret_cast<volatile int *>(smem + OFF_VERDICT) = 0;
     }
-    PHASE_BEGIN();
     // One step (two blocks).  FULL: all 32 tokens exist, which leaves the body without a branch
     // around its stores, so that the LDS reads of the whole step can be scheduled ahead of the
     // matrix products that use them.
@@ -404,7 +387,6 @@ __device__ __forceinline__ void fwd_matrix_waves(const ChunkFwdArgs &p, unsigned
         constexpr bool FULL = decltype(full_c)::value;
         if constexpr (decltype(bar_c)::value) {
             __syncthreads();        // the operand tiles of steps n and n + 1 are in LDS
-            PHASE_MARK(3);
         }
         const unsigned char *ops = smem + (n & 3) * OPS_BYTES;
         const u16 *QT = reinterpret_cast<const u16 *>(ops + OFF_QT);
@@ -468,7 +450,6 @@ __device__ __forceinline__ void fwd_matrix_waves(const ChunkFwdArgs &p, unsigned
                 S[j][3] *= aL * bl.w;
                 S[j] = OPE::mfma16(*reinterpret_cast<const uint2 *>(KH + (16 * j + r) * CS + tok0 + 4 * g), xh, S[j]);
             }
-            PHASE_MARK(hh);
         }
     };
     const int nfull = T / CH_STEP;
@@ -485,7 +466,6 @@ __device__ __forceinline__ void fwd_matrix_waves(const ChunkFwdArgs &p, unsigned
             step(nfull, std::false_type{}, std::true_type{});
     }
     store_state<IOE>(S, reinterpret_cast<u16 *>(p.next_state) + b * (CH_N * CH_N), d, g);
-    PHASE_END(tid >> 6);
 }
 
 // End of a workgroup's work on its (part of a) batch row.  A barrier publishes the prep waves'

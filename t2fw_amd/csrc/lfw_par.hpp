@@ -46,7 +46,6 @@ struct ParBwdArgs {
     float *vecs;                       // scratch [B, NC, PAR_NVEC, 64]
     int32_t *chunk_flags;              // scratch [B * NC]: 1 for chunks this form cannot take
     int32_t *row_flags;                // [B]: 1 for rows with such a chunk (their results are not valid)
-    unsigned long long *dbg;           // phase timestamps of workgroup 0 (diagnostic builds only; null otherwise)
     int64_t B, T, NC;
     int32_t C;                         // checkpoint interval = chunk length: 32 or 64
     int32_t heads;                     // as in ChunkFwdArgs
@@ -66,18 +65,6 @@ int par_backward(const ParBwdArgs &a, int dtype, hipStream_t stream);
 int par_forward(const ParFwdArgs &a, int dtype, hipStream_t stream);
 
 #if defined(__HIPCC__)
-// Build-time diagnostic (-DT2FW_PAR_TIMERS): the first lane of every wave of workgroup 0 records shader-clock
-// ticks at phase boundaries into p.dbg[wave * 32 + k]; off in the shipped library.
-#ifdef T2FW_PAR_TIMERS
-#define PT_DECL unsigned long long pt_t[32]; int pt_n = 0
-#define PT_MARK() do { if (pt_n < 32) pt_t[pt_n++] = __builtin_amdgcn_s_memtime(); } while (0)
-#define PT_FLUSH(p) do { if ((p).dbg != nullptr && blockIdx.x == 0 && (threadIdx.x & 63) == 0) { for (int pt_i = 0; pt_i < 32; ++pt_i) (p).dbg[(threadIdx.x >> 6) * 32 + pt_i] = pt_i < pt_n ? pt_t[pt_i] : 0ull; } } while (0)
-#else
-#define PT_DECL
-#define PT_MARK()
-#define PT_FLUSH(p)
-#endif
-
 namespace par {
 
 using namespace bwd;

@@ -13,11 +13,7 @@
 namespace t2fw {
 namespace {
 
-#ifdef STEP_THREADS_OVERRIDE
-constexpr int STEP_THREADS = STEP_THREADS_OVERRIDE;
-#else
 constexpr int STEP_THREADS = 128;
-#endif
 
 template <typename E> __device__ __forceinline__ void unpack8(const uint4 &v, float (&o)[8]) {
     const u32 w[4] = {v.x, v.y, v.z, v.w};

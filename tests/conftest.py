@@ -21,3 +21,14 @@ def pytest_collection_modifyitems(config, items):
     for item in items:
         if "gpu" in item.keywords:
             item.add_marker(skip)
+
+
+def pytest_terminal_summary(terminalreporter):
+    """After a GPU run: how much of every stated tolerance the worst element used."""
+    mod = sys.modules.get("tests.test_lfw_gpu")
+    use = getattr(mod, "TOLERANCE_USE", None)
+    if not use:
+        return
+    terminalreporter.write_sep("-", "largest |err| / bound per (rtol, afrac, tensor)")
+    for (rtol, afrac, what), v in sorted(use.items()):
+        terminalreporter.write_line("rtol %-8g afrac %-8g %-12s %.3f" % (rtol, afrac, what, v))

@@ -11,7 +11,7 @@ import torch
 
 from oracle import c_oracle
 from tests.lfw_cases import make_config_inputs, make_reference_test_inputs
-from tests.test_lfw_chunk_gpu import NAMES, flagged_rows, run_abi
+from tests.test_lfw_chunk_gpu import NAMES, chunk_parallel_backward, flagged_rows, run_abi
 from tests.test_lfw_gpu import TOL, TOL_CHUNK, TOL_CHUNK_GATE, assert_close, gate_grad_floor, on_chunk_path
 
 pytestmark = pytest.mark.gpu
@@ -72,7 +72,7 @@ def run_heads_abi(inputs, go, gs, B, H, C, flags=0):
                                            *[_lib.ptr(t) for t in grads], B, T, H, D, K, C, code, flags,
                                            _lib.ptr(ws), wsb, st))
     torch.cuda.synchronize()
-    flagged_bwd = flagged_rows(ws, B * H) if wsb else 0
+    flagged_bwd = flagged_rows(ws, B * H, chunk_parallel_backward(C, flags)) if wsb else 0
     folded = [from_heads(g) for g in grads[:5]] + [grads[5]]
     return from_heads(out), nxt, ckpt, folded, (flagged_fwd, flagged_bwd)
 

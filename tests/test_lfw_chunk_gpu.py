@@ -13,12 +13,23 @@ pytestmark = pytest.mark.gpu
 NAMES = ("d_x", "d_f", "d_q", "d_k", "d_f_key", "d_state")
 
 
-def flagged_rows(ws, B):
-    """rows the matrix-core kernels handed to the exact kernels: two flag slots per row (kernels that
-    split a row over two workgroups report per workgroup), the second at the batch padded to 8"""
+def flagged_rows(ws, B, chunk_parallel=False):
+    """Rows the matrix-core kernels handed to the exact kernels.  The block-wise kernels keep two
+    flag slots per row at the start of the workspace (kernels that split a row over two workgroups
+    report per workgroup), the second at the batch padded to 8; the chunk-parallel backward keeps
+    one slot per row in the 256-byte-aligned region after them."""
     f = ws.view(torch.int32)
     pad = (B + 7) // 8 * 8
+    if chunk_parallel:
+        base = (2 * pad * 4 + 255) // 256 * 256 // 4
+        return int((f[base:base + B] != 0).sum())
     return int(((f[:B] != 0) | (f[pad:pad + B] != 0)).sum())
+
+
+def chunk_parallel_backward(C, flags):
+    """the backward runs the chunk-parallel kernels unless a flag asks for the block-wise ones"""
+    from t2fw_amd import _lib
+    return C in (32, 64) and not flags & (_lib.FLAG_BLOCKWISE | 2 | 1)
 
 
 def run_abi(inputs, go, gs, C, flags=0, with_backward=True):
@@ -48,24 +59,50 @@ def run_abi(inputs, go, gs, C, flags=0, with_backward=True):
                                          _lib.ptr(ckpt), *[_lib.ptr(t) for t in grads], B, T, D, K, C, code, flags,
                                          _lib.ptr(ws), wsb, st))
         torch.cuda.synchronize()
-        flagged_bwd = flagged_rows(ws, B) if wsb else 0
+        flagged_bwd = flagged_rows(ws, B, chunk_parallel_backward(C, flags)) if wsb else 0
     return out, nxt, ckpt, grads, (flagged_fwd, flagged_bwd)
 
 
-def check_against_oracle(inputs, go, gs, C, dtype, flags=0, expect_flagged=None, tol=None, gate_tol=None):
-    out, nxt, ckpt, grads, flagged = run_abi(inputs, go, gs, C, flags)
-    if expect_flagged is not None:
-        assert flagged == (expect_flagged, expect_flagged), flagged
+def assert_within_reference_bounds(out, r_out, grads, r_grads):
+    """The tolerances of the reference's own fp16 test (tests/test_lfw.py:65,92), the outer bound.
+    The reference computes in fp32 and asserts these on its own shape grid (no 64 x 64 state, at
+    most 64 steps).  The matrix-core kernels round the contraction operands to bf16: their error is
+    a fraction of max|ref| (the chunk tolerance), which passes atol = 1e-2 on near-zero elements only
+    while max|ref| stays below about 3; tests whose outputs grow larger opt out and say so."""
+    assert torch.allclose(out.double().cpu(), torch.as_tensor(r_out).double(), atol=1e-2, rtol=1e-1)
+    for n, g, r in zip(NAMES, grads, r_grads):
+        assert torch.allclose(g.double().cpu(), torch.as_tensor(r).double(), atol=0.1, rtol=1e-1), n
+
+
+def check_against_oracle(inputs, go, gs, C, dtype, flags=0, expect_flagged=None, tol=None, gate_tol=None,
+                         reference_bounds=True, expect_flagged_parallel=None):
+    """Forward and backward against the fp64 oracle.  Where the chunk-parallel backward applies, the
+    block-wise backward (flag 8) is checked on the same inputs as well."""
+    from t2fw_amd import _lib
     r_out, r_nxt = c_oracle.lfw_forward(*inputs)
     r_grads = c_oracle.lfw_backward(go, gs, *inputs)
     tol = tol or TOL_CHUNK
     gate_tol = gate_tol or TOL_CHUNK_GATE
     floors = gate_grad_floor(inputs, go, r_out, r_grads)
-    assert_close(out, r_out, dtype, "outputs", tol=tol)
-    assert_close(nxt, r_nxt, dtype, "next_state", tol=tol)
-    for n, g, r in zip(NAMES, grads, r_grads):
-        assert_close(g, r, dtype, n, tol=gate_tol if n in ("d_f", "d_f_key") else tol, floor=floors.get(n, 0.0))
-    return out, nxt, ckpt, grads
+    variants = [flags] + ([flags | _lib.FLAG_BLOCKWISE] if chunk_parallel_backward(C, flags) else [])
+    first = None
+    for fl in variants:
+        tag = " (flags %d)" % fl
+        out, nxt, ckpt, grads, flagged = run_abi(inputs, go, gs, C, fl)
+        if expect_flagged is not None:
+            want = (expect_flagged, expect_flagged)
+            if expect_flagged_parallel is not None and chunk_parallel_backward(C, fl):
+                want = (expect_flagged, expect_flagged_parallel)     # the two backward forms accept different gate ranges
+            assert flagged == want, (flagged, fl)
+        assert_close(out, r_out, dtype, "outputs" + tag, tol=tol)
+        assert_close(nxt, r_nxt, dtype, "next_state" + tag, tol=tol)
+        for n, g, r in zip(NAMES, grads, r_grads):
+            assert_close(g, r, dtype, n + tag, tol=gate_tol if n in ("d_f", "d_f_key") else tol,
+                         floor=floors.get(n, 0.0))
+        if dtype == torch.float16 and reference_bounds:
+            assert_within_reference_bounds(out, r_out, grads, r_grads)
+        first = first or (out, nxt, ckpt, grads)
+    return first
 
 
 @pytest.mark.parametrize("dtype,gate_mean,state_std", [(torch.float16, 2.0, 0.0), (torch.bfloat16, 3.0, 0.1)])
@@ -157,9 +194,13 @@ def test_wide_gate_distribution_stays_on_the_chunked_path():
 
 def test_reference_test_gates_stay_on_the_chunked_path():
     # per-channel constant gates in (1/64, 1-1/64) as the reference's tests build them
+    # (16-step products down to 2^-96).  The chunk-parallel backward scales by products over half a
+    # chunk, which these gates take below its range in every row: it hands the rows to the exact scan.
+    # Unit-variance inputs over 256 steps give outputs up to 6, so atol = 1e-2 of the reference's test
+    # is below the bf16 rounding of the forward's operands: chunk tolerance only.
     x, f, q, k, fk, s, go, gs = make_reference_test_inputs(2, 256, 64, 64, torch.float16, seed=1)
     check_against_oracle((x, f, q, k, fk, s), go, gs, 64, torch.float16, expect_flagged=0,
-                         gate_tol=(2e-1, 4e-2))
+                         expect_flagged_parallel=2, gate_tol=(2e-1, 4e-2), reference_bounds=False)
 
 
 @pytest.mark.parametrize("kind", ["zero_gate", "zero_gate_upper_channels", "gate_above_one", "negative_gate",

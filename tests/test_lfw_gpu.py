@@ -27,7 +27,7 @@ TOL = {
 # rounded to bf16 (2^-9 relative), accumulation is fp32.  The gate gradients are differences
 # of products of such quantities and carry a wider bound.
 TOL_CHUNK = (2e-2, 1e-2)
-TOL_CHUNK_GATE = (4e-2, 4e-2)
+TOL_CHUNK_GATE = (2e-2, 2e-2)
 
 
 def on_chunk_path(dtype, D, K):
@@ -47,6 +47,11 @@ def gate_grad_floor(inputs, go, r_out, r_grads):
     return {"d_f": fl_f, "d_f_key": fl_k}
 
 
+# (rtol, afrac, tensor) -> largest |err| / bound seen in this session; printed after the run so the
+# stated tolerances can be compared with what the kernels actually use of them
+TOLERANCE_USE = {}
+
+
 def assert_close(got, ref, dtype, what, scale=1.0, tol=None, floor=0.0):
     rtol, afrac = tol if tol is not None else TOL[dtype]
     got = got.detach().double().cpu()
@@ -57,6 +62,8 @@ def assert_close(got, ref, dtype, what, scale=1.0, tol=None, floor=0.0):
     assert torch.isfinite(got).all(), what + " has non-finite values"
     bound = scale * (rtol * ref.abs() + afrac * max(float(ref.abs().max()), floor))
     bad = (got - ref).abs() > bound
+    key = (rtol, afrac, what.split("[")[0].split(" (")[0])
+    TOLERANCE_USE[key] = max(TOLERANCE_USE.get(key, 0.0), float(((got - ref).abs() / bound.clamp_min(1e-300)).max()))
     assert not bad.any(), "%s: %d/%d outside tolerance, max-abs err %.3e (max|ref| %.3e)" % (
         what, int(bad.sum()), ref.numel(), float((got - ref).abs().max()), float(ref.abs().max()))
 
