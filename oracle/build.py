@@ -12,12 +12,12 @@ import sys
 HERE = os.path.dirname(os.path.abspath(__file__))
 OUT_DIR = os.path.join(HERE, "_build")
 LIB = os.path.join(OUT_DIR, "liboracle.so")
-SOURCES = ["lfw_oracle.c", "dfw_oracle.c"]
+SOURCES = ["lfw_oracle.c"]
 
 
 def build(verbose: bool = False) -> str:
     os.makedirs(OUT_DIR, exist_ok=True)
-    srcs = [os.path.join(HERE, s) for s in SOURCES if os.path.exists(os.path.join(HERE, s))]
+    srcs = [os.path.join(HERE, s) for s in SOURCES]
     cmd = ["gcc", "-O2", "-fopenmp", "-shared", "-fPIC", "-std=c11", "-Wall", "-Wextra",
            "-o", LIB] + srcs + ["-lm"]
     if verbose:

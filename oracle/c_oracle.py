@@ -1,4 +1,4 @@
-"""ctypes front-end of the C oracle (oracle/lfw_oracle.c, oracle/dfw_oracle.c).
+"""ctypes front-end of the C oracle (oracle/lfw_oracle.c; the delta rule's oracle is oracle/dfw_ref.py).
 
 TEST INFRASTRUCTURE ONLY.  Loads oracle/_build/liboracle.so, building it with gcc
 when it is missing (the oracle is CPU code; building the checker is not using it).

@@ -57,7 +57,13 @@ class FastWeightState(torch.nn.Module):
             # generation step: the state is read and written once, in place
             if self.state is None:
                 self.state = state
+            elif self.state.grad_fn is not None or self.state.requires_grad:
+                # the state is still part of a recorded graph (a training call came before): step on a
+                # private copy, so that nothing the graph may read is overwritten behind autograd's back
+                self.state = self.state.detach().clone()
             out, _ = lfw_step(x, f, q, k, f_key, self.state, inplace=True)
+            # the kernel wrote through a raw pointer: tell autograd's version counter
+            torch.autograd.graph.increment_version(self.state)
             return out
         if single:
             x, f, q, k, f_key = (t.unsqueeze(1) for t in (x, f, q, k, f_key))
@@ -66,6 +72,14 @@ class FastWeightState(torch.nn.Module):
         # choice: detach_state() cuts it)
         self.state = new_state if needs_grad else new_state.detach()
         return out.squeeze(1) if single else out
+
+    def _apply(self, fn, *args, **kwargs):
+        """``.to()``, ``.half()``, ``.cuda()`` move the carried state with the module (it is neither a
+        parameter nor a buffer, so that it never lands in a state_dict)."""
+        super()._apply(fn, *args, **kwargs)
+        if self.state is not None:
+            self.state = fn(self.state.detach())
+        return self
 
     def detach_state(self):
         if self.state is not None:

@@ -73,6 +73,16 @@ def test_other_dtypes_and_shapes(dtype, shape):
     check(*make_inputs(B, T, D, M, dtype, seed=7), dtype)
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
+@pytest.mark.parametrize("shape", [(1, 6, 3, 100), (1, 6, 100, 3), (1, 5, 2, 600), (1, 5, 600, 2), (1, 4, 2, 2048),
+                                   (1, 4, 2048, 2)])
+def test_wide_states_every_lane_geometry(dtype, shape):
+    """state rows of 65..128, 513..1024 and 2048 columns on either side (32 lanes per row, 16 / 32
+    columns per lane)"""
+    B, T, D, M = shape
+    check(*make_inputs(B, T, D, M, dtype, seed=8), dtype)
+
+
 def test_value_dim_larger_than_key_dim():
     # D > M, the case where the reference's backward kernel overruns its shared memory
     # (dfw_kernel.cu:227 vs :523); nothing of the kind exists here

@@ -132,6 +132,36 @@ def test_general_shapes_all_dtypes(dtype, shape):
     check_all((x, f, q, k, fk, s), go, gs, dtype)
 
 
+WIDE_SHAPES = [(1, 6, 3, 100), (1, 6, 100, 3), (1, 5, 2, 600), (1, 5, 600, 2), (1, 4, 2, 2048), (1, 4, 2048, 2)]
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
+@pytest.mark.parametrize("shape", WIDE_SHAPES)
+def test_wide_states_every_lane_geometry(dtype, shape):
+    """State rows of 65..128, 513..1024 and 2048 columns on either side: 32 lanes per row and 16 / 32
+    columns per lane, which no narrower shape reaches."""
+    B, T, D, K = shape
+    x, f, q, k, fk, s, go, gs = make_config_inputs(B, T, D, K, dtype, seed=6, in_scale=0.5,
+                                                    gate_mean=1.0, state_std=0.5, gstate_std=0.5)
+    check_all((x, f, q, k, fk, s), go, gs, dtype)
+
+
+def test_too_wide_for_training_is_refused_in_the_forward():
+    """D above the exact backward's limit: refused when the forward is asked for checkpoints, not
+    later in backward(); the same shape runs without them."""
+    from t2fw.functional_lfw import LFWFunction
+    x, f, q, k, fk, s, go, gs = make_config_inputs(1, 3, 2100, 2, torch.float32, seed=6, in_scale=0.5,
+                                                    gate_mean=1.0, state_std=0.5)
+    ins = [t.cuda() for t in (x, f, q, k, fk, s)]
+    with torch.no_grad():
+        out, nxt = LFWFunction.apply(*ins)
+    r_out, r_nxt = c_oracle.lfw_forward(x, f, q, k, fk, s)
+    assert_close(out, r_out, torch.float32, "outputs")
+    assert_close(nxt, r_nxt, torch.float32, "next_state")
+    with pytest.raises(RuntimeError, match="exact kernels take K <= 2048"):
+        LFWFunction.apply(*[t.requires_grad_(True) for t in ins])
+
+
 @pytest.mark.parametrize("C", [1, 7, 16, 64, 100, 1000])
 def test_checkpoint_interval_any_value(C, monkeypatch):
     # C need not divide T; C > T keeps a single checkpoint

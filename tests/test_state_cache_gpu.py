@@ -64,3 +64,40 @@ def test_training_keeps_the_graph_through_the_state():
     r = c_oracle.lfw_backward(go, torch.zeros_like(s), x, f, q, k, fk, s)
     for name, leaf, ref in zip(("d_x", "d_f", "d_q", "d_k", "d_f_key"), leaves, r):
         assert_close(leaf.grad, ref, torch.float32, name)
+
+
+def test_generation_after_a_training_call_does_not_touch_the_recorded_state():
+    """A training call leaves a state that belongs to its graph; the in-place generation step that
+    follows works on a copy, and tensors derived from the old state keep their values."""
+    from t2fw_amd.state_cache import FastWeightState
+    B, T = 2, 16
+    x, f, q, k, fk, s, go, _ = make_config_inputs(B, T + 1, 64, 64, torch.float16, seed=24, state_std=0.2)
+    leaves = [t.cuda().requires_grad_(True) for t in (x, f, q, k, fk)]
+    layer = FastWeightState(64, 64).reset(s.cuda())
+    o1 = layer(*[t[:, :T].contiguous() for t in leaves])
+    recorded = layer.state
+    assert recorded.grad_fn is not None
+    before = recorded.detach().clone()
+    with torch.no_grad():
+        layer(*[t[:, T].contiguous() for t in leaves])
+    assert layer.state.data_ptr() != recorded.data_ptr() and layer.state.grad_fn is None
+    assert torch.equal(recorded.detach(), before)
+    version = layer.state._version
+    with torch.no_grad():
+        layer(*[t[:, T].contiguous() for t in leaves])
+    assert layer.state._version > version            # the raw in-place write is visible to autograd
+    (o1 * go[:, :T].cuda()).sum().backward()          # the graph of the training call is intact
+    assert all(t.grad is not None for t in leaves)
+
+
+def test_state_follows_the_module_across_dtype_changes():
+    from t2fw_amd.state_cache import FastWeightState
+    B = 2
+    x, f, q, k, fk, s, _, _ = make_config_inputs(B, 2, 64, 64, torch.float32, seed=25, state_std=0.2)
+    layer = FastWeightState(64, 64).reset(s.cuda())
+    layer.half()
+    assert layer.state.dtype == torch.float16
+    with torch.no_grad():
+        out = layer(*[t[:, 0].cuda().half().contiguous() for t in (x, f, q, k, fk)])
+    r_out, _ = c_oracle.lfw_forward(*[t[:, :1].half() for t in (x, f, q, k, fk)], s.half())
+    assert_close(out, r_out[:, 0], torch.float16, "out")
