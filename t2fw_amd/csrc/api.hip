@@ -242,12 +242,6 @@ static int lfw_forward_rows(const void *x, const void *f, const void *q, const v
         const bool split = 2 * chunk_rows_padded(B) <= cus;
         return chunk_forward(c, dtype, op, split, st);
     }
-    // The exact scan keeps a state row (forward: K columns; backward: K columns on one side, D on
-    // the other) in the registers of one lane group.  A forward that writes checkpoints is followed
-    // by a backward, so it refuses what that backward could not take.
-    if (K > SCAN_MAX_COLS || (ckpt != nullptr && D > SCAN_MAX_COLS))
-        return fail(T2FW_ERR_UNSUPPORTED, "D=%lld, K=%lld: the exact kernels take K <= %d%s", (long long)D, (long long)K,
-                    SCAN_MAX_COLS, ckpt != nullptr ? " and, with checkpoints for a backward pass, D <= the same" : "");
     return scan_forward(a, dtype, st);
 }
 
@@ -363,10 +357,6 @@ static int lfw_backward_rows(const void *g_out, const void *g_state, const void 
         a.row_select = c.row_flags;      // rows the chunked form could not take
         if (flags & T2FW_FLAG_NO_FIXUP) return T2FW_OK;
     }
-    // checked before the first of the exact backward's two launches, so that a refusal writes nothing
-    if (D > SCAN_MAX_COLS || K > SCAN_MAX_COLS)
-        return fail(T2FW_ERR_UNSUPPORTED, "D=%lld, K=%lld: the exact backward kernels take D, K <= %d", (long long)D,
-                    (long long)K, SCAN_MAX_COLS);
     return scan_backward(a, dtype, st);
 }
 

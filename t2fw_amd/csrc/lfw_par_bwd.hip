@@ -199,13 +199,13 @@ template <typename IOE> __global__ __launch_bounds__(SCAN_TPB) void lfw_par_scan
 //      masks them and leaves them in LDS as ready 16-bit A operands, plus the diagonal    | barrier
 //   S  per side: forward-like sweep (o' / q'), backward-like sweep (x' / k'), gate gradient; the
 //      results go to global memory from the accumulator layout
-constexpr int GR_THREADS = 256;
+constexpr int GR_THREADS = 512;
 constexpr int PT_TILE = 64 * 8;                  // one 16 x 16 product tile as 16-bit operand: 8 bytes per lane
 constexpr int GR_ADJ = 0;                        // adjoint-scaled tile of each side
 constexpr int GR_VAL = GR_ADJ + 2 * CM_BYTES;    // value-scaled tile of each side
 constexpr int GR_S0 = GR_VAL + 2 * CM_BYTES, GR_GH = GR_S0 + CM_BYTES;
-constexpr int GR_PT = GR_GH + CM_BYTES;          // per side: 10 forward-like tiles (m, n <= m), 10 backward-like tiles (n, m >= n)
-constexpr int GR_PD = GR_PT + 2 * 20 * PT_TILE;  // per side: diagonal of the product, 64 floats
+constexpr int GR_PT = GR_GH + CM_BYTES;          // per side: the 10 product tiles (m, n <= m)
+constexpr int GR_PD = GR_PT + 2 * 10 * PT_TILE;  // per side: diagonal of the product, 64 floats
 constexpr int GR_SMEM = GR_PD + 2 * CH_N * 4;
 static_assert(2 * GR_SMEM <= 160 * 1024, "two workgroups of the gradient kernel must fit the LDS of one CU");
 
@@ -218,7 +218,7 @@ template <typename IOE, int NT, bool HEADS, bool FULL> struct GradsItem {
     static constexpr int CL = 16 * NT;
     const ParBwdArgs &p;
     unsigned char *smem;
-    int tid, T, NC, cb, i, kg, c, lane, n_left;
+    int tid, T, NC, cb, side, i, kg, c, lane, n_left;
     u32 ts, off;
     int64_t item;
 
@@ -226,7 +226,8 @@ template <typename IOE, int NT, bool HEADS, bool FULL> struct GradsItem {
         tid = threadIdx.x;
         T = (int)p.T; NC = (int)p.NC;
         ts = HEADS ? (u32)p.heads * CH_N : (u32)CH_N;
-        cb = __builtin_amdgcn_readfirstlane(tid >> 6);
+        cb = __builtin_amdgcn_readfirstlane((tid >> 6) & 3);
+        side = __builtin_amdgcn_readfirstlane(tid >> 8);
         lane = tid & 63;
         i = lane & 15; kg = lane >> 4; c = 16 * cb + i;
         const int64_t b = item / NC;
@@ -261,75 +262,82 @@ template <typename IOE, int NT, bool HEADS, bool FULL> struct GradsItem {
         store_cm<NT>(tile_val<SIDE>(), c, kg, valT);
         store_cm<NT>(tile_adj<SIDE>(), c, kg, adjS);
     }
-    // the chunk-start state scaled to the middle of the chunk, as bf16, and Gh': two 16-byte pieces of each per thread
-    __device__ __forceinline__ void stage_mats() const {
-        const float *const vref = p.vecs + item * (PAR_NVEC * CH_N);
-        const u16 *const s0 = reinterpret_cast<const u16 *>(p.ckpt) + item * (CH_N * CH_N);
-        const u16 *const gh = reinterpret_cast<const u16 *>(p.gh) + item * (CH_N * CH_N);
-        uint4 sv[2], gv[2];
-        float ra[2];
+    // the chunk-start state scaled to the middle of the chunk, as bf16, and Gh': one 16-byte piece of each
+    // per thread (eight columns (tid & 7) of row tid >> 3); the loads are issued with the raw inputs
+    struct MatRegs {
+        uint4 s0, gh;
+        float ra;
         float4 rb[2];
-#pragma unroll
-        for (int u = 0; u < 2; ++u) {
-            const int o8 = tid + 256 * u;        // eight columns (o8 & 7) of row o8 >> 3
-            sv[u] = *reinterpret_cast<const uint4 *>(s0 + o8 * 8);
-            gv[u] = *reinterpret_cast<const uint4 *>(gh + o8 * 8);
-            ra[u] = vref[2 * CH_N + (o8 >> 3)];
-        }
-        rb[0] = *reinterpret_cast<const float4 *>(vref + 3 * CH_N + (tid & 7) * 8);
-        rb[1] = *reinterpret_cast<const float4 *>(vref + 3 * CH_N + (tid & 7) * 8 + 4);
-        const float rbv[8] = {rb[0].x, rb[0].y, rb[0].z, rb[0].w, rb[1].x, rb[1].y, rb[1].z, rb[1].w};
-#pragma unroll
-        for (int u = 0; u < 2; ++u) {
-            const int o8 = tid + 256 * u;
-            float v[8];
-            const u32 sw[4] = {sv[u].x, sv[u].y, sv[u].z, sv[u].w};
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                v[2 * e] = IOE::to_f32((u16)(sw[e] & 0xffffu)) * (ra[u] * rbv[2 * e]);
-                v[2 * e + 1] = IOE::to_f32((u16)(sw[e] >> 16)) * (ra[u] * rbv[2 * e + 1]);
-            }
-            const int o = (o8 >> 3) * CMS + (o8 & 7) * 8;
-            *reinterpret_cast<uint4 *>(reinterpret_cast<u16 *>(smem + GR_S0) + o) =
-                make_uint4(Bf16::pack2(v[0], v[1]), Bf16::pack2(v[2], v[3]), Bf16::pack2(v[4], v[5]), Bf16::pack2(v[6], v[7]));
-            *reinterpret_cast<uint4 *>(reinterpret_cast<u16 *>(smem + GR_GH) + o) = gv[u];
-        }
+    };
+    __device__ __forceinline__ void issue_mats(MatRegs &r) const {
+        const float *const vref = p.vecs + item * (PAR_NVEC * CH_N);
+        r.s0 = *reinterpret_cast<const uint4 *>(reinterpret_cast<const u16 *>(p.ckpt) + item * (CH_N * CH_N) + tid * 8);
+        r.gh = *reinterpret_cast<const uint4 *>(reinterpret_cast<const u16 *>(p.gh) + item * (CH_N * CH_N) + tid * 8);
+        r.ra = vref[2 * CH_N + (tid >> 3)];
+        r.rb[0] = *reinterpret_cast<const float4 *>(vref + 3 * CH_N + (tid & 7) * 8);
+        r.rb[1] = *reinterpret_cast<const float4 *>(vref + 3 * CH_N + (tid & 7) * 8 + 4);
     }
-    // forward-like tile (m, n), n <= m: rows s = 16 n + 4 kg + j, column t = 16 m + i, kept for s < t;
-    // backward-like tile (n, m), m >= n: rows t = 16 m + 4 kg + j, column s = 16 n + i, kept for t > s
-    template <int SIDE> __device__ __forceinline__ uint2 *fw_tile(int m, int n) const {
-        return reinterpret_cast<uint2 *>(smem + GR_PT + SIDE * 20 * PT_TILE + (m * (m + 1) / 2 + n) * PT_TILE) + lane;
+    __device__ __forceinline__ void stage_mats(const MatRegs &r) const {
+        const float rbv[8] = {r.rb[0].x, r.rb[0].y, r.rb[0].z, r.rb[0].w, r.rb[1].x, r.rb[1].y, r.rb[1].z, r.rb[1].w};
+        const u32 sw[4] = {r.s0.x, r.s0.y, r.s0.z, r.s0.w};
+        float v[8];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            v[2 * e] = IOE::to_f32((u16)(sw[e] & 0xffffu)) * (r.ra * rbv[2 * e]);
+            v[2 * e + 1] = IOE::to_f32((u16)(sw[e] >> 16)) * (r.ra * rbv[2 * e + 1]);
+        }
+        const int o = (tid >> 3) * CMS + (tid & 7) * 8;
+        *reinterpret_cast<uint4 *>(reinterpret_cast<u16 *>(smem + GR_S0) + o) =
+            make_uint4(Bf16::pack2(v[0], v[1]), Bf16::pack2(v[2], v[3]), Bf16::pack2(v[4], v[5]), Bf16::pack2(v[6], v[7]));
+        *reinterpret_cast<uint4 *>(reinterpret_cast<u16 *>(smem + GR_GH) + o) = r.gh;
     }
-    template <int SIDE> __device__ __forceinline__ uint2 *bw_tile(int n, int m) const {
-        return reinterpret_cast<uint2 *>(smem + GR_PT + SIDE * 20 * PT_TILE + (10 + m * (m + 1) / 2 + n) * PT_TILE) + lane;
+    // Product tile (m, n), n <= m, of a side: element [t = 16 m + i][s = 16 n + 4 kg + j] in lane (i, kg),
+    // kept for s < t; that is the A operand of the forward-like sweep.  The backward-like sweep contracts
+    // over t and reads the same tile transposed.
+    template <int SIDE> __device__ __forceinline__ u16 *pt_tile(int m, int n) const {
+        return reinterpret_cast<u16 *>(smem + GR_PT + SIDE * 10 * PT_TILE + (m * (m + 1) / 2 + n) * PT_TILE);
+    }
+    template <int SIDE> __device__ __forceinline__ uint2 fw_read(int m, int n) const {
+        return reinterpret_cast<const uint2 *>(pt_tile<SIDE>(m, n))[lane];
+    }
+    // lane (i, kg) receives [t = 16 m + 4 kg + j][s = 16 n + i]: row j of that 4 x 16 block lies in the four
+    // 8-byte pieces of lanes (4 kg + j, 0 .. 3)
+    template <int SIDE> __device__ __forceinline__ uint2 bw_read(int m, int n) const {
+        const u16 *q = pt_tile<SIDE>(m, n) + 4 * (16 * (i & 3) + 4 * kg + (i >> 2));
+        return __builtin_bit_cast(uint2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_short4_ptr)(q)));
     }
     template <int SIDE> __device__ __forceinline__ float *diag() const { return reinterpret_cast<float *>(smem + GR_PD) + SIDE * CH_N; }
 
-    // phase P of one side: token column / row cb of the product
-    template <int SIDE> __device__ __forceinline__ void products() const {
-        if (cb >= NT) return;                    // wave-uniform (chunks of 32 tokens have two token tiles)
-        const u16 *const oth_adj = tile_adj<1 - SIDE>(), *const oth_val = tile_val<1 - SIDE>();
+    // phase P of one side: the ten (NT = 4) or three (NT = 2) product tiles, spread over the side's four waves
+    template <int SIDE> __device__ __forceinline__ void product_tile(int m, int n, const uint4 &w0, const uint4 &w1) const {
+        const u16 *const oth_adj = tile_adj<1 - SIDE>();
         const floatx4 zero = {0.f, 0.f, 0.f, 0.f};
-        const uint4 a0 = tok_rows_op(oth_adj, 16 * cb, 0, i, kg), a1 = tok_rows_op(oth_adj, 16 * cb, 1, i, kg);
-        const uint4 v0 = tok_rows_op(oth_val, 16 * cb, 0, i, kg), v1 = tok_rows_op(oth_val, 16 * cb, 1, i, kg);
-        {
-            const floatx4 pt = Bf16::mfma32(v1, a1, Bf16::mfma32(v0, a0, zero));             // [s][t], diagonal tile
+        const uint4 a0 = tok_rows_op(oth_adj, 16 * m, 0, i, kg), a1 = tok_rows_op(oth_adj, 16 * m, 1, i, kg);
+        const floatx4 pt = Bf16::mfma32(w1, a1, Bf16::mfma32(w0, a0, zero));             // [s][t]
+        if (m == n) {
             float dg[4];
             tile_diagonal(dg, pt, kg);
-            if (i == 0) *reinterpret_cast<float4 *>(diag<SIDE>() + 16 * cb + 4 * kg) = make_float4(dg[0], dg[1], dg[2], dg[3]);
-            *fw_tile<SIDE>(cb, cb) = mask_pack<KEEP_ROW_LT_COL>(pt, i, kg);
-            const floatx4 pb = Bf16::mfma32(a1, v1, Bf16::mfma32(a0, v0, zero));             // [t][s], diagonal tile
-            *bw_tile<SIDE>(cb, cb) = mask_pack<KEEP_ROW_GT_COL>(pb, i, kg);
+            if (i == 0) *reinterpret_cast<float4 *>(diag<SIDE>() + 16 * m + 4 * kg) = make_float4(dg[0], dg[1], dg[2], dg[3]);
+            reinterpret_cast<uint2 *>(pt_tile<SIDE>(m, n))[lane] = mask_pack<KEEP_ROW_LT_COL>(pt, i, kg);
+        } else {
+            reinterpret_cast<uint2 *>(pt_tile<SIDE>(m, n))[lane] = mask_pack<KEEP_ALL>(pt, i, kg);
         }
+    }
+    template <int SIDE> __device__ __forceinline__ void products() const {
+        const u16 *const oth_val = tile_val<1 - SIDE>();
+        // wave cb: the diagonal tile (cb, cb) and, of the others, those of token column n = cb; the last
+        // wave has only its diagonal tile in that column and takes (1, 0) over from the first
+        if (cb < NT) {
+            const uint4 w0 = tok_rows_op(oth_val, 16 * cb, 0, i, kg), w1 = tok_rows_op(oth_val, 16 * cb, 1, i, kg);
+            product_tile<SIDE>(cb, cb, w0, w1);
 #pragma unroll
-        for (int o = 0; o < NT; ++o) {
-            if (o < cb) {                        // forward-like tiles of column cb: n = o < m = cb
-                const uint4 w0 = tok_rows_op(oth_val, 16 * o, 0, i, kg), w1 = tok_rows_op(oth_val, 16 * o, 1, i, kg);
-                *fw_tile<SIDE>(cb, o) = mask_pack<KEEP_ALL>(Bf16::mfma32(w1, a1, Bf16::mfma32(w0, a0, zero)), i, kg);
-            } else if (o > cb) {                 // backward-like tiles of row cb: m = o > n = cb
-                const uint4 w0 = tok_rows_op(oth_adj, 16 * o, 0, i, kg), w1 = tok_rows_op(oth_adj, 16 * o, 1, i, kg);
-                *bw_tile<SIDE>(cb, o) = mask_pack<KEEP_ALL>(Bf16::mfma32(w1, v1, Bf16::mfma32(w0, v0, zero)), i, kg);
-            }
+            for (int m = NT - 1; m > 1; --m)
+                if (m > cb) product_tile<SIDE>(m, cb, w0, w1);
+            if (NT == 2 && cb == 0) product_tile<SIDE>(1, 0, w0, w1);
+        }
+        if (NT == 4 && cb == 3) {
+            const uint4 w0 = tok_rows_op(oth_val, 0, 0, i, kg), w1 = tok_rows_op(oth_val, 0, 1, i, kg);
+            product_tile<SIDE>(1, 0, w0, w1);
         }
     }
 
@@ -347,9 +355,11 @@ template <typename IOE, int NT, bool HEADS, bool FULL> struct GradsItem {
             own_adj = g.template tile_adj<SIDE>(); own_val = g.template tile_val<SIDE>();
             oth_adj = g.template tile_adj<1 - SIDE>(); oth_val = g.template tile_val<1 - SIDE>();
             pd = g.template diag<SIDE>();
-            d_val = reinterpret_cast<u16 *>(SIDE ? g.p.d_k : g.p.d_x);
-            d_gate = reinterpret_cast<u16 *>(SIDE ? g.p.d_f_key : g.p.d_f);
-            d_adj = reinterpret_cast<u16 *>(g.p.d_q);                  // key side only
+            // at (the lane's first token, its channel): the token offsets below are then compile-time
+            // constants of the store instructions wherever the token stride is one
+            d_val = reinterpret_cast<u16 *>(SIDE ? g.p.d_k : g.p.d_x) + g.off;
+            d_gate = reinterpret_cast<u16 *>(SIDE ? g.p.d_f_key : g.p.d_f) + g.off;
+            d_adj = reinterpret_cast<u16 *>(g.p.d_q) + g.off;          // key side only
             anchor_acc = 0.f;
         }
         // operands of the own side (this lane's channel, tokens 16 m + 4 kg + j), re-read from the own tiles
@@ -363,7 +373,7 @@ template <typename IOE, int NT, bool HEADS, bool FULL> struct GradsItem {
         __device__ __forceinline__ void store4(u16 *dst, int mm, const float (&v)[4]) const {
 #pragma unroll
             for (int j = 0; j < 4; ++j)
-                if (FULL || 16 * mm + j < g.n_left) dst[g.off + (u32)(16 * mm + j) * g.ts] = cvt1<IOE>(v[j]);
+                if (FULL || 16 * mm + j < g.n_left) dst[(16 * mm + j) * (int)g.ts] = cvt1<IOE>(v[j]);
         }
         // forward-like sweep, token tile m: o' (value side) / q' (key side)
         __device__ __forceinline__ void forward_tile(int m, const uint4 &s0a, const uint4 &s0b) {
@@ -377,7 +387,7 @@ template <typename IOE, int NT, bool HEADS, bool FULL> struct GradsItem {
             for (int j = 0; j < 4; ++j) anchor_acc += af[j] * acc[j];
 #pragma unroll
             for (int n0 = 0; n0 <= m; n0 += 2)
-                acc = Bf16::mfma32(cat(*g.template fw_tile<SIDE>(m, n0), n0 + 1 <= m ? *g.template fw_tile<SIDE>(m, n0 + 1) : none),
+                acc = Bf16::mfma32(cat(g.template fw_read<SIDE>(m, n0), n0 + 1 <= m ? g.template fw_read<SIDE>(m, n0 + 1) : none),
                                    cat(b_val(n0), n0 + 1 <= m ? b_val(n0 + 1) : none), acc);
             if (SIDE == 1) {
                 const float4 dgv = *reinterpret_cast<const float4 *>(pd + 16 * m + 4 * g.kg);
@@ -399,7 +409,7 @@ template <typename IOE, int NT, bool HEADS, bool FULL> struct GradsItem {
             floatx4 acc = Bf16::mfma32(v1, ghb, Bf16::mfma32(v0, gha, zero));
 #pragma unroll
             for (int m0 = n; m0 < NT; m0 += 2)
-                acc = Bf16::mfma32(cat(*g.template bw_tile<SIDE>(n, m0), m0 + 1 < NT ? *g.template bw_tile<SIDE>(n, m0 + 1) : none),
+                acc = Bf16::mfma32(cat(g.template bw_read<SIDE>(m0, n), m0 + 1 < NT ? g.template bw_read<SIDE>(m0 + 1, n) : none),
                                    cat(b_adj(m0), m0 + 1 < NT ? b_adj(m0 + 1) : none), acc);
             const float4 dgv = *reinterpret_cast<const float4 *>(pd + 16 * n + 4 * g.kg);
             const float dg[4] = {dgv.x, dgv.y, dgv.z, dgv.w};
@@ -469,27 +479,31 @@ template <typename IOE, int NT, bool HEADS, bool FULL> struct GradsItem {
         w.gate_gradient(diag_part);
     }
 
-    __device__ __forceinline__ void run() const {
-        SideState<NT> sv, sk;
+    template <int SIDE> __device__ __forceinline__ void run_side() const {
+        SideState<NT> st;
         {
-            Raw r0, r1;
-            issue_raw<0>(r0);
-            issue_raw<1>(r1);                    // the key side's inputs travel while the value side is prepared
-            prep<0>(sv, r0);
-            prep<1>(sk, r1);
+            Raw r;
+            MatRegs mr;
+            issue_raw<SIDE>(r);
+            issue_mats(mr);
+            prep<SIDE>(st, r);
+            stage_mats(mr);
         }
-        stage_mats();
         __syncthreads();                         // tiles, S0', Gh' complete
-        products<0>();
-        products<1>();
+        products<SIDE>();
         __syncthreads();                         // product tiles complete
-        sweeps<0>(sv);
-        sweeps<1>(sk);
+        sweeps<SIDE>(st);
+    }
+    __device__ __forceinline__ void run() const {
+        if (side == 0)                           // wave-uniform; both branches meet the same two barriers
+            run_side<0>();
+        else
+            run_side<1>();
     }
 };
 
 template <typename IOE, int NT, bool HEADS>
-__global__ __launch_bounds__(GR_THREADS, 2) void lfw_par_grads_kernel(ParBwdArgs p) {
+__global__ __launch_bounds__(GR_THREADS, 4) void lfw_par_grads_kernel(ParBwdArgs p) {
     extern __shared__ __align__(16) unsigned char smem[];
     const int64_t item = blockIdx.x;
     if ((int)(item % p.NC) * 16 * NT + 16 * NT <= (int)p.T)

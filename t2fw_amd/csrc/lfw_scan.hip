@@ -34,6 +34,12 @@ __global__ __launch_bounds__(SCAN_THREADS) void lfw_fwd_scan_kernel(ScanFwdArgs 
 // states only (16 lanes per state row, segment-start buffer).
 constexpr int ROW_SELECT_GRID = 32;
 template <typename IO, int KPL, int SIDE> __device__ __forceinline__ void bwd_scan_rows(const ScanBwdArgs &p) {
+    // The usual case is that no row is flagged: every thread looks at one of the workgroup's rows, so
+    // that the workgroup learns it with one round trip to memory instead of one per row.
+    int mine = 0;
+    for (int64_t b = blockIdx.x + (int64_t)threadIdx.x * gridDim.x; b < p.B; b += (int64_t)gridDim.x * SCAN_THREADS)
+        mine |= p.row_select[b];
+    if (!__syncthreads_or(mine)) return;
     bool first = true;
     for (int64_t b = blockIdx.x; b < p.B; b += gridDim.x) {
         if (p.row_select[b] == 0) continue;          // the same for every thread of the workgroup
@@ -116,9 +122,9 @@ int launch_bwd(ScanBwdArgs a, const ScanGeom &g, hipStream_t stream) {
     return check_hip(hipGetLastError(), "lfw_bwd_scan_kernel launch");
 }
 
-template <typename IO> int fwd_by_kpl(ScanFwdArgs a, hipStream_t stream) {
-    if (a.K > SCAN_MAX_COLS) return fail(T2FW_ERR_UNSUPPORTED, "K=%lld exceeds the supported maximum %d", (long long)a.K, SCAN_MAX_COLS);
-    const ScanGeom g = scan_geometry(a.K);
+// One pass: the key channels [a.col0, a.col0 + width) of the state.
+template <typename IO> int fwd_pass(ScanFwdArgs a, int64_t width, hipStream_t stream) {
+    const ScanGeom g = scan_geometry(width);
     a.kg = g.kg;
     int tb = 32;
     const int by_cols = PFC * SCAN_THREADS / (g.kg * g.kpl);
@@ -137,11 +143,25 @@ template <typename IO> int fwd_by_kpl(ScanFwdArgs a, hipStream_t stream) {
     return fail(T2FW_ERR_UNSUPPORTED, "unsupported columns-per-lane %d", g.kpl);
 }
 
-template <typename IO, int SIDE> int bwd_by_kpl(const ScanBwdArgs &a, hipStream_t stream) {
-    const int64_t ncols = SIDE == 0 ? a.K : a.D;
-    if (ncols > SCAN_MAX_COLS)
-        return fail(T2FW_ERR_UNSUPPORTED, "%s=%lld exceeds the supported maximum %d", SIDE == 0 ? "K" : "D", (long long)ncols, SCAN_MAX_COLS);
-    const ScanGeom g = scan_geometry(ncols);
+// A lane group holds up to SCAN_MAX_COLS columns of a state row.  Wider states run as several
+// launches, one per window of columns: the columns of the state never interact (each has its own
+// gate and its own input), and the outputs are sums over them, which the later launches add to
+// (the reference tiles K over blocks, t2fw/csrc/lfw_kernel.cu:146-155).  With 16-bit tensors the
+// sum is rounded to the tensor type once per launch.
+template <typename IO> int fwd_by_kpl(ScanFwdArgs a, hipStream_t stream) {
+    if (a.K <= SCAN_MAX_COLS) return fwd_pass<IO>(a, a.K, stream);
+    for (int64_t c0 = 0; c0 < a.K; c0 += SCAN_MAX_COLS) {
+        a.col0 = c0;
+        a.colw = a.K - c0 < SCAN_MAX_COLS ? a.K - c0 : SCAN_MAX_COLS;
+        a.accumulate = c0 > 0 ? 1 : 0;
+        const int rc = fwd_pass<IO>(a, a.colw, stream);
+        if (rc != T2FW_OK) return rc;
+    }
+    return T2FW_OK;
+}
+
+template <typename IO, int SIDE> int bwd_pass(const ScanBwdArgs &a, int64_t width, hipStream_t stream) {
+    const ScanGeom g = scan_geometry(width);
     switch (g.kpl) {
         case 1: return launch_bwd<IO, 1, SIDE>(a, g, stream);
         case 2: return launch_bwd<IO, 2, SIDE>(a, g, stream);
@@ -151,6 +171,20 @@ template <typename IO, int SIDE> int bwd_by_kpl(const ScanBwdArgs &a, hipStream_
         case 32: return launch_bwd<IO, 32, SIDE>(a, g, stream);
     }
     return fail(T2FW_ERR_UNSUPPORTED, "unsupported columns-per-lane %d", g.kpl);
+}
+
+// The reduced dimension (K on side 0, D on side 1) in windows, as for the forward.
+template <typename IO, int SIDE> int bwd_by_kpl(ScanBwdArgs a, hipStream_t stream) {
+    const int64_t ncols = SIDE == 0 ? a.K : a.D;
+    if (ncols <= SCAN_MAX_COLS || SIDE == 2) return bwd_pass<IO, SIDE>(a, ncols, stream);
+    for (int64_t c0 = 0; c0 < ncols; c0 += SCAN_MAX_COLS) {
+        a.col0 = c0;
+        a.colw = ncols - c0 < SCAN_MAX_COLS ? ncols - c0 : SCAN_MAX_COLS;
+        a.accumulate = c0 > 0 ? 1 : 0;
+        const int rc = bwd_pass<IO, SIDE>(a, a.colw, stream);
+        if (rc != T2FW_OK) return rc;
+    }
+    return T2FW_OK;
 }
 
 template <typename IO> int bwd_both(const ScanBwdArgs &a, hipStream_t stream) {

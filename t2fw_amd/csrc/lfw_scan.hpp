@@ -11,6 +11,11 @@ struct ScanFwdArgs {
     int64_t B, T, D, K, NC;
     int32_t C, kg, tb, ntiles;
     int32_t heads;                      // 1, or H: row b is head b % H of [B/H, T, H, D|K] tensors (x, f, q, k, f_key, out)
+    // One pass over the key channels [col0, col0 + colw) of a state wider than a lane group holds
+    // (colw = 0: all of them).  The state's columns never interact, and the outputs are sums over
+    // them: a pass with accumulate set adds its share to what the passes before it left in out.
+    int64_t col0, colw;
+    int32_t accumulate;
 };
 
 struct ScanBwdArgs {
@@ -20,6 +25,10 @@ struct ScanBwdArgs {
     int64_t B, T, D, K, NC;
     int32_t C, kg, use_sub, ntiles;
     int32_t heads;                      // as for the forward (inputs, g_out and the five [.., T, .., D|K] gradients)
+    // One pass over the reduced channels [col0, col0 + colw) (key channels on side 0, value channels on
+    // side 1; colw = 0: all of them); with accumulate set the pass adds to the [.., T, .., D|K] gradients.
+    int64_t col0, colw;
+    int32_t accumulate;
 };
 
 int scan_forward(const ScanFwdArgs &a, int dtype, hipStream_t stream);

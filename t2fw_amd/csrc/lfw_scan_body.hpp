@@ -30,6 +30,8 @@ __device__ __forceinline__ void fwd_scan_body_kg(const ScanFwdArgs &p, int64_t b
     Acc *outL = rowL + (size_t)tb * 2 * g.rows;          // [tb][rows]
 
     const int64_t T = p.T, D = p.D, K = p.K;
+    const int64_t col0 = p.col0, KW = p.colw > 0 ? p.colw : K;      // this pass's window of key channels
+    const bool accumulate = p.accumulate != 0;
     const int64_t line0 = row_first_token(b, T, p.heads);      // [.., D] line of this row's step 0
     const int64_t d0 = (int64_t)tile * g.rows;
     const int64_t d = d0 + g.r;
@@ -43,10 +45,21 @@ __device__ __forceinline__ void fwd_scan_body_kg(const ScanFwdArgs &p, int64_t b
     Acc S[KPL];
 #pragma unroll
     for (int j = 0; j < KPL; ++j)
-        S[j] = (row_ok && g.k0 + j < K) ? to_acc(s0[(b * D + d) * K + g.k0 + j]) : Acc(0);
+        S[j] = (row_ok && g.k0 + j < KW) ? to_acc(s0[(b * D + d) * K + col0 + g.k0 + j]) : Acc(0);
+
+    // outputs of a block of steps: written, or added to what the passes over other key channels left
+    auto flush = [&](int n_blk, int64_t t_blk) {
+        for (int idx = threadIdx.x; idx < n_blk * g.rows; idx += SCAN_THREADS) {
+            const int tt = idx / g.rows, rr = idx % g.rows;
+            if (d0 + rr < D) {
+                IO *const o = out + (line0 + (t_blk + tt) * p.heads) * D + d0 + rr;
+                *o = from_acc<IO>(accumulate ? to_acc(*o) + outL[idx] : outL[idx]);
+            }
+        }
+    };
 
     Prefetch<IO, 3, 2> pf;
-    block_load(pf, g, colp, rowp, b, T, 0, (int)(T < tb ? T : tb), K, D, d0, p.heads);
+    block_load(pf, g, colp, rowp, b, T, 0, (int)(T < tb ? T : tb), K, D, d0, p.heads, col0, p.colw);
 
     int until_ckpt = 0;          // steps until the next checkpoint is due
     int64_t chunk = 0;
@@ -56,15 +69,12 @@ __device__ __forceinline__ void fwd_scan_body_kg(const ScanFwdArgs &p, int64_t b
         const int n = (int)(T - t0 < tb ? T - t0 : tb);
         __syncthreads();                                   // previous block fully consumed
         // flush the previous block's outputs, then publish this block's inputs
-        for (int idx = threadIdx.x; idx < n_prev * g.rows; idx += SCAN_THREADS) {
-            const int tt = idx / g.rows, rr = idx % g.rows;
-            if (d0 + rr < D) out[(line0 + (t_prev + tt) * p.heads) * D + d0 + rr] = from_acc<IO>(outL[idx]);
-        }
+        flush(n_prev, t_prev);
         block_store<IO, Acc, 3, 2>(pf, g, colL, rowL, tb);
         __syncthreads();
         if (t0 + tb < T) {
             const int64_t tn = t0 + tb;
-            block_load(pf, g, colp, rowp, b, T, tn, (int)(T - tn < tb ? T - tn : tb), K, D, d0, p.heads);
+            block_load(pf, g, colp, rowp, b, T, tn, (int)(T - tn < tb ? T - tn : tb), K, D, d0, p.heads, col0, p.colw);
         }
 #pragma unroll 4
         for (int tt = 0; tt < n; ++tt) {
@@ -73,8 +83,8 @@ __device__ __forceinline__ void fwd_scan_body_kg(const ScanFwdArgs &p, int64_t b
                     if (row_ok) {
 #pragma unroll
                         for (int j = 0; j < KPL; ++j)
-                            if (g.k0 + j < K)
-                                ckpt[((b * p.NC + chunk) * D + d) * K + g.k0 + j] = from_acc<IO>(S[j]);
+                            if (g.k0 + j < KW)
+                                ckpt[((b * p.NC + chunk) * D + d) * K + col0 + g.k0 + j] = from_acc<IO>(S[j]);
                     }
                     until_ckpt = p.C;
                     ++chunk;
@@ -99,14 +109,11 @@ __device__ __forceinline__ void fwd_scan_body_kg(const ScanFwdArgs &p, int64_t b
         t_prev = t0;
     }
     __syncthreads();
-    for (int idx = threadIdx.x; idx < n_prev * g.rows; idx += SCAN_THREADS) {
-        const int tt = idx / g.rows, rr = idx % g.rows;
-        if (d0 + rr < D) out[(line0 + (t_prev + tt) * p.heads) * D + d0 + rr] = from_acc<IO>(outL[idx]);
-    }
+    flush(n_prev, t_prev);
     if (row_ok) {
 #pragma unroll
         for (int j = 0; j < KPL; ++j)
-            if (g.k0 + j < K) next_state[(b * D + d) * K + g.k0 + j] = from_acc<IO>(S[j]);
+            if (g.k0 + j < KW) next_state[(b * D + d) * K + col0 + g.k0 + j] = from_acc<IO>(S[j]);
     }
 }
 
@@ -152,6 +159,8 @@ __device__ __forceinline__ void bwd_scan_body_kg(const ScanBwdArgs &p, int64_t b
     const int64_t T = p.T;
     const int64_t line0 = row_first_token(b, T, p.heads);      // [.., D|K] line of this row's step 0
     const int64_t nrows = SIDE == 0 ? p.D : p.K, ncols = SIDE == 0 ? p.K : p.D;
+    const int64_t col0 = p.col0, colw = p.colw > 0 ? p.colw : ncols;      // this pass's window of the reduced channels
+    const bool accumulate = p.accumulate != 0;
     const int64_t row0 = (int64_t)tile * g.rows;
     const int64_t row = row0 + g.r;
     const bool row_ok = row < nrows;
@@ -168,9 +177,9 @@ __device__ __forceinline__ void bwd_scan_body_kg(const ScanBwdArgs &p, int64_t b
 
     // element offset of (row, col0 + j) inside one [D,K] state
     auto st_off = [&](int j) -> int64_t {
-        return SIDE == 0 ? row * p.K + (g.k0 + j) : (int64_t)(g.k0 + j) * p.K + row;
+        return SIDE == 0 ? row * p.K + (col0 + g.k0 + j) : (col0 + g.k0 + j) * p.K + row;
     };
-    auto el_ok = [&](int j) -> bool { return row_ok && g.k0 + j < ncols; };
+    auto el_ok = [&](int j) -> bool { return row_ok && g.k0 + j < colw; };
 
     Acc G[KPL];
     {
@@ -251,9 +260,16 @@ __device__ __forceinline__ void bwd_scan_body_kg(const ScanBwdArgs &p, int64_t b
             const int tt = idx / g.rows, rr = idx % g.rows;
             if (row0 + rr < nrows) {
                 const int64_t o = (line0 + (t0 + tt) * p.heads) * nrows + row0 + rr;
-                d_a[o] = from_acc<IO>(outL[(tt * 3 + 0) * g.rows + rr]);
-                d_gate[o] = from_acc<IO>(outL[(tt * 3 + 1) * g.rows + rr]);
-                if (SIDE == 1) d_u[o] = from_acc<IO>(outL[(tt * 3 + 2) * g.rows + rr]);
+                Acc va = outL[(tt * 3 + 0) * g.rows + rr], vg = outL[(tt * 3 + 1) * g.rows + rr];
+                Acc vu = SIDE == 1 ? outL[(tt * 3 + 2) * g.rows + rr] : Acc(0);
+                if (accumulate) {            // the passes over other reduced channels came first
+                    va += to_acc(d_a[o]);
+                    vg += to_acc(d_gate[o]);
+                    if (SIDE == 1) vu += to_acc(d_u[o]);
+                }
+                d_a[o] = from_acc<IO>(va);
+                d_gate[o] = from_acc<IO>(vg);
+                if (SIDE == 1) d_u[o] = from_acc<IO>(vu);
             }
         }
     };
@@ -267,7 +283,7 @@ __device__ __forceinline__ void bwd_scan_body_kg(const ScanBwdArgs &p, int64_t b
             const int len = chunk_len(c), nseg = (len + SEG - 1) / SEG;
             const int sg = q < nseg - 1 ? q : 2 * nseg - 2 - q;
             const int n = q < nseg - 1 ? SEG : (len - sg * SEG < SEG ? len - sg * SEG : SEG);
-            block_load<SEG>(pf, g, colp, rowp, b, T, c * C + (int64_t)sg * SEG, n, ncols, nrows, row0, p.heads);
+            block_load<SEG>(pf, g, colp, rowp, b, T, c * C + (int64_t)sg * SEG, n, ncols, nrows, row0, p.heads, col0, p.colw);
         };
         Acc Snext[KPL];                      // checkpoint of the chunk that comes next
         load_ckpt(Snext, p.NC - 1);
@@ -309,12 +325,12 @@ __device__ __forceinline__ void bwd_scan_body_kg(const ScanBwdArgs &p, int64_t b
                 Acc st[SEG + 1][KPL];
                 load_ckpt(st[0], c);
                 for (int s2 = 0; s2 < s; ++s2) {
-                    block_load<SEG>(pf, g, colp, rowp, b, T, tc0 + (int64_t)s2 * SEG, SEG, ncols, nrows, row0, p.heads);
+                    block_load<SEG>(pf, g, colp, rowp, b, T, tc0 + (int64_t)s2 * SEG, SEG, ncols, nrows, row0, p.heads, col0, p.colw);
                     stage();
                     advance(st[0]);
                 }
                 const int n = len - s * SEG < SEG ? len - s * SEG : SEG;
-                block_load<SEG>(pf, g, colp, rowp, b, T, tc0 + (int64_t)s * SEG, n, ncols, nrows, row0, p.heads);
+                block_load<SEG>(pf, g, colp, rowp, b, T, tc0 + (int64_t)s * SEG, n, ncols, nrows, row0, p.heads, col0, p.colw);
                 stage();
                 reverse_segment(st, n, tc0 + (int64_t)s * SEG);
             }

@@ -49,11 +49,14 @@ __device__ __forceinline__ void block_load(Prefetch<IO, NCA, NRA> &pf, const Til
                                            const IO *const (&colp)[NCA],
                                            const IO *const (&rowp)[NRA],
                                            int64_t b, int64_t T, int64_t t0, int n,
-                                           int64_t ncols, int64_t nrows, int64_t row0, int64_t heads = 1) {
+                                           int64_t ncols, int64_t nrows, int64_t row0, int64_t heads = 1,
+                                           int64_t col0 = 0, int64_t colw = 0) {
+    // col0, colw: the window of the column arrays this pass works on (colw = 0: all ncols columns)
     const int csub = threadIdx.x % g.CW, tsub = threadIdx.x / g.CW;
     const int64_t line0 = row_first_token(b, T, heads) + t0 * heads;      // [.., width] line of step t0
     const int64_t cstep = heads * ncols, rstep = heads * nrows;           // elements between consecutive steps
-    const int64_t cbase = line0 * ncols;
+    const int64_t cbase = line0 * ncols + col0;
+    if (colw > 0) ncols = colw;
 #pragma unroll
     for (int m = 0; m < PFC; ++m) {
         if (g.SP * (m >> g.lncc) >= TMAX) continue;

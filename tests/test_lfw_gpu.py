@@ -146,20 +146,16 @@ def test_wide_states_every_lane_geometry(dtype, shape):
     check_all((x, f, q, k, fk, s), go, gs, dtype)
 
 
-def test_too_wide_for_training_is_refused_in_the_forward():
-    """D above the exact backward's limit: refused when the forward is asked for checkpoints, not
-    later in backward(); the same shape runs without them."""
-    from t2fw.functional_lfw import LFWFunction
-    x, f, q, k, fk, s, go, gs = make_config_inputs(1, 3, 2100, 2, torch.float32, seed=6, in_scale=0.5,
-                                                    gate_mean=1.0, state_std=0.5)
-    ins = [t.cuda() for t in (x, f, q, k, fk, s)]
-    with torch.no_grad():
-        out, nxt = LFWFunction.apply(*ins)
-    r_out, r_nxt = c_oracle.lfw_forward(x, f, q, k, fk, s)
-    assert_close(out, r_out, torch.float32, "outputs")
-    assert_close(nxt, r_nxt, torch.float32, "next_state")
-    with pytest.raises(RuntimeError, match="exact kernels take K <= 2048"):
-        LFWFunction.apply(*[t.requires_grad_(True) for t in ins])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+@pytest.mark.parametrize("shape", [(1, 5, 3, 5000), (1, 5, 5000, 3), (2, 9, 2, 2049), (1, 4, 2100, 2500)])
+def test_states_wider_than_a_lane_group_run_in_column_passes(dtype, shape):
+    """More than 2048 columns on either side (the reference tiles K over blocks,
+    t2fw/csrc/lfw_kernel.cu:146-155): several launches, each over a window of columns, the later ones
+    adding to the outputs.  16-bit outputs are rounded once per launch, hence the scale."""
+    B, T, D, K = shape
+    x, f, q, k, fk, s, go, gs = make_config_inputs(B, T, D, K, dtype, seed=13, in_scale=0.5,
+                                                    gate_mean=1.0, state_std=0.5, gstate_std=0.5)
+    check_all((x, f, q, k, fk, s), go, gs, dtype, scale=1.0 if dtype == torch.float32 else 3.0)
 
 
 @pytest.mark.parametrize("C", [1, 7, 16, 64, 100, 1000])
