@@ -5,9 +5,9 @@
 //   qs_t = q_t*b_t   kt_t = k_t/b_t   xt_t = x_t/a_t   gs_t = g_t*a_t
 // everything inside a chunk is a dense contraction of those four [CL, 64] tiles with each other,
 // with the chunk-start state S0 (the checkpoint) and with the adjoint entering the chunk from the
-// future (lfw_par_bwd.hip, lfw_par_fwd.hip).  Only the chunk-to-chunk hand-over of the state (forward)
-// and of the adjoint (backward) is sequential; it is a light pass of its own that reads four of the
-// inputs, and the rest runs as one workgroup per (batch row, chunk) over the whole grid.
+// future (lfw_par_bwd.hip).  Only the chunk-to-chunk hand-over of the adjoint is sequential; its
+// per-chunk increments are a light pass of their own that reads four of the inputs, the hand-over
+// itself is elementwise, and the rest runs as one workgroup per (batch row, chunk) over the whole grid.
 //
 // Range: the scalings are taken relative to the MIDDLE of the chunk (a'_t = a_t / a_mid, likewise
 // b'), so that 1/a'_t and a'_t each grow over half a chunk only: the form needs the gate products of
@@ -37,7 +37,7 @@ namespace t2fw {
 // Backward, three launches: the adjoint's per-chunk increments sum_t gs_t (x) qs_t and gate products
 // (one workgroup per (row, chunk)); their scan over the chunks of a row, last to first, which leaves
 // the adjoint entering every chunk (Gh', bf16) in place of the increments and writes d_s0 (elementwise,
-// one workgroup per row); and the gradients (one workgroup per (row, chunk)).
+// eight workgroups per row); and the gradients (one workgroup per (row, chunk)).
 constexpr int PAR_NVEC = 6;            // per (row, chunk): totA, totB, refA, refB, sfxA, sfxB, [64] floats each
 struct ParBwdArgs {
     const void *g_out, *g_state, *x, *f, *q, *k, *f_key, *ckpt;
@@ -51,18 +51,7 @@ struct ParBwdArgs {
     int32_t heads;                     // as in ChunkFwdArgs
 };
 
-// Forward, two launches: the state hand-over (one workgroup per batch row, writes the checkpoints
-// and the final state) and the outputs (one workgroup per (row, chunk)).
-struct ParFwdArgs {
-    const void *x, *f, *q, *k, *f_key, *s0;
-    void *out, *next_state, *ckpt;     // ckpt [B, NC, 64, 64] in the tensors' dtype (the caller's, or scratch)
-    int32_t *row_flags;
-    int64_t B, T, NC;
-    int32_t C, heads;
-};
-
 int par_backward(const ParBwdArgs &a, int dtype, hipStream_t stream);
-int par_forward(const ParFwdArgs &a, int dtype, hipStream_t stream);
 
 #if defined(__HIPCC__)
 namespace par {

@@ -23,7 +23,7 @@
 //
 // Launch 1 (lfw_par_incr_kernel, one workgroup per (row, chunk)): the chunk's increment of the adjoint,
 // sum_t gs_t (x) qs_t with prefixes from the chunk START (factors <= 1), as bf16, and the chunk's
-// gate products.  Launch 2 (lfw_par_scan_kernel, elementwise, 32 workgroups per row): the
+// gate products.  Launch 2 (lfw_par_scan_kernel, elementwise, eight workgroups per row): the
 // adjoint chain over the chunks of a row, last to first, in fp32; it overwrites every increment
 // with the Gh of its chunk (bf16, the type the third launch feeds to the matrix cores) and writes
 // d_s0.  Launch 3 (lfw_par_grads_kernel, one workgroup per (row, chunk)) computes everything else.
@@ -185,18 +185,18 @@ template <typename IOE> __global__ __launch_bounds__(SCAN_TPB) void lfw_par_scan
 }
 
 // ---- launch 3: gradients --------------------------------------------------------------------------
-// One workgroup of 4 waves per (row, chunk) item; wave cb owns channel block cb of BOTH sides (first the
-// value side, then the key side in every phase): lane (i, kg) owns channel 16 cb + i and the tokens
-// 16 m + 4 kg + j (m < NT, j < 4) of the chunk.  Two such workgroups fit a compute unit (LDS, 256
-// registers per lane) and run independently of each other, so the memory latency and the barrier
-// waits of one are filled with the other's work.
+// One workgroup of 8 waves per (row, chunk) item; wave (side, cb) owns channel block cb of its side:
+// lane (i, kg) owns channel 16 cb + i and the tokens 16 m + 4 kg + j (m < NT, j < 4) of the chunk.
+// Two such workgroups fit a compute unit (LDS; 128 registers per lane, four waves per SIMD) and run
+// independently of each other, so the memory latency and the barrier waits of one are filled with
+// the other's work.
 //   A  raw inputs (2-byte loads, a token row of a channel block = 32 contiguous bytes) -> gate products
 //      relative to the middle of the chunk -> scaled operands -> channel-major tiles; the
 //      chunk-start state (scaled, as bf16) and Gh' go to LDS                              | barrier
 //   P  the token x token products of a side (P for the value side, W for the key side) are the same
-//      for all channel blocks: wave cb computes the tiles of token column cb (forward-like
-//      orientation) and of token row cb (backward-like orientation), 5 of the 20 tiles per side,
-//      masks them and leaves them in LDS as ready 16-bit A operands, plus the diagonal    | barrier
+//      for all channel blocks: the side's four waves share its ten 16 x 16 tiles (s <= t), mask
+//      them and leave them in LDS as ready 16-bit A operands of the forward-like sweep, plus the
+//      diagonal; the backward-like sweep reads the same tiles transposed                  | barrier
 //   S  per side: forward-like sweep (o' / q'), backward-like sweep (x' / k'), gate gradient; the
 //      results go to global memory from the accumulator layout
 constexpr int GR_THREADS = 512;
