@@ -9,12 +9,15 @@ What it follows in the reference (paths relative to the reference tree):
 * ``dfw_backward_two_pass``  -> t2fw/torch.py:59-145 (``t2dfw_torch_bw``) = the two reverse
                                 passes of t2fw/csrc/dfw_kernel.cu:250-276 (d_value, d_state)
                                 and :345-383 (d_query, d_key with the state walked backwards)
+* ``dfw_backward_one_pass``  -> t2fw/torch.py:148-242 (``t2dfw_torch_bw_simple``): the overwritten values
+                                S_{t-1} k_t recomputed by a forward sweep, then all four gradients
+                                in one reverse sweep from the final state
 * ``dfw_deltas``             -> the ``delta_value`` tensor the forward kernel emits
                                 (t2fw/csrc/dfw_kernel.cu:176-183), which the backward consumes
 
 Pinning (tests/test_oracle_dfw.py): closed forms (zero keys, single step, unit-norm key
 retrieval S_t k_t = v_t, orthonormal keys), ``torch.autograd`` through the restated forward
-vs the two-pass backward, ``gradcheck``, segment composition, linearity in (v, S_0).
+vs the two-pass and the one-pass backward, ``gradcheck``, segment composition, linearity in (v, S_0).
 The reference holds no stored vectors for this path (tests/test_dfw.py:30-60 draws random
 tensors at run time).
 """
@@ -80,3 +83,31 @@ def dfw_backward_two_pass(grad_output, grad_state, query, key, delta, final_stat
         d_k[:, t] = (G * delta[:, t, :, None]).sum(1) - (S * d_v[:, t, :, None]).sum(1)
         G = G - d_v[:, t, :, None] * key[:, t, None, :] + grad_output[:, t, :, None] * query[:, t, None, :]
     return d_q, d_k, d_v, d_state
+
+
+def dfw_backward_one_pass(grad_output, grad_state, query, key, value, state, final_state):
+    """The reference's second derivation (t2fw/torch.py:148-242): a forward sweep recomputes the
+    value each step overwrote, old_t = S_{t-1} k_t (torch.py:159-168); one reverse sweep then walks
+    the state back from ``final_state`` and carries the adjoint G.  Returns (d_q, d_k, d_v, d_state)."""
+    B, T, D = value.shape
+    olds = []
+    s = state
+    for t in range(T):                                               # torch.py:159-168
+        old = (s * key[:, t, None, :]).sum(-1)
+        s = s + (value[:, t] - old)[:, :, None] * key[:, t, None, :]
+        olds.append(old)
+    d_q, d_k, d_v = torch.zeros_like(query), torch.zeros_like(key), torch.zeros_like(value)
+    G = grad_state.clone()
+    S = final_state.clone()
+    for t in range(T - 1, -1, -1):                                   # torch.py:178-233
+        k, v, g = key[:, t], value[:, t], grad_output[:, t]
+        Gk = (G * k[:, None, :]).sum(-1)                             # [B, D]
+        d_v[:, t] = Gk                                               # torch.py:186
+        S = S - (v - olds[t])[:, :, None] * k[:, None, :]            # S_{t-1}, torch.py:190
+        a = (G * v[:, :, None]).sum(1)                               # G^T v       torch.py:217
+        c = (G * olds[t][:, :, None]).sum(1)                         # G^T old     torch.py:219
+        b = (S * Gk[:, :, None]).sum(1)                              # S_{t-1}^T G k   torch.py:221
+        d_k[:, t] = a - (b + c)
+        G = G - Gk[:, :, None] * k[:, None, :] + g[:, :, None] * query[:, t, None, :]   # torch.py:227-230
+        d_q[:, t] = (S * g[:, :, None]).sum(1)                       # torch.py:234
+    return d_q, d_k, d_v, G

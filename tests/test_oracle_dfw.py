@@ -78,6 +78,22 @@ def test_two_pass_backward_matches_autograd(shape):
         assert torch.allclose(a, m, atol=1e-11)
 
 
+@pytest.mark.parametrize("shape", [(2, 5, 3, 4), (1, 1, 1, 1), (3, 7, 4, 2), (2, 6, 1, 5)])
+def test_one_pass_backward_matches_autograd_and_the_two_pass_form(shape):
+    """the reference's second derivation (t2fw/torch.py:148-242): a dropped term or a state that is not
+    walked back before use shows against either of the other two"""
+    from oracle.dfw_ref import dfw_backward_one_pass
+    B, T, D, M = shape
+    q, k, v, s = small(B, T, D, M, seed=11)
+    go, gs = rnd(B, T, D, seed=72), rnd(B, D, M, seed=73)
+    out, fin, auto = dfw_reference_grads(q, k, v, s, go, gs)
+    one = dfw_backward_one_pass(go, gs, q, k, v, s, fin)
+    two = dfw_backward_two_pass(go, gs, q, k, dfw_deltas(q, k, v, s), fin)
+    for a, m, w in zip(auto, one, two):
+        assert torch.allclose(a, m, atol=1e-11)
+        assert torch.allclose(m, w, atol=1e-11)
+
+
 def test_gradcheck_finite_differences():
     ins = [t.clone().requires_grad_(True) for t in small(B=1, T=3, D=2, M=3, seed=21)]
     assert torch.autograd.gradcheck(dfw_reference, ins, eps=1e-6, atol=1e-6)
