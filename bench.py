@@ -205,6 +205,7 @@ def main():
     if backward and not H:
         from t2fw.functional_lfw import LFWFunction
         os.environ["T2FW_CKPT_INTERVAL"] = str(C)
+        os.environ["T2FW_FLAGS"] = str(flags)          # the same kernel path as the C-ABI legs above
         leaves = [[t.detach().clone().requires_grad_(True) for t in d["ins"]] for d in sets[:2]]
 
         def astep(i):

@@ -32,8 +32,8 @@
  *     ckpt[b, 0] == s0[b].  It replaces the reference's [B, T, D, K] "ckpt_states"
  *     (lfw_kernel.cu:140-144), which stores every step.
  *   - The library owns no memory and keeps no state between calls.  Scratch space is
- *     passed by the caller (`workspace`, size from the *_workspace_bytes query; may be
- *     NULL when the query returns 0).
+ *     passed by the caller (`workspace`, size from the *_workspace_bytes query, 16-byte
+ *     aligned, no initialisation needed; may be NULL when the query returns 0).
  *   - `stream` is a hipStream_t (NULL = the null stream).  Launches are asynchronous;
  *     the current HIP device must be the one that owns the pointers.
  *   - Every function returns 0 on success, otherwise one of T2FW_ERR_* ; a message for
@@ -78,13 +78,18 @@ extern "C" {
 #define T2FW_FLAG_NO_FIXUP 4      /* matrix-core path: do not redo what it flagged with the exact
                                      recurrence (the forward redoes it inside its kernel, the
                                      backward with one more launch); the caller reads the flags
-                                     from the workspace (int32 [2][B rounded up to 8], nonzero in
-                                     either slot = that row's results are not valid) and redoes
-                                     those rows with T2FW_FLAG_FORCE_SCAN, or knows its gates are
-                                     in range.  Saves the backward's extra launch.              */
+                                     from the workspace (nonzero = that row's results are not
+                                     valid: int32 [2][B rounded up to 8] at its start for the
+                                     forward and the block-wise backward, either slot; int32 [B]
+                                     in the next 256-byte aligned region for the chunk-parallel
+                                     backward) and redoes those rows with T2FW_FLAG_FORCE_SCAN,
+                                     or knows its gates are in range.  Saves the backward's extra
+                                     launch.                                                      */
 
-#define T2FW_FLAG_BLOCKWISE 8     /* matrix-core path: the block-wise kernels (16-step blocks, one or two
-                                     workgroups per batch row) instead of the chunk-parallel ones    */
+#define T2FW_FLAG_BLOCKWISE 8     /* matrix-core path, backward: the block-wise kernel (16-step blocks in one
+                                     pass per batch row; takes 16-step gate products down to 2^-100)
+                                     instead of the chunk-parallel ones (every chunk of every row at once;
+                                     gate products over half a chunk down to 2^-80)                  */
 
 int t2fw_abi_version(void);
 const char *t2fw_last_error(void);
@@ -93,8 +98,8 @@ const char *t2fw_last_error(void);
 int64_t t2fw_lfw_num_ckpt(int64_t T, int32_t C);
 
 /* Bytes of caller-provided scratch that serve both the forward and the backward call of a
- * shape (0 = none): row flags, and for the chunk-parallel backward kernels the adjoint entering
- * every chunk, [B, NC, D, K] bf16. */
+ * shape (0 = none): row flags, and for the chunk-parallel backward kernels per chunk its flag,
+ * six [64] fp32 gate-product vectors and the adjoint entering it, [B, NC, 64, 64] bf16. */
 size_t t2fw_lfw_workspace_bytes(int64_t B, int64_t T, int64_t D, int64_t K,
                                 int32_t C, int32_t dtype, int32_t flags);
 /* The same for a caller that only runs the forward call. */

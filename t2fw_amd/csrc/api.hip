@@ -228,6 +228,7 @@ static int lfw_forward_rows(const void *x, const void *f, const void *q, const v
         const size_t need = forward_workspace_bytes(B, D, K, dtype, flags);
         if (workspace == nullptr || workspace_bytes < need)
             return fail(T2FW_ERR_WORKSPACE, "workspace of %zu bytes needed, %zu given", need, workspace_bytes);
+        if (!aligned16({workspace})) return fail(T2FW_ERR_MISALIGNED, "the workspace must be 16-byte aligned");
         ChunkFwdArgs c{};
         c.x = x; c.f = f; c.q = q; c.k = k; c.f_key = f_key; c.s0 = s0;
         c.out = out; c.next_state = next_state; c.ckpt = ckpt;
@@ -327,6 +328,7 @@ static int lfw_backward_rows(const void *g_out, const void *g_state, const void 
         const size_t need = backward_workspace_bytes(B, T, D, K, C, dtype, flags);
         if (workspace == nullptr || workspace_bytes < need)
             return fail(T2FW_ERR_WORKSPACE, "workspace of %zu bytes needed, %zu given", need, workspace_bytes);
+        if (!aligned16({workspace})) return fail(T2FW_ERR_MISALIGNED, "the workspace must be 16-byte aligned");
         ChunkBwdArgs c{};
         c.g_out = g_out; c.g_state = g_state; c.x = x; c.f = f; c.q = q; c.k = k; c.f_key = f_key; c.ckpt = ckpt;
         c.d_x = d_x; c.d_f = d_f; c.d_q = d_q; c.d_k = d_k; c.d_f_key = d_f_key; c.d_s0 = d_s0;

@@ -5,7 +5,7 @@ and the final state saved by forward (t2fw/functional_dfw.py:46-51)."""
 import torch
 
 from . import _lib
-from .functional_lfw import _check_input, _dtype_code
+from .functional_lfw import _check_input, _dtype_code, _on_device
 
 
 class DFWFunction(torch.autograd.Function):
@@ -32,7 +32,7 @@ class DFWFunction(torch.autograd.Function):
         code = _dtype_code(value.dtype)
         lib = _lib.load()
         dev = value.device
-        with torch.cuda.device(dev):
+        with _on_device(dev):
             outputs = torch.empty_like(value)
             final_state = torch.empty_like(state)
             delta = torch.empty_like(value)
@@ -54,7 +54,7 @@ class DFWFunction(torch.autograd.Function):
         M = query.shape[2]
         lib = _lib.load()
         dev = delta.device
-        with torch.cuda.device(dev):
+        with _on_device(dev):
             d_q, d_k = torch.empty_like(query), torch.empty_like(key)
             d_v, d_s = torch.empty_like(delta), torch.empty_like(final_state)
             _lib.check(lib.t2fw_dfw_backward(

@@ -9,6 +9,8 @@ Differences from the reference that a caller can observe:
   * bf16 is accepted in addition to fp64/fp32/fp16.
   * kernels run on the current torch stream and on the inputs' device.
 """
+import contextlib
+import functools
 import os
 
 import torch
@@ -29,6 +31,22 @@ def _flags():
     Overridable with T2FW_FLAGS."""
     v = os.environ.get("T2FW_FLAGS")
     return int(v) if v else _lib.FLAG_AUTO
+
+
+@functools.lru_cache(maxsize=256)
+def _sizes(rows, T, D, K, C, code, flags):
+    """(checkpoints per row, forward workspace bytes, forward + backward workspace bytes) of a shape:
+    three calls into the library that a training loop would otherwise repeat every step"""
+    lib = _lib.load()
+    return (lib.t2fw_lfw_num_ckpt(T, C), lib.t2fw_lfw_forward_workspace_bytes(rows, T, D, K, C, code, flags),
+            lib.t2fw_lfw_workspace_bytes(rows, T, D, K, C, code, flags))
+
+
+def _on_device(dev):
+    """Make ``dev`` current for the allocations and the launch, without the cost of switching when it already is."""
+    if dev.index is None or dev.index == torch.cuda.current_device():
+        return contextlib.nullcontext()
+    return torch.cuda.device(dev)
 
 
 def _check_input(t, name):
@@ -78,14 +96,13 @@ def _lfw_forward(value, forget, query, key, f_key, state, need_grad, heads=False
     C = _ckpt_interval()
     flags = _flags()
     dev = value.device
-    with torch.cuda.device(dev):
+    nc, ws_bytes, _ = _sizes(B * H, T, D, K, C, code, flags)
+    with _on_device(dev):
         outputs = torch.empty_like(value)
         next_state = torch.empty_like(state)
         ckpt = None
         if need_grad:
-            nc = lib.t2fw_lfw_num_ckpt(T, C)
             ckpt = torch.empty((B * H, nc, D, K), dtype=value.dtype, device=dev)
-        ws_bytes = lib.t2fw_lfw_forward_workspace_bytes(B * H, T, D, K, C, code, flags)
         ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev) if ws_bytes else None
         ptrs = (_lib.ptr(value), _lib.ptr(forget), _lib.ptr(query), _lib.ptr(key), _lib.ptr(f_key),
                 _lib.ptr(state), _lib.ptr(outputs), _lib.ptr(next_state), _lib.ptr(ckpt))
@@ -110,14 +127,14 @@ def _lfw_backward(grad_output, grad_state, value, forget, query, key, f_key, sta
     code = _dtype_code(value.dtype)
     lib = _lib.load()
     dev = value.device
-    with torch.cuda.device(dev):
+    ws_bytes = _sizes(B * H, T, D, K, C, code, flags)[2]
+    with _on_device(dev):
         d_x = torch.empty_like(value)
         d_f = torch.empty_like(forget)
         d_q = torch.empty_like(query)
         d_k = torch.empty_like(key)
         d_fk = torch.empty_like(f_key)
         d_s = torch.empty_like(state)
-        ws_bytes = lib.t2fw_lfw_workspace_bytes(B * H, T, D, K, C, code, flags)
         ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev) if ws_bytes else None
         ptrs = (_lib.ptr(grad_output), _lib.ptr(grad_state), _lib.ptr(value), _lib.ptr(forget),
                 _lib.ptr(query), _lib.ptr(key), _lib.ptr(f_key), _lib.ptr(state), _lib.ptr(ckpt),
@@ -159,7 +176,7 @@ def sigmoid_gates(f_logit, fk_logit, out_f=None, out_fk=None):
     assert f_logit.dtype == fk_logit.dtype
     lib = _lib.load()
     dev = f_logit.device
-    with torch.cuda.device(dev):
+    with _on_device(dev):
         f = torch.empty_like(f_logit) if out_f is None else out_f
         fk = torch.empty_like(fk_logit) if out_fk is None else out_fk
         _lib.check(lib.t2fw_gate_forward(_lib.ptr(f_logit), _lib.ptr(fk_logit), _lib.ptr(f), _lib.ptr(fk),
@@ -172,7 +189,7 @@ def _gate_backward_inplace(d_f, d_fk, forget, f_key):
     """d_f, d_fk: gate gradients on entry, logit gradients d_gate * gate * (1 - gate) on return."""
     lib = _lib.load()
     dev = d_f.device
-    with torch.cuda.device(dev):
+    with _on_device(dev):
         _lib.check(lib.t2fw_gate_backward(_lib.ptr(d_f), _lib.ptr(d_fk), _lib.ptr(forget), _lib.ptr(f_key),
                                           _lib.ptr(d_f), _lib.ptr(d_fk), d_f.numel(), d_fk.numel(),
                                           _dtype_code(d_f.dtype), _lib.current_stream_handle(dev)))
@@ -258,7 +275,7 @@ def lfw_step(x, f, query, key, f_key, state, out=None, inplace=True):
     assert key.shape == query.shape and f_key.shape == query.shape
     lib = _lib.load()
     dev = x.device
-    with torch.cuda.device(dev):
+    with _on_device(dev):
         if out is None:
             out = torch.empty_like(x)
         nxt = state if inplace else torch.empty_like(state)
