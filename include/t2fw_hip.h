@@ -75,9 +75,10 @@ extern "C" {
 #define T2FW_FLAG_FP16_OPERANDS 2 /* fp16 tensors: fp16 (not bf16) matrix-core operands;
                                      more mantissa, but rows whose 16-step gate products
                                      fall below 2^-8 take the exact scan path          */
-#define T2FW_FLAG_NO_FIXUP 4      /* matrix-core path: do not redo what it flagged with the exact
-                                     recurrence (the forward redoes it inside its kernel, the
-                                     backward with one more launch); the caller reads the flags
+#define T2FW_FLAG_NO_FIXUP 4      /* matrix-core path: do not redo what it flagged (the forward redoes it
+                                     with the exact recurrence inside its kernel; the backward with one
+                                     more launch of the block-wise kernel, which in turn redoes exactly
+                                     what it cannot take); the caller reads the flags
                                      from the workspace (nonzero = that row's results are not
                                      valid: int32 [2][B rounded up to 8] at its start for the
                                      forward and the block-wise backward, either slot; int32 [B]

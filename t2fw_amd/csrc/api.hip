@@ -318,7 +318,6 @@ static int lfw_backward_rows(const void *g_out, const void *g_state, const void 
     ScanBwdArgs a{};
     a.g_out = g_out; a.g_state = g_state; a.x = x; a.f = f; a.q = q; a.k = k; a.f_key = f_key; a.ckpt = ckpt;
     a.d_x = d_x; a.d_f = d_f; a.d_q = d_q; a.d_k = d_k; a.d_f_key = d_f_key; a.d_s0 = d_s0;
-    a.row_select = nullptr;
     a.B = B; a.T = T; a.D = D; a.K = K; a.C = C;
     a.heads = (int32_t)heads;
     a.NC = t2fw_lfw_num_ckpt(T, C);
@@ -337,7 +336,7 @@ static int lfw_backward_rows(const void *g_out, const void *g_state, const void 
         c.B = B; c.T = T; c.NC = a.NC; c.C = C;
         c.heads = (int32_t)heads;
         if (par_ok(C, flags)) {
-            // chunk-parallel kernels; the rows they flag are redone with the exact scan
+            // chunk-parallel kernels
             ParBwdArgs pa{};
             pa.g_out = g_out; pa.g_state = g_state; pa.x = x; pa.f = f; pa.q = q; pa.k = k; pa.f_key = f_key; pa.ckpt = ckpt;
             pa.d_x = d_x; pa.d_f = d_f; pa.d_q = d_q; pa.d_k = d_k; pa.d_f_key = d_f_key; pa.d_s0 = d_s0;
@@ -351,13 +350,16 @@ static int lfw_backward_rows(const void *g_out, const void *g_state, const void 
             pa.heads = (int32_t)heads;
             if ((rc = par_backward(pa, dtype, st))) return rc;
             if (flags & T2FW_FLAG_NO_FIXUP) return T2FW_OK;
-            a.row_select = pa.row_flags;
-            return scan_backward(a, dtype, st);
+            // The rows it declined go to the block-wise kernel (16-step products instead of products over
+            // half a chunk), which redoes with the exact scan, inside the kernel, what it cannot take
+            // either.  Every other workgroup of that launch reads its row's flag and leaves.
+            c.row_select = pa.row_flags;
+            c.redo = 1;
+            return chunk_backward(c, dtype, 0, st);
         }
         const int op = (dtype == T2FW_F16 && (flags & T2FW_FLAG_FP16_OPERANDS)) ? 1 : 0;
-        if ((rc = chunk_backward(c, dtype, op, st))) return rc;
-        a.row_select = c.row_flags;      // rows the chunked form could not take
-        if (flags & T2FW_FLAG_NO_FIXUP) return T2FW_OK;
+        c.redo = (flags & T2FW_FLAG_NO_FIXUP) ? 0 : 1;
+        return chunk_backward(c, dtype, op, st);
     }
     return scan_backward(a, dtype, st);
 }

@@ -45,6 +45,9 @@ struct ChunkBwdArgs {
     const int32_t *row_select;         // null: every row; else only rows b with row_select[b] != 0 (the others report "not flagged")
     int64_t B, T, NC;
     int32_t C;
+    int32_t redo;                      // nonzero: a workgroup whose row the chunked form cannot take redoes its side
+                                       // of that row with the exact scan, inside the kernel
+    int32_t scan_kg, scan_ntiles;      // geometry of the exact scan body for a 64 x 64 state (set by the launcher)
     int32_t heads;                     // as for the forward (inputs, g_out and the five [.., T, .., 64] gradients)
 };
 

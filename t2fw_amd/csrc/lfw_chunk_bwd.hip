@@ -58,6 +58,7 @@
 #include <type_traits>
 
 #include "lfw_chunk_bwd_dev.hpp"
+#include "lfw_scan_body.hpp"
 
 namespace t2fw {
 namespace {
@@ -87,7 +88,8 @@ constexpr int STAGE_BYTES = OFF_RPART + 2 * RBLOCK_BYTES;
 // after the two stage buffers: per matrix wave, room to park its fp32 state slab (64 lanes x 16 floats)
 // while the B part of a stage needs the registers
 constexpr int OFF_PARK = 2 * STAGE_BYTES;
-constexpr int BW_SMEM = OFF_PARK + 4 * 64 * 16 * 4;
+constexpr int OFF_VERDICT = OFF_PARK + 4 * 64 * 16 * 4;      // one int: a prep wave of this workgroup flagged the row
+constexpr int BW_SMEM = OFF_VERDICT + 16;
 static_assert(BW_SMEM <= 160 * 1024, "backward stage buffers exceed the LDS of one CU");
 static_assert(BLOCK_BYTES % 16 == 0 && RBLOCK_BYTES % 16 == 0, "tile regions must keep 16-byte alignment");
 
@@ -483,7 +485,10 @@ __device__ __forceinline__ void bwd_prep_waves(const ChunkBwdArgs &p, unsigned c
     }
     // Both workgroups of a row see all four gates' blocks and reach the same verdict, so either
     // order of their writes leaves the same flag.
-    if (bad) p.row_flags[b] = 1;
+    if (bad) {
+        p.row_flags[b] = 1;
+        *reinterpret_cast<volatile int *>(smem + OFF_VERDICT) = 1;
+    }
 }
 
 template <typename IOE, typename OPE, int NB, bool HEADS, int SIDE>
@@ -536,6 +541,7 @@ __device__ __forceinline__ void bwd_matrix_waves(const ChunkBwdArgs &p, unsigned
     if (tid == 0) {      // both flag slots of the row (the backward kernels report in the first)
         p.row_flags[b] = 0;
         p.row_flags[chunk_rows_padded(p.B) + b] = 0;
+        *reinterpret_cast<volatile int *>(smem + OFF_VERDICT) = 0;      // published by the first stage's barrier
     }
 
     // R part of a stage: the states at the start of blocks i2 and i2 + 1 of a chunk with nbc blocks
@@ -773,6 +779,26 @@ __global__ __launch_bounds__(BW_THREADS) void lfw_bwd_chunk_kernel(ChunkBwdArgs 
     } else {
         bwd_prep_waves<IOE, OPE, NB, HEADS>(p, smem, tid - 256, b, side);
     }
+    // A barrier publishes the prep waves' verdict.  If the chunked form could not take the row, the first
+    // SCAN_THREADS threads redo this workgroup's side of it with the exact scan, in place, and everyone
+    // else leaves (a workgroup barrier only waits for the waves that are still there).  The scan body
+    // needs more registers than this kernel's waves have: it spills here, which only such rows pay for.
+    __syncthreads();
+    if (tid >= SCAN_THREADS || !p.redo) return;
+    if (*reinterpret_cast<volatile int *>(smem + OFF_VERDICT) == 0) return;
+    ScanBwdArgs sa{};
+    sa.g_out = p.g_out; sa.g_state = p.g_state; sa.x = p.x; sa.f = p.f; sa.q = p.q; sa.k = p.k; sa.f_key = p.f_key;
+    sa.ckpt = p.ckpt;
+    sa.d_x = p.d_x; sa.d_f = p.d_f; sa.d_q = p.d_q; sa.d_k = p.d_k; sa.d_f_key = p.d_f_key; sa.d_s0 = p.d_s0;
+    sa.B = p.B; sa.T = p.T; sa.D = CH_N; sa.K = CH_N; sa.NC = p.NC;
+    sa.C = p.C; sa.kg = p.scan_kg; sa.use_sub = 1; sa.ntiles = p.scan_ntiles; sa.heads = p.heads;
+    for (int tile = 0; tile < p.scan_ntiles; ++tile) {
+        __syncthreads();        // the stage buffers, or the tile before, are no longer read
+        if (side == 0)
+            scan::bwd_scan_body_kg<typename IOE::io_type, 4, 0, 16, 1>(sa, b, tile);
+        else
+            scan::bwd_scan_body_kg<typename IOE::io_type, 4, 1, 16, 1>(sa, b, tile);
+    }
 }
 
 template <typename IOE, typename OPE, int NB, bool HEADS> int launch(const ChunkBwdArgs &a, hipStream_t stream) {
@@ -786,7 +812,16 @@ template <typename IOE, typename OPE, int NB, bool HEADS> int launch(const Chunk
     if (a.heads < 1 || a.T * a.heads >= CHUNK_MAX_T)
         return fail(T2FW_ERR_UNSUPPORTED, "T=%lld with %d heads is too long for 32-bit row offsets", (long long)a.T, a.heads);
     const int rows_padded = (int)((a.B + 7) / 8 * 8);
-    hipLaunchKernelGGL(kern, dim3(2u * (unsigned)rows_padded), dim3(BW_THREADS), BW_SMEM, stream, a, rows_padded);
+    ChunkBwdArgs a2 = a;
+    {
+        // the exact scan body for flagged rows: 16 lanes per state row, four columns per lane, the
+        // segment-start states of a chunk in LDS (which this kernel's allocation holds with room to spare)
+        const ScanGeom g = scan_geometry(CH_N);
+        if (g.kg != 16 || g.kpl != 4) return fail(T2FW_ERR_UNSUPPORTED, "unexpected scan geometry for a 64 x 64 state");
+        a2.scan_kg = g.kg;
+        a2.scan_ntiles = (CH_N + g.rows - 1) / g.rows;
+    }
+    hipLaunchKernelGGL(kern, dim3(2u * (unsigned)rows_padded), dim3(BW_THREADS), BW_SMEM, stream, a2, rows_padded);
     return check_hip(hipGetLastError(), "lfw_bwd_chunk_kernel launch");
 }
 

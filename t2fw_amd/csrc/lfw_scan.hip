@@ -28,47 +28,12 @@ __global__ __launch_bounds__(SCAN_THREADS) void lfw_fwd_scan_kernel(ScanFwdArgs 
     fwd_scan_body<IO, KPL>(p, blockIdx.x / p.ntiles, (int)(blockIdx.x % p.ntiles));
 }
 
-// The rows another kernel has flagged (row_select): a small grid of workgroups that walk over the
-// batch rows, and over the tiles of a flagged row, themselves, so that the launch, in which
-// normally every workgroup finds nothing to do, dispatches as little as possible.  64 x 64
-// states only (16 lanes per state row, segment-start buffer).
-constexpr int ROW_SELECT_GRID = 32;
-template <typename IO, int KPL, int SIDE> __device__ __forceinline__ void bwd_scan_rows(const ScanBwdArgs &p) {
-    // The usual case is that no row is flagged: every thread looks at one of the workgroup's rows, so
-    // that the workgroup learns it with one round trip to memory instead of one per row.
-    int mine = 0;
-    for (int64_t b = blockIdx.x + (int64_t)threadIdx.x * gridDim.x; b < p.B; b += (int64_t)gridDim.x * SCAN_THREADS)
-        mine |= p.row_select[b];
-    if (!__syncthreads_or(mine)) return;
-    bool first = true;
-    for (int64_t b = blockIdx.x; b < p.B; b += gridDim.x) {
-        if (p.row_select[b] == 0) continue;          // the same for every thread of the workgroup
-        for (int tile = 0; tile < p.ntiles; ++tile) {
-            if (!first) __syncthreads();
-            first = false;
-            bwd_scan_body_kg<IO, KPL, SIDE, 16, 1>(p, b, tile);
-        }
-    }
-}
-
 // One workgroup per (batch row, tile); a kernel per geometry (KG lanes per state row, 0 = any) and
 // per use of the segment-start buffer, so that each is register-allocated on its own: a spill
 // in the loop would wait for the prefetched global loads, which return in order with it.
 template <typename IO, int KPL, int SIDE, int KG, int SUB>
 __global__ __launch_bounds__(SCAN_THREADS) void lfw_bwd_scan_kernel(ScanBwdArgs p) {
     bwd_scan_body_kg<IO, KPL, SIDE, KG, SUB>(p, blockIdx.x / p.ntiles, (int)(blockIdx.x % p.ntiles));
-}
-
-
-// Both sides in one launch (blockIdx.y = side) for square states, where the two sides share
-// their geometry.  Used when the kernel only redoes the rows another kernel has flagged:
-// then most workgroups exit at once and a launch costs more than it computes.
-template <typename IO, int KPL>
-__global__ __launch_bounds__(SCAN_THREADS) void lfw_bwd_scan_both_kernel(ScanBwdArgs p) {
-    if (blockIdx.y == 0)
-        bwd_scan_rows<IO, KPL, 0>(p);
-    else
-        bwd_scan_rows<IO, KPL, 1>(p);
 }
 
 // ------------------------------------------------------------------------------------
@@ -99,26 +64,15 @@ int launch_bwd(ScanBwdArgs a, const ScanGeom &g, hipStream_t stream) {
     const size_t smem = base + (a.use_sub ? sub : 0);
     a.kg = g.kg;
     a.ntiles = (int)((nrows + g.rows - 1) / g.rows);
-    const int64_t nblocks = a.row_select != nullptr ? (a.B < ROW_SELECT_GRID ? a.B : ROW_SELECT_GRID) : a.B * a.ntiles;
+    const int64_t nblocks = a.B * a.ntiles;
     if (nblocks > 0x7fffffffLL) return fail(T2FW_ERR_UNSUPPORTED, "grid of %lld workgroups is too large", (long long)nblocks);
-    if constexpr (SIDE == 2) {
-        // only the chunked kernels select rows: 64 x 64 states of 16-bit elements
-        if constexpr (KPL == 4 && sizeof(IO) == 2) {
-            if (g.kg != 16 || !a.use_sub) return fail(T2FW_ERR_UNSUPPORTED, "unexpected scan geometry for a 64 x 64 state");
-            hipLaunchKernelGGL((lfw_bwd_scan_both_kernel<IO, KPL>), dim3((unsigned)nblocks, 2, 1), dim3(SCAN_THREADS), smem,
-                               stream, a);
-            return check_hip(hipGetLastError(), "lfw_bwd_scan_both_kernel launch");
-        }
-        return fail(T2FW_ERR_UNSUPPORTED, "row selection takes 64 x 64 states of 16-bit elements");
-    } else {
-        dim3 grid((unsigned)nblocks, 1, 1);
-        if (KPL <= 4 && g.kg == 16 && a.use_sub)
-            hipLaunchKernelGGL((lfw_bwd_scan_kernel<IO, KPL, SIDE, (KPL <= 4 ? 16 : 0), 1>), grid, dim3(SCAN_THREADS), smem, stream, a);
-        else if (a.use_sub)
-            hipLaunchKernelGGL((lfw_bwd_scan_kernel<IO, KPL, SIDE, 0, 1>), grid, dim3(SCAN_THREADS), smem, stream, a);
-        else
-            hipLaunchKernelGGL((lfw_bwd_scan_kernel<IO, KPL, SIDE, 0, 0>), grid, dim3(SCAN_THREADS), smem, stream, a);
-    }
+    dim3 grid((unsigned)nblocks, 1, 1);
+    if (KPL <= 4 && g.kg == 16 && a.use_sub)
+        hipLaunchKernelGGL((lfw_bwd_scan_kernel<IO, KPL, SIDE, (KPL <= 4 ? 16 : 0), 1>), grid, dim3(SCAN_THREADS), smem, stream, a);
+    else if (a.use_sub)
+        hipLaunchKernelGGL((lfw_bwd_scan_kernel<IO, KPL, SIDE, 0, 1>), grid, dim3(SCAN_THREADS), smem, stream, a);
+    else
+        hipLaunchKernelGGL((lfw_bwd_scan_kernel<IO, KPL, SIDE, 0, 0>), grid, dim3(SCAN_THREADS), smem, stream, a);
     return check_hip(hipGetLastError(), "lfw_bwd_scan_kernel launch");
 }
 
@@ -176,7 +130,7 @@ template <typename IO, int SIDE> int bwd_pass(const ScanBwdArgs &a, int64_t widt
 // The reduced dimension (K on side 0, D on side 1) in windows, as for the forward.
 template <typename IO, int SIDE> int bwd_by_kpl(ScanBwdArgs a, hipStream_t stream) {
     const int64_t ncols = SIDE == 0 ? a.K : a.D;
-    if (ncols <= SCAN_MAX_COLS || SIDE == 2) return bwd_pass<IO, SIDE>(a, ncols, stream);
+    if (ncols <= SCAN_MAX_COLS) return bwd_pass<IO, SIDE>(a, ncols, stream);
     for (int64_t c0 = 0; c0 < ncols; c0 += SCAN_MAX_COLS) {
         a.col0 = c0;
         a.colw = ncols - c0 < SCAN_MAX_COLS ? ncols - c0 : SCAN_MAX_COLS;
@@ -188,11 +142,6 @@ template <typename IO, int SIDE> int bwd_by_kpl(ScanBwdArgs a, hipStream_t strea
 }
 
 template <typename IO> int bwd_both(const ScanBwdArgs &a, hipStream_t stream) {
-    // SIDE 2 = both sides in one launch (the rows another kernel has flagged)
-    if (a.row_select != nullptr) {
-        if (a.D != a.K) return fail(T2FW_ERR_UNSUPPORTED, "row selection takes square states");
-        return bwd_by_kpl<IO, 2>(a, stream);
-    }
     int rc = bwd_by_kpl<IO, 0>(a, stream);
     if (rc != T2FW_OK) return rc;
     return bwd_by_kpl<IO, 1>(a, stream);

@@ -21,7 +21,6 @@ struct ScanFwdArgs {
 struct ScanBwdArgs {
     const void *g_out, *g_state, *x, *f, *q, *k, *f_key, *ckpt;
     void *d_x, *d_f, *d_q, *d_k, *d_f_key, *d_s0;
-    const int32_t *row_select;          // null, or per batch row: 0 = skip the row
     int64_t B, T, D, K, NC;
     int32_t C, kg, use_sub, ntiles;
     int32_t heads;                      // as for the forward (inputs, g_out and the five [.., T, .., D|K] gradients)

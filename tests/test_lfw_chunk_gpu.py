@@ -26,6 +26,16 @@ def flagged_rows(ws, B, chunk_parallel=False):
     return int(((f[:B] != 0) | (f[pad:pad + B] != 0)).sum())
 
 
+class Flagged(tuple):
+    """(rows flagged by the forward, rows flagged by the backward's first kernel); ``exact`` = rows the
+    backward handed on to the exact scan (for the chunk-parallel backward: rows that the block-wise kernel,
+    which takes what it declines, declined as well)"""
+    def __new__(cls, fwd, bwd, exact):
+        obj = super().__new__(cls, (fwd, bwd))
+        obj.exact = exact
+        return obj
+
+
 def chunk_parallel_backward(C, flags):
     """the backward runs the chunk-parallel kernels unless a flag asks for the block-wise ones"""
     from t2fw_amd import _lib
@@ -51,7 +61,7 @@ def run_abi(inputs, go, gs, C, flags=0, with_backward=True):
                                     B, T, D, K, C, code, flags, _lib.ptr(ws), wsb, st))
     torch.cuda.synchronize()
     flagged_fwd = flagged_rows(ws, B) if wsb else 0
-    grads, flagged_bwd = None, 0
+    grads, flagged_bwd, exact_bwd = None, 0, 0
     if with_backward:
         grads = [torch.empty_like(t) for t in ins]
         go_d, gs_d = go.cuda(), gs.cuda()      # keep the device copies alive across the launch
@@ -60,7 +70,8 @@ def run_abi(inputs, go, gs, C, flags=0, with_backward=True):
                                          _lib.ptr(ws), wsb, st))
         torch.cuda.synchronize()
         flagged_bwd = flagged_rows(ws, B, chunk_parallel_backward(C, flags)) if wsb else 0
-    return out, nxt, ckpt, grads, (flagged_fwd, flagged_bwd)
+        exact_bwd = flagged_rows(ws, B) if wsb else 0
+    return out, nxt, ckpt, grads, Flagged(flagged_fwd, flagged_bwd, exact_bwd)
 
 
 def assert_within_reference_bounds(out, r_out, grads, r_grads):

@@ -71,7 +71,8 @@ def test_gate_products_down_to_the_accepted_range_stay_on_the_matrix_cores(C):
 @pytest.mark.parametrize("where", ["first_half", "second_half", "key_side", "last_partial_chunk"])
 def test_half_chunk_products_below_the_range_are_flagged_in_the_backward_only(where):
     """32 gates of 0.15 (product 2^-87.6) in one half of a chunk: the forward's 16-step blocks take
-    them (2^-43.8 each), the backward hands the row to the exact scan."""
+    them (2^-43.8 each); the chunk-parallel backward declines the row, and the block-wise kernel that
+    follows it takes it (nothing reaches the exact scan)."""
     B, T, C = 3, 230, 64
     x, f, q, k, fk, s, go, gs = make_config_inputs(B, T, 64, 64, torch.float16, seed=19, state_std=0.3)
     f, fk = f.clone(), fk.clone()
@@ -84,10 +85,25 @@ def test_half_chunk_products_below_the_range_are_flagged_in_the_backward_only(wh
     else:
         fk[1, 192:224, 0] = 0.15            # the last chunk holds 38 tokens
     out, nxt, ckpt, grads, flagged = run_abi((x, f, q, k, fk, s), go, gs, C)
-    assert flagged == (0, 1), flagged
+    assert flagged == (0, 1) and flagged.exact == 0, (flagged, flagged.exact)
     (r_out, r_nxt), r_grads = oracle((x, f, q, k, fk, s), go, gs)
     assert_all_chunk(grads, r_grads, torch.float16)
-    assert_rows_exact(grads, r_grads, [1], torch.float16)
+
+
+def test_rows_that_neither_matrix_core_form_takes_reach_the_exact_scan():
+    """a row with small gates over half a chunk (declined by the chunk-parallel form only) next to a row
+    with a 16-step product below the block-wise form's limit and a row with a zero gate"""
+    B, T, C = 4, 256, 64
+    x, f, q, k, fk, s, go, gs = make_config_inputs(B, T, 64, 64, torch.float16, seed=21, state_std=0.3)
+    f, fk = f.clone(), fk.clone()
+    f[0, 64:96, 3] = 0.15               # 2^-87.6 over half a chunk, 2^-43.8 per block
+    fk[1, 128:144, 9] = 0.01            # 2^-106 in one block
+    f[3, 200, 60] = 0.0
+    out, nxt, ckpt, grads, flagged = run_abi((x, f, q, k, fk, s), go, gs, C)
+    assert flagged[1] == 3 and flagged.exact == 2, (flagged, flagged.exact)
+    (r_out, r_nxt), r_grads = oracle((x, f, q, k, fk, s), go, gs)
+    assert_all_chunk(grads, r_grads, torch.float16)
+    assert_rows_exact(grads, r_grads, [1, 3], torch.float16)
 
 
 def test_small_gates_across_a_half_chunk_boundary_are_accepted():
