@@ -84,9 +84,13 @@ int compute_units() {
 //   [B, NC, PAR_NVEC, 64] fp32, adjoint entering every chunk [B, NC, 64, 64] bf16
 size_t row_flag_bytes(int64_t B) { return (size_t)((2 * chunk_rows_padded(B) * 4 + 255) / 256 * 256); }
 
-// The chunk-parallel kernels take checkpoint intervals 32 and 64 and bf16 matrix-core operands.
-bool par_ok(int32_t C, int32_t flags) {
-    return (C == 32 || C == 64) && (flags & (T2FW_FLAG_BLOCKWISE | T2FW_FLAG_FP16_OPERANDS)) == 0;
+// The chunk-parallel kernels take checkpoint intervals 32 and 64, bf16 matrix-core operands and
+// [B, T, 64] arrays of fewer than 2^31 elements (32-bit element offsets); anything else that the
+// matrix cores can take runs block-wise.
+bool par_ok(int64_t B, int64_t T, int32_t C, int32_t flags) {
+    if ((C != 32 && C != 64) || (flags & (T2FW_FLAG_BLOCKWISE | T2FW_FLAG_FP16_OPERANDS)) != 0) return false;
+    const long double elems = (long double)B * (long double)T * CH_N;
+    return elems < 2147483647.0L && (long double)B * (long double)((T + C - 1) / C) <= (long double)0x3fffffff;
 }
 
 struct ParScratch {
@@ -110,7 +114,7 @@ size_t forward_workspace_bytes(int64_t B, int64_t D, int64_t K, int32_t dtype, i
 
 size_t backward_workspace_bytes(int64_t B, int64_t T, int64_t D, int64_t K, int32_t C, int32_t dtype, int32_t flags) {
     if (B > 0 && chunk_shape_ok(D, K, dtype, flags))
-        return par_ok(C, flags) ? par_scratch(B, T, C).total : 2 * row_flag_bytes(B);
+        return par_ok(B, T, C, flags) ? par_scratch(B, T, C).total : 2 * row_flag_bytes(B);
     return 0;
 }
 
@@ -335,7 +339,7 @@ static int lfw_backward_rows(const void *g_out, const void *g_state, const void 
         c.row_select = nullptr;
         c.B = B; c.T = T; c.NC = a.NC; c.C = C;
         c.heads = (int32_t)heads;
-        if (par_ok(C, flags)) {
+        if (par_ok(B, T, C, flags)) {
             // chunk-parallel kernels
             ParBwdArgs pa{};
             pa.g_out = g_out; pa.g_state = g_state; pa.x = x; pa.f = f; pa.q = q; pa.k = k; pa.f_key = f_key; pa.ckpt = ckpt;

@@ -53,6 +53,19 @@ def test_abi_version_and_ckpt_count(lib):
     assert lib.t2fw_lfw_num_ckpt(8192, 1) == 8192
 
 
+def test_workspace_queries(lib):
+    fwd = lib.t2fw_lfw_forward_workspace_bytes(96, 1024, 64, 64, 64, 1, 0)
+    both = lib.t2fw_lfw_workspace_bytes(96, 1024, 64, 64, 64, 1, 0)
+    assert fwd == 2 * 768 and both > 96 * 16 * 8192                      # flags; + per-chunk scratch of the backward
+    assert lib.t2fw_lfw_workspace_bytes(96, 1024, 64, 64, 64, 1, 8) == fwd     # block-wise backward: flags only
+    assert lib.t2fw_lfw_workspace_bytes(96, 1024, 64, 64, 16, 1, 0) == fwd     # interval the chunk-parallel form does not take
+    assert lib.t2fw_lfw_workspace_bytes(96, 1024, 33, 17, 64, 1, 0) == 0       # exact kernels: none
+    assert lib.t2fw_lfw_workspace_bytes(96, 1024, 64, 64, 64, 0, 0) == 0       # fp32: exact kernels
+    # arrays of 2^31 elements and more are beyond the chunk-parallel kernels' 32-bit offsets: block-wise, flags only
+    big = lib.t2fw_lfw_workspace_bytes(4096, 16384, 64, 64, 64, 1, 0)
+    assert big == lib.t2fw_lfw_forward_workspace_bytes(4096, 16384, 64, 64, 64, 1, 0)
+
+
 def _fwd(lib, ptrs, B, T, D, K, C, dtype):
     return lib.t2fw_lfw_forward(*ptrs, B, T, D, K, C, dtype, 0, None, 0, None)
 
