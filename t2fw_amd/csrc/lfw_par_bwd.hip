@@ -118,8 +118,11 @@ constexpr int SCAN_TPB = 256, SCAN_BATCH = 16, SCAN_VEC = 2 * 8 + 2 * CH_N;     
 
 template <typename IOE> __global__ __launch_bounds__(SCAN_TPB) void lfw_par_scan_kernel(ParBwdArgs p) {
     __shared__ float vl[SCAN_BATCH * SCAN_VEC];
-    const int64_t b = blockIdx.x >> 3;
-    const int slab = (int)(blockIdx.x & 7), tid = threadIdx.x;
+    // Consecutive workgroups go to the eight XCDs in turn: the eight slabs of a batch row, which all read
+    // the row's gate-product vectors, get ids that are 8 apart and share one XCD's L2.
+    const int64_t b = (int64_t)(blockIdx.x >> 6) * 8 + (blockIdx.x & 7);
+    if (b >= p.B) return;
+    const int slab = (int)((blockIdx.x >> 3) & 7), tid = threadIdx.x;
     const int dl = tid >> 5, d = slab * 8 + dl, k = (tid & 31) * 2;
     const int NC = (int)p.NC;
     float G0, G1;
@@ -525,7 +528,7 @@ template <typename IOE, int NT, bool HEADS> int launch(const ParBwdArgs &a, hipS
         return fail(T2FW_ERR_UNSUPPORTED, "B=%lld T=%lld with %d heads is too large for 32-bit element offsets", (long long)a.B, (long long)a.T, a.heads);
     hipLaunchKernelGGL(incr, dim3((unsigned)items), dim3(PAR_THREADS), INCR_SMEM, stream, a);
     if ((rc = check_hip(hipGetLastError(), "lfw_par_incr_kernel launch"))) return rc;
-    hipLaunchKernelGGL(scan, dim3((unsigned)(8 * a.B)), dim3(SCAN_TPB), 0, stream, a);
+    hipLaunchKernelGGL(scan, dim3((unsigned)(64 * ((a.B + 7) / 8))), dim3(SCAN_TPB), 0, stream, a);
     if ((rc = check_hip(hipGetLastError(), "lfw_par_scan_kernel launch"))) return rc;
     hipLaunchKernelGGL(grads, dim3((unsigned)items), dim3(GR_THREADS), GR_SMEM, stream, a);
     return check_hip(hipGetLastError(), "lfw_par_grads_kernel launch");
