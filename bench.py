@@ -11,11 +11,12 @@ synthetic input already resident in HBM, at the headline configuration
 value      = B*T*steps / wall time of the timed region, in Mtokens/s (token = one
              (batch row, time step) pair), driving the C ABI directly with preallocated
              outputs; `autograd_api` repeats it through LFWFunction.apply + backward.
-roofline   = algorithmic bytes of the dominant kernel / its mean duration measured with
-             events on the launch stream (the call is repeated with the flag that skips the
-             exact redo of flagged rows, for the backward a launch of its own, so that the
-             events bracket that one kernel), against
-             8 TB/s.  `traffic` comes from profiles/traffic_<workload>.json (rocprofv3 counters).
+roofline   = algorithmic bytes of the dominant call (the backward: three launches, named in
+             `launches`) / its mean duration measured with events on the launch stream (the call is
+             repeated with the flag that skips the launch for flagged rows that follows them, so
+             that the events bracket those kernels; `call_with_fixup_launch_ms` is the call as
+             shipped), against 8 TB/s.  `traffic` = measured HBM bytes of the same launches, from
+             profiles/traffic_<workload>.json (rocprofv3 counters).
 dfw        = the delta-rule kernels (forward + backward) at cfg3's shape in fp32, the dtype the
              reference tests them in.
 copy256    = calibration workload for those counters: a 256 MiB device-to-device copy.
@@ -194,8 +195,19 @@ def main():
             traffic = json.load(open(tpath)).get(dom)
         except Exception:
             traffic = None
+    # which launches `dom` stands for (the names under which rocprofv3 lists them)
+    flags_now = flags
+    if dom == "forward":
+        launches = ["lfw_fwd_scan_kernel"] if args.force_scan else ["lfw_fwd_chunk_half_kernel" if 2 * ((B + 7) // 8 * 8) <= 256
+                                                                    else "lfw_fwd_chunk_kernel"]
+    elif args.force_scan:
+        launches = ["lfw_bwd_scan_kernel (value side)", "lfw_bwd_scan_kernel (key side)"]
+    elif C in (32, 64) and not flags_now & (_lib.FLAG_BLOCKWISE | _lib.FLAG_FP16_OPERANDS):
+        launches = ["lfw_par_incr_kernel", "lfw_par_scan_kernel", "lfw_par_grads_kernel"]
+    else:
+        launches = ["lfw_bwd_chunk_kernel"]
     roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic, "kernel": dom,
+                "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic, "kernel": dom, "launches": launches,
                 "call_with_fixup_launch_ms": round(bwd_avg if dom == "backward" else fwd_avg, 5),
                 "algorithmic_bytes": dom_bytes, "avg_launch_ms": round(dom_ms, 5)}
     whole = (fwd_bytes + bwd_bytes) / (ms_per_step * 1e-3) / 1e9
