@@ -149,24 +149,39 @@ template <int NT> struct LaneChunk {
 };
 
 // Raw 16-bit loads of one array: this lane's NT * 4 tokens of channel c, two tokens per register
-// (the loads write the low and the high half of a register directly).  p: the array at token
-// (chunk start + 4 kg), channel c; ts: elements between consecutive tokens; n_left: tokens from p's
-// token to the end of the sequence (tokens at or past the end are read from the last one).
+// (the loads write the low and the high half of a register directly).  ubase: the array at the
+// chunk's first token, channel 0 (the same for the whole workgroup, so that a token's address is a
+// scalar base plus the lane's fixed offset, whatever the token stride); lane_off = 4 kg * ts + c; ts:
+// elements between consecutive tokens; n_left: tokens from the lane's first token to the end of the
+// sequence (tokens at or past the end are read from the last one).
 typedef unsigned short us2 __attribute__((ext_vector_type(2)));
 template <int NT> struct RawTokens {
     us2 p[NT][2];
     __device__ __forceinline__ u16 at(int m, int j) const { return (j & 1) ? p[m][j >> 1].y : p[m][j >> 1].x; }
 };
 
+// a value that is the same in every lane, moved to scalar registers (the compiler computes 64-bit
+// divisions in vector registers and would otherwise keep what is derived from them there)
+__device__ __forceinline__ int64_t wave_uniform(int64_t v) {
+    const u32 lo = __builtin_amdgcn_readfirstlane((u32)(unsigned long long)v);
+    const u32 hi = __builtin_amdgcn_readfirstlane((u32)((unsigned long long)v >> 32));
+    return (int64_t)(((unsigned long long)hi << 32) | lo);
+}
+
 template <int NT, bool FULL>
-__device__ __forceinline__ void load_tokens(RawTokens<NT> &r, const u16 *p, u32 ts, int n_left) {
+__device__ __forceinline__ void load_tokens(RawTokens<NT> &r, const u16 *ubase, u32 lane_off, u32 ts, int n_left) {
 #pragma unroll
     for (int m = 0; m < NT; ++m)
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-            int o = 16 * m + j;
-            if (!FULL) o = min(o, n_left - 1);
-            const u16 v = p[o * (int)ts];
+            u16 v;
+            if (FULL) {
+                const u16 *const tok = ubase + (size_t)(16 * m + j) * ts;      // wave-uniform
+                v = tok[lane_off];
+            } else {
+                const int o = min(16 * m + j, n_left - 1);
+                v = ubase[lane_off + (u32)o * ts];
+            }
             if (j & 1)
                 r.p[m][j >> 1].y = v;
             else

@@ -55,22 +55,24 @@ __global__ __launch_bounds__(PAR_THREADS) void lfw_par_incr_kernel(ParBwdArgs p)
     const int chunk = item - (int)b * NC;
     const u32 ts = HEADS ? (u32)p.heads * CH_N : (u32)CH_N;
     const int tok0 = chunk * CL + 4 * kg, n_left = T - tok0;
-    const int64_t off = row_first_token(b, p.T, HEADS ? p.heads : 1) * CH_N + (int64_t)tok0 * ts + c;
-    const u16 *const gate = reinterpret_cast<const u16 *>(side ? p.f_key : p.f) + off;
-    const u16 *const adj = reinterpret_cast<const u16 *>(side ? p.q : p.g_out) + off;
+    // the chunk's first token (wave-uniform) and the lane's offset from there
+    const int64_t chunk_off = wave_uniform(row_first_token(b, p.T, HEADS ? p.heads : 1) * CH_N + (int64_t)(chunk * CL) * ts);
+    const u32 lane_off = (u32)(4 * kg) * ts + (u32)c;
+    const u16 *const gate = reinterpret_cast<const u16 *>(side ? p.f_key : p.f) + chunk_off;
+    const u16 *const adj = reinterpret_cast<const u16 *>(side ? p.q : p.g_out) + chunk_off;
     u32 bad;
     {
         RawTokens<NT> rg, ra;
         LaneChunk<NT> lc;
         float gt[NT][4], av[NT][4];
         if (chunk * CL + CL <= T) {
-            load_tokens<NT, true>(rg, gate, ts, n_left);
-            load_tokens<NT, true>(ra, adj, ts, n_left);
+            load_tokens<NT, true>(rg, gate, lane_off, ts, n_left);
+            load_tokens<NT, true>(ra, adj, lane_off, ts, n_left);
             gate_scan<IOE, NT, true>(lc, gt, rg, kg, n_left);
             to_floats<IOE, NT, true>(av, ra, n_left);
         } else {
-            load_tokens<NT, false>(rg, gate, ts, n_left);
-            load_tokens<NT, false>(ra, adj, ts, n_left);
+            load_tokens<NT, false>(rg, gate, lane_off, ts, n_left);
+            load_tokens<NT, false>(ra, adj, lane_off, ts, n_left);
             gate_scan<IOE, NT, false>(lc, gt, rg, kg, n_left);
             to_floats<IOE, NT, false>(av, ra, n_left);
         }
@@ -222,8 +224,8 @@ template <typename IOE, int NT, bool HEADS, bool FULL> struct GradsItem {
     const ParBwdArgs &p;
     unsigned char *smem;
     int tid, T, NC, cb, side, i, kg, c, lane, n_left;
-    u32 ts, off;
-    int64_t item;
+    u32 ts, lane_off;
+    int64_t item, chunk_off;
 
     __device__ __forceinline__ GradsItem(const ParBwdArgs &p_, unsigned char *smem_, int64_t item_) : p(p_), smem(smem_), item(item_) {
         tid = threadIdx.x;
@@ -236,9 +238,11 @@ template <typename IOE, int NT, bool HEADS, bool FULL> struct GradsItem {
         const int64_t b = item / NC;
         const int chunk = (int)(item - b * NC);
         n_left = T - (chunk * CL + 4 * kg);
-        // element offset of (the lane's first token, its channel) in the [.., T, .., 64] arrays (the launcher
-        // admits arrays of less than 2^31 elements only)
-        off = (u32)(row_first_token(b, p.T, HEADS ? p.heads : 1) * CH_N) + (u32)(chunk * CL + 4 * kg) * ts + (u32)c;
+        // element offsets in the [.., T, .., 64] arrays: the chunk's first token (wave-uniform: token addresses
+        // are a scalar base plus the lane's fixed offset, whatever the token stride) and the lane's
+        // (first token, channel) from there
+        chunk_off = wave_uniform(row_first_token(b, p.T, HEADS ? p.heads : 1) * CH_N + (int64_t)(chunk * CL) * ts);
+        lane_off = (u32)(4 * kg) * ts + (u32)c;
     }
     template <int SIDE> __device__ __forceinline__ u16 *tile_adj() const { return reinterpret_cast<u16 *>(smem + GR_ADJ + SIDE * CM_BYTES); }
     template <int SIDE> __device__ __forceinline__ u16 *tile_val() const { return reinterpret_cast<u16 *>(smem + GR_VAL + SIDE * CM_BYTES); }
@@ -247,9 +251,9 @@ template <typename IOE, int NT, bool HEADS, bool FULL> struct GradsItem {
         RawTokens<NT> g, v, a;
     };
     template <int SIDE> __device__ __forceinline__ void issue_raw(Raw &r) const {
-        load_tokens<NT, FULL>(r.g, reinterpret_cast<const u16 *>(SIDE ? p.f_key : p.f) + off, ts, n_left);
-        load_tokens<NT, FULL>(r.v, reinterpret_cast<const u16 *>(SIDE ? p.k : p.x) + off, ts, n_left);
-        load_tokens<NT, FULL>(r.a, reinterpret_cast<const u16 *>(SIDE ? p.q : p.g_out) + off, ts, n_left);
+        load_tokens<NT, FULL>(r.g, reinterpret_cast<const u16 *>(SIDE ? p.f_key : p.f) + chunk_off, lane_off, ts, n_left);
+        load_tokens<NT, FULL>(r.v, reinterpret_cast<const u16 *>(SIDE ? p.k : p.x) + chunk_off, lane_off, ts, n_left);
+        load_tokens<NT, FULL>(r.a, reinterpret_cast<const u16 *>(SIDE ? p.q : p.g_out) + chunk_off, lane_off, ts, n_left);
     }
     // phase A of one side: gate products relative to the middle of the chunk, scaled operands -> tiles
     template <int SIDE> __device__ __forceinline__ void prep(SideState<NT> &st, const Raw &r) const {
@@ -358,11 +362,11 @@ template <typename IOE, int NT, bool HEADS, bool FULL> struct GradsItem {
             own_adj = g.template tile_adj<SIDE>(); own_val = g.template tile_val<SIDE>();
             oth_adj = g.template tile_adj<1 - SIDE>(); oth_val = g.template tile_val<1 - SIDE>();
             pd = g.template diag<SIDE>();
-            // at (the lane's first token, its channel): the token offsets below are then compile-time
-            // constants of the store instructions wherever the token stride is one
-            d_val = reinterpret_cast<u16 *>(SIDE ? g.p.d_k : g.p.d_x) + g.off;
-            d_gate = reinterpret_cast<u16 *>(SIDE ? g.p.d_f_key : g.p.d_f) + g.off;
-            d_adj = reinterpret_cast<u16 *>(g.p.d_q) + g.off;          // key side only
+            // at the chunk's first token (wave-uniform); a store adds the token's scalar offset and the
+            // lane's fixed one
+            d_val = reinterpret_cast<u16 *>(SIDE ? g.p.d_k : g.p.d_x) + g.chunk_off;
+            d_gate = reinterpret_cast<u16 *>(SIDE ? g.p.d_f_key : g.p.d_f) + g.chunk_off;
+            d_adj = reinterpret_cast<u16 *>(g.p.d_q) + g.chunk_off;          // key side only
             anchor_acc = 0.f;
         }
         // operands of the own side (this lane's channel, tokens 16 m + 4 kg + j), re-read from the own tiles
@@ -376,7 +380,7 @@ template <typename IOE, int NT, bool HEADS, bool FULL> struct GradsItem {
         __device__ __forceinline__ void store4(u16 *dst, int mm, const float (&v)[4]) const {
 #pragma unroll
             for (int j = 0; j < 4; ++j)
-                if (FULL || 16 * mm + j < g.n_left) dst[(16 * mm + j) * (int)g.ts] = cvt1<IOE>(v[j]);
+                if (FULL || 16 * mm + j < g.n_left) (dst + (size_t)(16 * mm + j) * g.ts)[g.lane_off] = cvt1<IOE>(v[j]);
         }
         // forward-like sweep, token tile m: o' (value side) / q' (key side)
         __device__ __forceinline__ void forward_tile(int m, const uint4 &s0a, const uint4 &s0b) {
