@@ -5,7 +5,7 @@ A "step" is one forward + backward pass of the decay-rule recurrence over one ba
 synthetic input already resident in HBM, at the headline configuration
 (B*H=96, T=1024, D=K=64, fp16 I/O, checkpoint interval 64).  Prints ONE JSON line.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg3|cfg3_heads|cfg2|cfg4|cfg5|dfw|copy256]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg3|cfg3_heads|cfg2|cfg4|cfg5|dfw|copy256|copy64]
                     [--no-cpu-baseline]
 
 value      = B*T*steps / wall time of the timed region, in Mtokens/s (token = one
@@ -20,6 +20,7 @@ roofline   = algorithmic bytes of the dominant call (the backward: three launche
 dfw        = the delta-rule kernels (forward + backward) at cfg3's shape in fp32, the dtype the
              reference tests them in.
 copy256    = calibration workload for those counters: a 256 MiB device-to-device copy.
+copy64     = the same copy at 64 MiB: source and destination together stay inside the 256 MB of last-level cache.
 cpu_baseline = the TorchScript restatement of the reference loop (oracle/), fp32,
              forward + autograd backward, timed on this host's cores on a bounded sample.
 parity     = computed in the same CPU leg: per tensor, the GPU results of the first three rows of
@@ -68,7 +69,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", default="cfg3", choices=sorted(WORKLOADS) + ["dfw", "copy256"])
+    ap.add_argument("--workload", default="cfg3", choices=sorted(WORKLOADS) + ["dfw", "copy256", "copy64"])
     ap.add_argument("--ckpt-interval", type=int, default=64)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--force-scan", action="store_true", help="exact scan kernels only")
@@ -87,7 +88,7 @@ def main():
         sys.exit(1)
     if args.workload == "cfg5":
         return bench_generation(args)
-    if args.workload == "copy256":
+    if args.workload in ("copy256", "copy64"):
         return bench_copy(args)
     if args.workload == "dfw":
         return bench_dfw(args)
@@ -314,9 +315,10 @@ def parity_report(d, fwd, bwd, rows=3):
 
 
 def bench_copy(args):
-    """Calibration of the HBM traffic counters: a 256 MiB device-to-device copy per step."""
+    """Calibration of the HBM traffic counters: a 256 MiB (or 64 MiB) device-to-device copy per step."""
     import torch
-    n = 256 * 1024 * 1024
+    mib = int(args.workload[4:])
+    n = mib * 1024 * 1024
     src = torch.empty(n, dtype=torch.uint8, device="cuda").fill_(1)
     dst = torch.empty_like(src)
     for _ in range(args.warmup):
@@ -328,11 +330,11 @@ def bench_copy(args):
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
     gbs = 2 * n * args.steps / wall / 1e9
-    print(json.dumps({"metric": "device copy GB/s (read + write), 256 MiB", "value": round(gbs, 1), "unit": "GB/s",
+    print(json.dumps({"metric": "device copy GB/s (read + write), %d MiB" % mib, "value": round(gbs, 1), "unit": "GB/s",
                       "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
                       "ms_per_step": round(wall / args.steps * 1e3, 5), "higher_is_better": True, "scaling": "weak",
                       "vs_baseline": None, "dtype": "u8", "data": "synthetic",
-                      "config": {"workload": "copy256: torch copy_ of 268435456 bytes, device to device"}}))
+                      "config": {"workload": "%s: torch copy_ of %d bytes, device to device" % (args.workload, n)}}))
 
 
 def bench_dfw(args):
