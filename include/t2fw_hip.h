@@ -50,7 +50,7 @@
 extern "C" {
 #endif
 
-#define T2FW_ABI_VERSION 2
+#define T2FW_ABI_VERSION 3
 
 /* dtype codes (reference dispatch: AT_DISPATCH_FLOATING_TYPES_AND_HALF,
  * lfw_kernel.cu:157 -> fp64/fp32/fp16; bf16 is added here) */
@@ -80,12 +80,11 @@ extern "C" {
                                      more launch of the block-wise kernel, which in turn redoes exactly
                                      what it cannot take); the caller reads the flags
                                      from the workspace (nonzero = that row's results are not
-                                     valid: int32 [2][B rounded up to 8] at its start for the
-                                     forward and the block-wise backward, either slot; int32 [B]
-                                     in the next 256-byte aligned region for the chunk-parallel
-                                     backward) and redoes those rows with T2FW_FLAG_FORCE_SCAN,
-                                     or knows its gates are in range.  Saves the backward's extra
-                                     launch.                                                      */
+                                     valid; t2fw_lfw_flag_regions says where they are) and redoes
+                                     those rows with T2FW_FLAG_FORCE_SCAN, or knows its gates are in
+                                     range: a forward call whose hints (below) are all zero proves
+                                     that for the backward call on the same gates.  Saves the
+                                     backward's extra launch.                                     */
 
 #define T2FW_FLAG_BLOCKWISE 8     /* matrix-core path, backward: the block-wise kernel (16-step blocks in one
                                      pass per batch row; takes 16-step gate products down to 2^-100)
@@ -106,6 +105,28 @@ size_t t2fw_lfw_workspace_bytes(int64_t B, int64_t T, int64_t D, int64_t K,
 /* The same for a caller that only runs the forward call. */
 size_t t2fw_lfw_forward_workspace_bytes(int64_t B, int64_t T, int64_t D, int64_t K,
                                         int32_t C, int32_t dtype, int32_t flags);
+
+/*
+ * Where the calls of a shape leave their per-row flags in the workspace: three regions of int32,
+ * written to regions[0..5] as (byte offset from the start of the workspace, number of entries):
+ *   [0],[1]  forward verdicts: nonzero = the matrix-core form could not take the row (it has been redone
+ *            exactly unless T2FW_FLAG_NO_FIXUP was given);
+ *   [2],[3]  forward hints for the backward call on the same gates: all zero = the chunk-parallel
+ *            backward will flag no row, so that call may be given T2FW_FLAG_NO_FIXUP; many nonzero =
+ *            most rows would be declined and redone, and T2FW_FLAG_BLOCKWISE is the faster path
+ *            (a gate outside [0, 1] or a 16-step gate product below 2^-40 sets a row's hint);
+ *   [4],[5]  backward verdicts, as [0],[1].
+ * A region a path does not write has zero entries (exact kernels: all three).  The workspace may be
+ * any memory the GPU can write, pinned host memory included: a caller that wants to steer the
+ * backward call from the host gives the forward call a pinned workspace and reads the hints once
+ * the forward call has completed.  No counterpart in the reference, which has one path.
+ */
+int t2fw_lfw_flag_regions(int64_t B, int64_t T, int64_t D, int64_t K,
+                          int32_t C, int32_t dtype, int32_t flags, int64_t *regions);
+
+/* The address under which the current GPU sees a pinned host allocation (hipHostMalloc), for a caller
+ * that keeps a workspace there; fails with T2FW_ERR_HIP for memory the GPU cannot reach. */
+int t2fw_host_workspace_device_pointer(void *host_workspace, void **device_pointer);
 
 /*
  * Forward scan.  S_t = S_{t-1} * (f_t (x) f_key_t) + x_t (x) k_t ;  out_t = S_t q_t ;

@@ -12,7 +12,7 @@ import torch  # noqa: F401  (must be loaded before the HIP library)
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "lib", "libt2fw_hip.so")
 
-ABI_VERSION = 2
+ABI_VERSION = 3
 
 F32, F16, BF16, F64 = 0, 1, 2, 3
 DTYPE_CODE = {torch.float32: F32, torch.float16: F16, torch.bfloat16: BF16, torch.float64: F64}
@@ -32,6 +32,8 @@ SIGNATURES = {
     "t2fw_lfw_num_ckpt": (_i64, [_i64, _i32]),
     "t2fw_lfw_workspace_bytes": (_sz, [_i64, _i64, _i64, _i64, _i32, _i32, _i32]),
     "t2fw_lfw_forward_workspace_bytes": (_sz, [_i64, _i64, _i64, _i64, _i32, _i32, _i32]),
+    "t2fw_lfw_flag_regions": (ctypes.c_int, [_i64] * 4 + [_i32] * 3 + [ctypes.POINTER(ctypes.c_int64)]),
+    "t2fw_host_workspace_device_pointer": (ctypes.c_int, [_vp, ctypes.POINTER(ctypes.c_void_p)]),
     "t2fw_lfw_forward": (ctypes.c_int, [_vp] * 9 + [_i64] * 4 + [_i32] * 3 + [_vp, _sz, _vp]),
     "t2fw_lfw_forward_static": (ctypes.c_int, [_vp] * 9 + [_i64] * 4 + [_i32] * 3 + [_vp]),
     "t2fw_lfw_backward": (ctypes.c_int, [_vp] * 15 + [_i64] * 4 + [_i32] * 3 + [_vp, _sz, _vp]),

@@ -11,6 +11,8 @@
 #include <cstring>
 #include <initializer_list>
 #include <mutex>
+#include <set>
+#include <utility>
 
 namespace t2fw {
 
@@ -29,6 +31,19 @@ int fail(int code, const char *fmt, ...) {
 int check_hip(hipError_t e, const char *what) {
     if (e == hipSuccess) return T2FW_OK;
     return fail(T2FW_ERR_HIP, "%s: %s", what, hipGetErrorString(e));
+}
+
+int enable_lds(const void *kernel, int bytes, const char *what) {
+    static std::mutex mu;
+    static std::set<std::pair<const void *, int>> done;
+    int dev = 0;
+    int rc = check_hip(hipGetDevice(&dev), "hipGetDevice");
+    if (rc) return rc;
+    std::lock_guard<std::mutex> lock(mu);
+    if (done.count({kernel, dev})) return T2FW_OK;
+    if ((rc = check_hip(hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes), what))) return rc;
+    done.insert({kernel, dev});
+    return T2FW_OK;
 }
 
 namespace {
@@ -187,6 +202,33 @@ size_t t2fw_lfw_forward_workspace_bytes(int64_t B, int64_t T, int64_t D, int64_t
     return forward_workspace_bytes(B, D, K, dtype, flags);
 }
 
+int t2fw_host_workspace_device_pointer(void *host_workspace, void **device_pointer) {
+    if (host_workspace == nullptr || device_pointer == nullptr) return fail(T2FW_ERR_NULL_POINTER, "null pointer");
+    *device_pointer = nullptr;
+    return check_hip(hipHostGetDevicePointer(device_pointer, host_workspace, 0), "hipHostGetDevicePointer");
+}
+
+int t2fw_lfw_flag_regions(int64_t B, int64_t T, int64_t D, int64_t K, int32_t C, int32_t dtype, int32_t flags,
+                          int64_t *regions) {
+    if (regions == nullptr) return fail(T2FW_ERR_NULL_POINTER, "regions is a null pointer");
+    for (int i = 0; i < 6; ++i) regions[i] = 0;
+    if (elem_size(dtype) == 0) return fail(T2FW_ERR_BAD_DTYPE, "unknown dtype code %d", dtype);
+    const int rc = check_dims(B, T, D, K);
+    if (rc) return rc;
+    if (B == 0 || !chunk_shape_ok(D, K, dtype, flags)) return T2FW_OK;       // exact kernels: no flags
+    const int64_t slots = 2 * chunk_rows_padded(B), region = (int64_t)row_flag_bytes(B);
+    regions[0] = 0; regions[1] = slots;                  // forward verdicts
+    regions[2] = region; regions[3] = slots;             // forward hints for the backward
+    if (C == 32 || C == 64) {                            // else the backward runs on the exact kernels
+        if (par_ok(B, T, C, flags)) {
+            regions[4] = region; regions[5] = B;
+        } else {
+            regions[4] = 0; regions[5] = slots;
+        }
+    }
+    return T2FW_OK;
+}
+
 // B batch rows; heads = 1: rows are contiguous [T, D|K] slabs, heads = H > 1: row b is head b % H of
 // [B / H, T, H, D|K] tensors (x, f, q, k, f_key, out); states and checkpoints are per row either way
 static int lfw_forward_rows(const void *x, const void *f, const void *q, const void *k, const void *f_key,
@@ -237,6 +279,7 @@ static int lfw_forward_rows(const void *x, const void *f, const void *q, const v
         c.x = x; c.f = f; c.q = q; c.k = k; c.f_key = f_key; c.s0 = s0;
         c.out = out; c.next_state = next_state; c.ckpt = ckpt;
         c.row_flags = static_cast<int32_t *>(workspace);
+        c.par_hint = reinterpret_cast<int32_t *>(static_cast<unsigned char *>(workspace) + row_flag_bytes(B));
         c.B = B; c.T = T; c.NC = a.NC; c.C = a.C;
         c.heads = (int32_t)heads;
         c.redo = (flags & T2FW_FLAG_NO_FIXUP) ? 0 : 1;       // flagged rows are redone inside the kernel

@@ -19,6 +19,9 @@ namespace t2fw {
 // ----------------------------------------------------------------------------------
 int fail(int code, const char *fmt, ...);   // records the message, returns code
 int check_hip(hipError_t e, const char *what);
+// Allows `kernel` to be launched with up to `bytes` of dynamic LDS (more than 64 KB has to be enabled per
+// function and device); the runtime is asked once per (kernel, device).
+int enable_lds(const void *kernel, int bytes, const char *what);
 
 // ----------------------------------------------------------------------------------
 // layout of the [.., T, .., width] tensors: batch rows are either contiguous [T, width] slabs

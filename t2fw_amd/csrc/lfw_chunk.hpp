@@ -30,6 +30,8 @@ struct ChunkFwdArgs {
     const void *x, *f, *q, *k, *f_key, *s0;
     void *out, *next_state, *ckpt;     // ckpt may be null
     int32_t *row_flags;                // [2 * chunk_rows_padded(B)]: set to 1 for rows the chunked form cannot take
+    int32_t *par_hint;                 // same shape, may be null: set to 1 for rows the chunk-parallel backward may decline
+                                       // (a 16-step gate product below PAR_HINT_MIN_PRODUCT, or what row_flags reports)
     int64_t B, T, NC;
     int32_t C;                         // checkpoint interval, multiple of 32
     int32_t heads;                     // 1: rows are [T, 64] slabs; H > 1: row b is head b % H of a [B / H, T, H, 64] tensor
@@ -83,9 +85,15 @@ typedef unsigned int u32;
 // gfx950 (two of the four result elements wrong); VALU reads of MFMA results are interlocked
 // by the compiler's wait states.
 // 16-bit element types as raw bits + conversions ---------------------------------------
+// A row none of whose 16-step gate products is below this is inside the chunk-parallel backward's range
+// (products over half a chunk, i.e. one or two blocks, at or above 2^-80).
+constexpr float PAR_HINT_MIN_PRODUCT = 9.094947017729282e-13f;      // 2^-40
+
 struct Bf16 {
     using io_type = __hip_bfloat16;      // the same tensor element as the exact kernels see it
     static constexpr u16 ONE_BITS = 0x3F80;
+    static constexpr u16 FLOOR_BITS = 0x3380;        // 2^-24: gates enter the forward's products no smaller
+    static constexpr u16 BWD_FLOOR_BITS = 0x3980;    // 2^-12: ... and the chunk-parallel backward's
     // smallest 16-step gate product accepted with operands of this type: the inverse
     // 1/product scales the intra-block operands and must stay far from overflow
     static constexpr float MIN_PRODUCT = 7.8886090522101181e-31f;   // 2^-100
@@ -110,6 +118,8 @@ struct Bf16 {
 struct Fp16 {
     using io_type = __half;
     static constexpr u16 ONE_BITS = 0x3C00;
+    static constexpr u16 FLOOR_BITS = 0x0001;        // 2^-24, the smallest positive fp16
+    static constexpr u16 BWD_FLOOR_BITS = 0x0C00;    // 2^-12
     static constexpr float MIN_PRODUCT = 0.00390625f;               // 2^-8
     static __device__ __forceinline__ float to_f32(u16 v) { return (float)__builtin_bit_cast(_Float16, v); }
     // products of raw 16-bit values (a fused form with fp16 operands converted on the fly exists,

@@ -804,9 +804,7 @@ __global__ __launch_bounds__(BW_THREADS) void lfw_bwd_chunk_kernel(ChunkBwdArgs 
 template <typename IOE, typename OPE, int NB, bool HEADS> int launch(const ChunkBwdArgs &a, hipStream_t stream) {
     auto kern = lfw_bwd_chunk_kernel<IOE, OPE, NB, HEADS>;
     // more than 64 KB of dynamic LDS has to be enabled per function (and per device)
-    int rc = check_hip(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, BW_SMEM),
-                       "hipFuncSetAttribute(backward chunk kernel)");
+    int rc = enable_lds(reinterpret_cast<const void *>(kern), BW_SMEM, "hipFuncSetAttribute(backward chunk kernel)");
     if (rc) return rc;
     if (a.B > 0x1fffffffLL) return fail(T2FW_ERR_UNSUPPORTED, "B=%lld is too large", (long long)a.B);
     if (a.heads < 1 || a.T * a.heads >= CHUNK_MAX_T)

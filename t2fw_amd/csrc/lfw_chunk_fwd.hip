@@ -113,8 +113,16 @@ __device__ __forceinline__ void raw_issue_tail(RawSet<NV> &r, const u16 *gate, c
 
 template <int NV> struct RawF {
     float gown[8], goth_prod, val[NV][8];
-    u32 bad;      // own gates outside (0, 1]
+    u32 bad;      // own gates outside [0, 1]
 };
+
+// Gates enter the products no smaller than FLOOR_BITS (2^-24): an exactly zero gate, which an fp16
+// sigmoid returns below a logit of about -17, would make the block's prefix products zero and their
+// inverses infinite.  What the floor lets through from before such a step, 2^-24 of the state, is far
+// below the rounding of the 16-bit outputs.
+template <typename IOE> __device__ __forceinline__ u16 floor_gate(u16 bits) {
+    return bits > IOE::FLOOR_BITS ? bits : IOE::FLOOR_BITS;
+}
 
 // Registers -> floats.
 template <typename IOE, int NV> __device__ __forceinline__ RawF<NV> raw_take(const RawSet<NV> &r) {
@@ -125,14 +133,13 @@ template <typename IOE, int NV> __device__ __forceinline__ RawF<NV> raw_take(con
     float po = 1.0f;
 #pragma unroll
     for (int t = 0; t < 8; ++t) {
-        const u16 m1 = (u16)(r.gown[t] - 1);      // gates must lie in (0, 1]: 0 < bits <= bits(1.0)
-        mx = m1 > mx ? m1 : mx;
-        f.gown[t] = IOE::to_f32(r.gown[t]);
-        po *= IOE::to_f32(r.goth[t]);
+        mx = r.gown[t] > mx ? r.gown[t] : mx;     // gates must lie in [0, 1]: bits <= bits(1.0) (negative, NaN: above)
+        f.gown[t] = IOE::to_f32(floor_gate<IOE>(r.gown[t]));
+        po *= IOE::to_f32(floor_gate<IOE>(r.goth[t]));
 #pragma unroll
         for (int a = 0; a < NV; ++a) f.val[a][t] = IOE::to_f32(r.val[a][t]);
     }
-    f.bad = (mx >= IOE::ONE_BITS) ? 1u : 0u;
+    f.bad = (mx > IOE::ONE_BITS) ? 1u : 0u;
     f.goth_prod = po;
     return f;
 }
@@ -145,15 +152,15 @@ __device__ __forceinline__ RawF<NV> raw_take_tail(const RawSet<NV> &r, int tok_o
     float po = 1.0f;
 #pragma unroll
     for (int t = 0; t < 8; ++t) {
-        if (tok_oth + t < T) po *= IOE::to_f32(r.goth[t]);
+        if (tok_oth + t < T) po *= IOE::to_f32(floor_gate<IOE>(r.goth[t]));
         const bool own = tok_own + t < T;
-        const u16 m1 = own ? (u16)(r.gown[t] - 1) : (u16)0;
-        mx = m1 > mx ? m1 : mx;
-        f.gown[t] = own ? IOE::to_f32(r.gown[t]) : 1.0f;
+        const u16 gb = own ? r.gown[t] : (u16)0;
+        mx = gb > mx ? gb : mx;
+        f.gown[t] = own ? IOE::to_f32(floor_gate<IOE>(r.gown[t])) : 1.0f;
 #pragma unroll
         for (int a = 0; a < NV; ++a) f.val[a][t] = own ? IOE::to_f32(r.val[a][t]) : 0.0f;
     }
-    f.bad = (mx >= IOE::ONE_BITS) ? 1u : 0u;
+    f.bad = (mx > IOE::ONE_BITS) ? 1u : 0u;
     f.goth_prod = po;
     return f;
 }
@@ -188,7 +195,7 @@ __device__ __forceinline__ void write_cm8(unsigned char *tile, int c, int tok0, 
 //   pre[t] = prod_{r<=t} gate_r from the block start, hat = v * prod_{r>t} gate_r, til = hat / total.
 template <typename OPE, int NV>
 __device__ __forceinline__ float scale_half(const RawF<NV> &f, int h, float (&pre)[8], float (&hat)[8], float (&til)[8],
-                                            u32 &bad) {
+                                            u32 &bad, float &min_tot) {
     float run = h ? f.goth_prod : 1.0f;
 #pragma unroll
     for (int t = 0; t < 8; ++t) {
@@ -196,7 +203,8 @@ __device__ __forceinline__ float scale_half(const RawF<NV> &f, int h, float (&pr
         pre[t] = run;
     }
     const float tot = h ? run : run * f.goth_prod;
-    bad |= f.bad | ((tot >= OPE::MIN_PRODUCT) ? 0u : 1u);
+    bad |= f.bad;
+    min_tot = fminf(min_tot, tot);       // the smallest 16-step product of the row decides at the end
     const float itot = __builtin_amdgcn_rcpf(tot);
     float sfx = h ? 1.0f : f.goth_prod;
 #pragma unroll
@@ -233,12 +241,13 @@ __device__ __forceinline__ void fwd_prep_side(const ChunkFwdArgs &p, unsigned ch
         oth_off[t] = HEADS ? lane_bytes + 2u * (u32)(8 * (1 - h) + t) * ts : 0u;
     }
     u32 bad = 0;
+    float min_tot = 1.0f;
 
     // this wave's share of the operand tiles of step n
     auto build = [&](const RawF<NV> &f, int n) {
         unsigned char *ops = smem + (n & 3) * OPS_BYTES;
         float pre[8], hat[8], til[8];
-        const float tot = scale_half<OPE, NV>(f, h, pre, hat, til, bad);
+        const float tot = scale_half<OPE, NV>(f, h, pre, hat, til, bad, min_tot);
         const int tok0 = CH_L * hh + 8 * h;
         if constexpr (KEY) {
             float qs[8];
@@ -332,10 +341,13 @@ __device__ __forceinline__ void fwd_prep_side(const ChunkFwdArgs &p, unsigned ch
         build(raw_take_tail<IOE, NV>(r, t_own, t_oth, T), nfull);
         publish(nfull);
     }
-    if (bad) {
+    if (bad || !(min_tot >= OPE::MIN_PRODUCT)) {
         p.row_flags[flag_slot] = 1;
         *reinterpret_cast<volatile int *>(smem + OFF_VERDICT) = 1;
     }
+    // what the chunk-parallel backward will make of this row: with every 16-step product at or above
+    // PAR_HINT_MIN_PRODUCT its products over half a chunk (one or two blocks) are inside its range
+    if (p.par_hint != nullptr && (bad || !(min_tot >= PAR_HINT_MIN_PRODUCT))) p.par_hint[flag_slot] = 1;
 }
 
 template <typename E> __device__ __forceinline__ uint2 pack4(const floatx4 &v) {
@@ -377,6 +389,10 @@ __device__ __forceinline__ void fwd_matrix_waves(const ChunkFwdArgs &p, unsigned
     if (tid == 0) {
         p.row_flags[flag_slot] = 0;
         if (clear_other_slot) p.row_flags[chunk_rows_padded(p.B) + b] = 0;
+        if (p.par_hint != nullptr) {
+            p.par_hint[flag_slot] = 0;
+            if (clear_other_slot) p.par_hint[chunk_rows_padded(p.B) + b] = 0;
+        }
         *reinterpret_cast<volatile int *>(smem + OFF_VERDICT) = 0;
     }
     // One step (two blocks).  FULL: all 32 tokens exist, which leaves the body without a branch
@@ -543,18 +559,14 @@ template <typename IOE, typename OPE, bool HEADS> int launch(const ChunkFwdArgs 
     // more than 64 KB of dynamic LDS has to be enabled per function (and per device)
     if (split) {
         auto kern = lfw_fwd_chunk_half_kernel<IOE, OPE, HEADS>;
-        int rc = check_hip(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
-                                               hipFuncAttributeMaxDynamicSharedMemorySize, FWD_SMEM),
-                           "hipFuncSetAttribute(forward chunk kernel, two workgroups per row)");
+        int rc = enable_lds(reinterpret_cast<const void *>(kern), FWD_SMEM, "hipFuncSetAttribute(forward chunk kernel, two workgroups per row)");
         if (rc) return rc;
         const int rows_padded = (int)chunk_rows_padded(a.B);
         hipLaunchKernelGGL(kern, dim3(2u * (unsigned)rows_padded), dim3(FWD_THREADS_HALF), FWD_SMEM, stream, a, rows_padded);
         return check_hip(hipGetLastError(), "lfw_fwd_chunk_half_kernel launch");
     }
     auto kern = lfw_fwd_chunk_kernel<IOE, OPE, HEADS>;
-    int rc = check_hip(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, FWD_SMEM),
-                       "hipFuncSetAttribute(forward chunk kernel)");
+    int rc = enable_lds(reinterpret_cast<const void *>(kern), FWD_SMEM, "hipFuncSetAttribute(forward chunk kernel)");
     if (rc) return rc;
     hipLaunchKernelGGL(kern, dim3((unsigned)a.B), dim3(FWD_THREADS), FWD_SMEM, stream, a);
     return check_hip(hipGetLastError(), "lfw_fwd_chunk_kernel launch");

@@ -191,10 +191,20 @@ __device__ __forceinline__ void load_tokens(RawTokens<NT> &r, const u16 *ubase, 
 
 // Gates -> prefix products (and the range verdict).  FULL = false: tokens at or past n_left act as
 // identity (gate 1).
+//
+// Gates below 2^-12 (an exactly zero gate above all, which an fp16 sigmoid returns below a logit of
+// about -17) enter as 2^-12.  The forward's state after such a step holds at most 2^-24 of what was there
+// before it; here 2^-12 of it leaks through, 2.4e-4 of a term that the operands' bf16 rounding already
+// perturbs by 2^-9.  The floor is this high for the gate gradient of that very step: gate * d_gate is
+// what the sweeps produce (lfw_par_bwd.hip), with an absolute error of fp32 rounding (2^-24) of the
+// terms that cancel in it, and d_gate = that / gate with the floored gate is then good to 2^-12 of those
+// terms.  (d_gate at a step does not depend on the step's own gate, so the floored gate gives the right
+// value.)
 template <typename IOE, int NT, bool FULL>
 __device__ __forceinline__ void gate_scan(LaneChunk<NT> &lc, float (&gate)[NT][4], const RawTokens<NT> &raw, int kg,
                                           int n_left) {
-    us2 mx = {0, 0}, mn = {0xffff, 0xffff};
+    us2 mx = {0, 0};
+    const us2 floor_bits = {IOE::BWD_FLOOR_BITS, IOE::BWD_FLOOR_BITS};
 #pragma unroll
     for (int m = 0; m < NT; ++m)
 #pragma unroll
@@ -205,7 +215,7 @@ __device__ __forceinline__ void gate_scan(LaneChunk<NT> &lc, float (&gate)[NT][4
                 if (!(16 * m + 2 * jj + 1 < n_left)) bits.y = IOE::ONE_BITS;
             }
             mx = __builtin_elementwise_max(mx, bits);      // > bits(1.0): above one, negative, NaN
-            mn = __builtin_elementwise_min(mn, bits);      // 0: a zero gate
+            bits = __builtin_elementwise_max(bits, floor_bits);      // gates in [0, 2^-12) count as 2^-12
             gate[m][2 * jj] = IOE::to_f32(bits.x);
             gate[m][2 * jj + 1] = IOE::to_f32(bits.y);
         }
@@ -226,8 +236,8 @@ __device__ __forceinline__ void gate_scan(LaneChunk<NT> &lc, float (&gate)[NT][4
     }
     lc.tot = carry;
     lc.sfx = second;
-    const u16 hi = mx.x > mx.y ? mx.x : mx.y, lo = mn.x < mn.y ? mn.x : mn.y;
-    lc.bad = (hi > IOE::ONE_BITS || lo == 0 || !(lc.ref >= PAR_MIN_PRODUCT) || !(second >= PAR_MIN_PRODUCT)) ? 1u : 0u;
+    const u16 hi = mx.x > mx.y ? mx.x : mx.y;
+    lc.bad = (hi > IOE::ONE_BITS || !(lc.ref >= PAR_MIN_PRODUCT) || !(second >= PAR_MIN_PRODUCT)) ? 1u : 0u;
 }
 
 // 1 / pre: one reciprocal per run of four tokens, the others by multiplying the gates back in

@@ -523,8 +523,7 @@ template <typename IOE, int NT, bool HEADS> int launch(const ParBwdArgs &a, hipS
     auto incr = lfw_par_incr_kernel<IOE, NT, HEADS>;
     auto scan = lfw_par_scan_kernel<IOE>;
     auto grads = lfw_par_grads_kernel<IOE, NT, HEADS>;
-    int rc = check_hip(hipFuncSetAttribute(reinterpret_cast<const void *>(grads), hipFuncAttributeMaxDynamicSharedMemorySize, GR_SMEM),
-                       "hipFuncSetAttribute(gradient kernel)");
+    int rc = enable_lds(reinterpret_cast<const void *>(grads), GR_SMEM, "hipFuncSetAttribute(gradient kernel)");
     if (rc) return rc;
     const int64_t items = a.B * a.NC;
     if (items > 0x3fffffffLL || a.B > 0x0fffffffLL) return fail(T2FW_ERR_UNSUPPORTED, "B * chunks = %lld is too large", (long long)items);

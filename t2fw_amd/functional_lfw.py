@@ -10,12 +10,14 @@ Differences from the reference that a caller can observe:
   * kernels run on the current torch stream and on the inputs' device.
 """
 import contextlib
+import ctypes
 import functools
 import os
 
 import torch
 
 from . import _lib
+from .path_hint import ForwardHints, choose_backward_flags
 
 DEFAULT_CKPT_INTERVAL = 64
 
@@ -35,11 +37,18 @@ def _flags():
 
 @functools.lru_cache(maxsize=256)
 def _sizes(rows, T, D, K, C, code, flags):
-    """(checkpoints per row, forward workspace bytes, forward + backward workspace bytes) of a shape:
-    three calls into the library that a training loop would otherwise repeat every step"""
+    """(checkpoints per row, forward workspace bytes, forward + backward workspace bytes, flag regions)
+    of a shape: calls into the library that a training loop would otherwise repeat every step"""
     lib = _lib.load()
+    regions = (ctypes.c_int64 * 6)()
+    _lib.check(lib.t2fw_lfw_flag_regions(rows, T, D, K, C, code, flags, regions))
     return (lib.t2fw_lfw_num_ckpt(T, C), lib.t2fw_lfw_forward_workspace_bytes(rows, T, D, K, C, code, flags),
-            lib.t2fw_lfw_workspace_bytes(rows, T, D, K, C, code, flags))
+            lib.t2fw_lfw_workspace_bytes(rows, T, D, K, C, code, flags), tuple(regions))
+
+
+def _host_hints_enabled():
+    """T2FW_HOST_HINTS=0 keeps every workspace in device memory (the backward then decides on the device)."""
+    return os.environ.get("T2FW_HOST_HINTS", "1") != "0"
 
 
 def _on_device(dev):
@@ -68,7 +77,8 @@ def _lfw_forward(value, forget, query, key, f_key, state, need_grad, heads=False
     """Checks as in t2fw/functional_lfw.py:42-49 and t2fw/csrc/lfw.cpp:24-26,36-41, then the forward
     kernels.  heads=False: x,f [B,T,D]; q,k,f_key [B,T,K]; state [B,D,K].  heads=True: x,f [B,T,H,D];
     q,k,f_key [B,T,H,K]; state [B,H,D,K].  Returns (outputs, next_state, ckpt or None, checkpoint
-    interval, flags)."""
+    interval, flags, hints): ``hints`` is None, or the forward's verdict on which backward path the
+    gates allow, readable from the host once the forward has run (path_hint.py)."""
     assert value.shape == forget.shape
     assert query.shape == key.shape
     assert query.shape == f_key.shape
@@ -96,26 +106,37 @@ def _lfw_forward(value, forget, query, key, f_key, state, need_grad, heads=False
     C = _ckpt_interval()
     flags = _flags()
     dev = value.device
-    nc, ws_bytes, _ = _sizes(B * H, T, D, K, C, code, flags)
+    nc, ws_bytes, _, regions = _sizes(B * H, T, D, K, C, code, flags)
     with _on_device(dev):
         outputs = torch.empty_like(value)
         next_state = torch.empty_like(state)
         ckpt = None
         if need_grad:
             ckpt = torch.empty((B * H, nc, D, K), dtype=value.dtype, device=dev)
-        ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev) if ws_bytes else None
+        hints = None
+        if need_grad and ws_bytes and regions[3] and regions[5] and _host_hints_enabled() and ForwardHints.usable(dev):
+            # a backward on the matrix cores will follow: the workspace goes to pinned host memory
+            hints = ForwardHints(dev, ws_bytes, regions[2], regions[3], B * H)
+            ws_ptr = hints.workspace()[0]
+        else:
+            ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev) if ws_bytes else None
+            ws_ptr = _lib.ptr(ws)
         ptrs = (_lib.ptr(value), _lib.ptr(forget), _lib.ptr(query), _lib.ptr(key), _lib.ptr(f_key),
                 _lib.ptr(state), _lib.ptr(outputs), _lib.ptr(next_state), _lib.ptr(ckpt))
-        tail = (D, K, C, code, flags, _lib.ptr(ws), ws_bytes, _lib.current_stream_handle(dev))
+        tail = (D, K, C, code, flags, ws_ptr, ws_bytes, _lib.current_stream_handle(dev))
         if heads:
             _lib.check(lib.t2fw_lfw_forward_heads(*ptrs, B, T, H, *tail))
         else:
             _lib.check(lib.t2fw_lfw_forward(*ptrs, B, T, *tail))
-    return outputs, next_state, ckpt, C, flags
+        if hints is not None:
+            hints.launched()
+    return outputs, next_state, ckpt, C, flags, hints
 
 
-def _lfw_backward(grad_output, grad_state, value, forget, query, key, f_key, state, ckpt, C, flags, heads=False):
-    """The backward kernels; gradients in the order of t2fw/csrc/lfw.cpp:95, laid out as their inputs."""
+def _lfw_backward(grad_output, grad_state, value, forget, query, key, f_key, state, ckpt, C, flags, heads=False,
+                  hints=None):
+    """The backward kernels; gradients in the order of t2fw/csrc/lfw.cpp:95, laid out as their inputs.
+    ``hints``: what the forward call on the same gates left for this call (path_hint.py), or None."""
     # t2fw/functional_lfw.py:71-72
     assert grad_state.dtype == value.dtype
     assert grad_output.dtype == value.dtype
@@ -127,6 +148,8 @@ def _lfw_backward(grad_output, grad_state, value, forget, query, key, f_key, sta
     code = _dtype_code(value.dtype)
     lib = _lib.load()
     dev = value.device
+    if hints is not None:
+        flags = choose_backward_flags(flags, hints.hinted_rows(), B * H)
     ws_bytes = _sizes(B * H, T, D, K, C, code, flags)[2]
     with _on_device(dev):
         d_x = torch.empty_like(value)
@@ -155,18 +178,19 @@ class LFWFunction(torch.autograd.Function):
     def forward(ctx, value, forget, query, key, f_key, state):
         """Return: (outputs [B,T,D], final state [B,D,K])"""
         need_grad = any(ctx.needs_input_grad)
-        outputs, next_state, ckpt, C, flags = _lfw_forward(value, forget, query, key, f_key, state, need_grad)
+        outputs, next_state, ckpt, C, flags, hints = _lfw_forward(value, forget, query, key, f_key, state, need_grad)
         if need_grad:
             ctx.save_for_backward(value, forget, query, key, f_key, state, ckpt)
             ctx.ckpt_interval = C
             ctx.flags = flags
+            ctx.hints = hints
         return outputs, next_state
 
     @staticmethod
     def backward(ctx, grad_output, grad_state):
         value, forget, query, key, f_key, state, ckpt = ctx.saved_tensors
         return _lfw_backward(grad_output, grad_state, value, forget, query, key, f_key, state, ckpt,
-                             ctx.ckpt_interval, ctx.flags)
+                             ctx.ckpt_interval, ctx.flags, hints=ctx.hints)
 
 
 def sigmoid_gates(f_logit, fk_logit, out_f=None, out_fk=None):
@@ -208,18 +232,19 @@ class LFWGatedFunction(torch.autograd.Function):
         assert f_logit.dtype == value.dtype and fk_logit.dtype == value.dtype
         forget, f_key = sigmoid_gates(f_logit, fk_logit)
         need_grad = any(ctx.needs_input_grad)
-        outputs, next_state, ckpt, C, flags = _lfw_forward(value, forget, query, key, f_key, state, need_grad)
+        outputs, next_state, ckpt, C, flags, hints = _lfw_forward(value, forget, query, key, f_key, state, need_grad)
         if need_grad:
             ctx.save_for_backward(value, forget, query, key, f_key, state, ckpt)
             ctx.ckpt_interval = C
             ctx.flags = flags
+            ctx.hints = hints
         return outputs, next_state
 
     @staticmethod
     def backward(ctx, grad_output, grad_state):
         value, forget, query, key, f_key, state, ckpt = ctx.saved_tensors
         d_x, d_f, d_q, d_k, d_fk, d_s = _lfw_backward(grad_output, grad_state, value, forget, query, key, f_key,
-                                                      state, ckpt, ctx.ckpt_interval, ctx.flags)
+                                                      state, ckpt, ctx.ckpt_interval, ctx.flags, hints=ctx.hints)
         _gate_backward_inplace(d_f, d_fk, forget, f_key)
         return d_x, d_f, d_q, d_k, d_fk, d_s
 
@@ -242,12 +267,13 @@ class LFWHeadsFunction(torch.autograd.Function):
             assert forget.dtype == value.dtype and f_key.dtype == value.dtype
             forget, f_key = sigmoid_gates(forget, f_key)
         need_grad = any(ctx.needs_input_grad)
-        outputs, next_state, ckpt, C, flags = _lfw_forward(value, forget, query, key, f_key, state, need_grad,
-                                                           heads=True)
+        outputs, next_state, ckpt, C, flags, hints = _lfw_forward(value, forget, query, key, f_key, state, need_grad,
+                                                                  heads=True)
         if need_grad:
             ctx.save_for_backward(value, forget, query, key, f_key, state, ckpt)
             ctx.ckpt_interval = C
             ctx.flags = flags
+            ctx.hints = hints
             ctx.logits = bool(logits)
         return outputs, next_state
 
@@ -255,7 +281,8 @@ class LFWHeadsFunction(torch.autograd.Function):
     def backward(ctx, grad_output, grad_state):
         value, forget, query, key, f_key, state, ckpt = ctx.saved_tensors
         d_x, d_f, d_q, d_k, d_fk, d_s = _lfw_backward(grad_output, grad_state, value, forget, query, key, f_key,
-                                                      state, ckpt, ctx.ckpt_interval, ctx.flags, heads=True)
+                                                      state, ckpt, ctx.ckpt_interval, ctx.flags, heads=True,
+                                                      hints=ctx.hints)
         if ctx.logits:
             _gate_backward_inplace(d_f, d_fk, forget, f_key)
         return d_x, d_f, d_q, d_k, d_fk, d_s, None

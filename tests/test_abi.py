@@ -45,7 +45,7 @@ def test_binding_covers_every_declared_symbol():
 
 
 def test_abi_version_and_ckpt_count(lib):
-    assert lib.t2fw_abi_version() == 2
+    assert lib.t2fw_abi_version() == 3
     assert lib.t2fw_lfw_num_ckpt(1024, 64) == 16
     assert lib.t2fw_lfw_num_ckpt(1025, 64) == 17
     assert lib.t2fw_lfw_num_ckpt(1, 64) == 1

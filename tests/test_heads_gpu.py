@@ -125,7 +125,7 @@ def test_flagged_rows_are_redone_by_the_exact_kernels_in_place():
     B, H, T = 2, 3, 90
     x, f, q, k, fk, s, go, gs = make_config_inputs(B * H, T, 64, 64, torch.float16, seed=11, state_std=0.3)
     f, fk = f.clone(), fk.clone()
-    f[1, 40, 9] = 0.0                  # batch 0, head 1
+    f[1, 40, 9] = -0.0                 # batch 0, head 1
     fk[5, 89, 63] = 2.0                # batch 1, head 2, in the partial last block
     check_heads((x, f, q, k, fk, s), go, gs, B, H, 32, torch.float16, expect_flagged=2)
 
@@ -135,7 +135,7 @@ def test_flagged_rows_with_one_workgroup_per_row():
     x, f, q, k, fk, s, go, gs = make_config_inputs(B * H, T, 64, 64, torch.bfloat16, seed=19, gate_mean=3.0,
                                                     state_std=0.3)
     f, fk = f.clone(), fk.clone()
-    f[137, 69, 33] = 0.0               # last row, last token
+    f[137, 69, 33] = -0.0              # last row, last token
     fk[6, 0, 0] = -1.0                 # batch 1, head 0, first token
     check_heads((x, f, q, k, fk, s), go, gs, B, H, 64, torch.bfloat16, expect_flagged=2,
                 oracle_rows=[0, 5, 6, 7, 136, 137])

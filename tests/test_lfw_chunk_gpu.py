@@ -148,7 +148,7 @@ def test_batch_larger_than_half_the_device():
     x, f, q, k, fk, s, go, gs = make_config_inputs(B, T, 64, 64, torch.float16, seed=31, state_std=0.2)
     f = f.clone()
     f[135, 70, 50] = 1.25               # rows for the exact recurrence: one in the last workgroup,
-    f[64, 3, 7] = 0.0                   # one whose chunked form divides by zero
+    f[64, 3, 7] = -0.0                  # one with a sign bit (a plain zero gate stays on the matrix cores)
     out, nxt, ckpt, grads, flagged = run_abi((x, f, q, k, fk, s), go, gs, 64)
     assert flagged == (2, 2), flagged
     rows = [0, 63, 64, 127, 128, 135]
@@ -171,7 +171,7 @@ def test_flagged_rows_with_a_partial_last_block():
     B, T = 3, 90
     x, f, q, k, fk, s, go, gs = make_config_inputs(B, T, 64, 64, torch.float16, seed=11, state_std=0.3)
     f, fk = f.clone(), fk.clone()
-    f[0, 40, 9] = 0.0
+    f[0, 40, 9] = -0.0
     fk[2, 89, 63] = 2.0                 # in the partial last block
     out, nxt, ckpt, grads, flagged = run_abi((x, f, q, k, fk, s), go, gs, 32)
     assert flagged == (2, 2), flagged
@@ -187,7 +187,7 @@ def test_no_fixup_flag_reports_but_does_not_repair():
     B, T = 2, 64
     x, f, q, k, fk, s, go, gs = make_config_inputs(B, T, 64, 64, torch.float16, seed=12, state_std=0.3)
     f = f.clone()
-    f[1, 5, 2] = 0.0
+    f[1, 5, 2] = -0.0
     out, nxt, ckpt, grads, flagged = run_abi((x, f, q, k, fk, s), go, gs, 64, flags=_lib.FLAG_NO_FIXUP)
     assert flagged == (1, 1), flagged
     # the unflagged row is valid without the exact kernels having run
@@ -214,16 +214,16 @@ def test_reference_test_gates_stay_on_the_chunked_path():
                          expect_flagged_parallel=2, gate_tol=(2e-1, 4e-2), reference_bounds=False)
 
 
-@pytest.mark.parametrize("kind", ["zero_gate", "zero_gate_upper_channels", "gate_above_one", "negative_gate",
+@pytest.mark.parametrize("kind", ["negative_zero_gate", "negative_zero_gate_upper_channels", "gate_above_one", "negative_gate",
                                   "tiny_product", "nan_free_inf_gate"])
 def test_rows_outside_the_gate_range_fall_back_to_the_exact_kernels(kind):
     B, T = 4, 160
     x, f, q, k, fk, s, go, gs = make_config_inputs(B, T, 64, 64, torch.float16, seed=3, state_std=0.3)
     f, fk = f.clone(), fk.clone()
-    if kind == "zero_gate":
-        f[1, 70, 5] = 0.0
-    elif kind == "zero_gate_upper_channels":
-        f[1, 70, 40] = 0.0              # seen only by the workgroup that owns value channels 32..63
+    if kind == "negative_zero_gate":            # the range check is on the bits: a sign bit is outside [0, 1]
+        f[1, 70, 5] = -0.0
+    elif kind == "negative_zero_gate_upper_channels":
+        f[1, 70, 40] = -0.0             # seen only by the workgroup that owns value channels 32..63
     elif kind == "gate_above_one":
         fk[1, 3, 60] = 1.5
     elif kind == "negative_gate":
@@ -241,7 +241,7 @@ def test_rows_outside_the_gate_range_fall_back_to_the_exact_kernels(kind):
     # the others.  The backward redoes the whole row from the checkpoints the forward left, so its
     # value-side results are tight on the same channels and its key-side results (sums over all
     # value channels) are tight when the whole row was redone.
-    exact = {"zero_gate": slice(0, 32), "zero_gate_upper_channels": slice(32, 64), "negative_gate": slice(0, 32),
+    exact = {"negative_zero_gate": slice(0, 32), "negative_zero_gate_upper_channels": slice(32, 64), "negative_gate": slice(0, 32),
              "nan_free_inf_gate": slice(0, 32)}.get(kind, slice(0, 64))
     whole = exact == slice(0, 64)
     r_out, r_nxt = c_oracle.lfw_forward(x, f, q, k, fk, s)

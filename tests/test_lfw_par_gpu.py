@@ -45,7 +45,7 @@ def test_more_items_than_compute_units():
     B, T = 300, 130
     x, f, q, k, fk, s, go, gs = make_config_inputs(B, T, 64, 64, torch.float16, seed=41, state_std=0.2)
     f = f.clone()
-    f[299, 129, 63] = 0.0               # the last token of the last row, in a chunk of two tokens
+    f[299, 129, 63] = -0.0              # the last token of the last row, in a chunk of two tokens
     f[150, 64, 0] = 1.5
     out, nxt, ckpt, grads, flagged = run_abi((x, f, q, k, fk, s), go, gs, 64)
     assert flagged == (2, 2), flagged
@@ -92,13 +92,13 @@ def test_half_chunk_products_below_the_range_are_flagged_in_the_backward_only(wh
 
 def test_rows_that_neither_matrix_core_form_takes_reach_the_exact_scan():
     """a row with small gates over half a chunk (declined by the chunk-parallel form only) next to a row
-    with a 16-step product below the block-wise form's limit and a row with a zero gate"""
+    with a 16-step product below the block-wise form's limit and a row with a gate that has a sign bit"""
     B, T, C = 4, 256, 64
     x, f, q, k, fk, s, go, gs = make_config_inputs(B, T, 64, 64, torch.float16, seed=21, state_std=0.3)
     f, fk = f.clone(), fk.clone()
     f[0, 64:96, 3] = 0.15               # 2^-87.6 over half a chunk, 2^-43.8 per block
     fk[1, 128:144, 9] = 0.01            # 2^-106 in one block
-    f[3, 200, 60] = 0.0
+    f[3, 200, 60] = -0.0
     out, nxt, ckpt, grads, flagged = run_abi((x, f, q, k, fk, s), go, gs, C)
     assert flagged[1] == 3 and flagged.exact == 2, (flagged, flagged.exact)
     (r_out, r_nxt), r_grads = oracle((x, f, q, k, fk, s), go, gs)
@@ -117,7 +117,7 @@ def test_small_gates_across_a_half_chunk_boundary_are_accepted():
 
 
 @pytest.mark.parametrize("chunk", [0, 15, 16, 17, 36])
-@pytest.mark.parametrize("bad", [0.0, -0.25, 1.0625])
+@pytest.mark.parametrize("bad", [-0.0, -0.25, 1.0625])
 def test_a_gate_outside_the_range_in_any_chunk_flags_the_row(chunk, bad):
     B, C = 3, 32
     T = 37 * C - 5
@@ -152,7 +152,7 @@ def test_flags_are_forgotten_between_calls_on_one_workspace():
     B, T, C = 2, 128, 64
     x, f, q, k, fk, s, go, gs = make_config_inputs(B, T, 64, 64, torch.float16, seed=37, state_std=0.3)
     bad_f = f.clone()
-    bad_f[0, 3, 3] = 0.0
+    bad_f[0, 3, 3] = -0.0
     code = _lib.DTYPE_CODE[x.dtype]
     wsb = lib.t2fw_lfw_workspace_bytes(B, T, 64, 64, C, code, 0)
     ws = torch.zeros(wsb, dtype=torch.uint8, device="cuda")
