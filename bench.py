@@ -64,36 +64,24 @@ def algorithmic_bytes(B, T, D, K, es, C, backward):
     return fwd, bwd
 
 
-def main():
-    ap = argparse.ArgumentParser()
-    ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=200)
-    ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", default="cfg3", choices=sorted(WORKLOADS) + ["dfw", "copy256", "copy64"])
-    ap.add_argument("--ckpt-interval", type=int, default=64)
-    ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--force-scan", action="store_true", help="exact scan kernels only")
-    args = ap.parse_args()
-    if args.gpus != 1:
-        print("bench.py: this build measures one GPU only (the path shards over the batch with no "
-              "exchange); run with --gpus 1", file=sys.stderr)
-        sys.exit(2)
+def percentiles(v):
+    """median, 20th and 80th percentile (the three figures the reference's do_bench returns,
+    tests/benchmark.py:66-71)"""
+    import numpy as np
+    a = np.asarray(v, dtype=np.float64)
+    return {"p50": round(float(np.percentile(a, 50)), 5), "p20": round(float(np.percentile(a, 20)), 5),
+            "p80": round(float(np.percentile(a, 80)), 5)}
 
+
+def bench_lfw(args, name, steps, warmup, extras, max_sets=16, gates="config"):
+    """Forward (+ backward) of the decay rule through the C ABI on workload `name`; returns the JSON line
+    as a dict.  extras: also the autograd leg, the CPU baseline and the parity report."""
     import torch
     from t2fw_amd import _lib
-    from t2fw_amd.synthetic import make_config_inputs
+    from t2fw_amd.synthetic import make_config_inputs, make_reference_test_inputs
 
-    if not torch.cuda.is_available():
-        print("bench.py: no GPU visible", file=sys.stderr)
-        sys.exit(1)
-    if args.workload == "cfg5":
-        return bench_generation(args)
-    if args.workload in ("copy256", "copy64"):
-        return bench_copy(args)
-    if args.workload == "dfw":
-        return bench_dfw(args)
     lib = _lib.load()
-    w = WORKLOADS[args.workload]
+    w = WORKLOADS[name]
     B, T, D, K = w["B"], w["T"], w["D"], w["K"]
     H = w.get("H")                     # None: folded rows [B, T, D]; else rows are the heads of [B / H, T, H, D] tensors
     dtype = getattr(torch, w["dtype"])
@@ -108,13 +96,17 @@ def main():
     # several independent input sets so that consecutive steps do not re-read the same
     # lines out of the 256 MB last-level cache
     per_set = (5 * B * T * D + (B * T * D if backward else 0)) * es * (2 if backward else 1) + 2 * B * T * D * es
-    nsets = max(2, min(16, int(1.2e9 // max(per_set, 1)) + 1))
+    nsets = max(2, min(max_sets, int(1.2e9 // max(per_set, 1)) + 1))
     sets = []
     nc = lib.t2fw_lfw_num_ckpt(T, C)
     ws_bytes = lib.t2fw_lfw_workspace_bytes(B, T, D, K, C, code, flags)
     for i in range(nsets):
-        x, f, q, k, fk, s, go, gs = make_config_inputs(B, T, D, K, dtype, seed=i, gate_mean=w["gate_mean"],
-                                                        state_std=w["state_std"])
+        if gates == "reference_test":      # per-channel constant gates in (1/64, 63/64), tests/test_lfw.py:10-16
+            x, f, q, k, fk, s, go, gs = make_reference_test_inputs(B, T, D, K, dtype, seed=i)
+            x, q, k = x / 8, q / 8, k / 8
+        else:
+            x, f, q, k, fk, s, go, gs = make_config_inputs(B, T, D, K, dtype, seed=i, gate_mean=w["gate_mean"],
+                                                            state_std=w["state_std"])
         if H:
             heads = lambda t: t.view(B // H, H, T, t.shape[2]).transpose(1, 2).contiguous()
             x, f, q, k, fk, go = (heads(t) for t in (x, f, q, k, fk, go))
@@ -132,16 +124,17 @@ def main():
     lfw_forward = lib.t2fw_lfw_forward_heads if H else lib.t2fw_lfw_forward
     lfw_backward = lib.t2fw_lfw_backward_heads if H else lib.t2fw_lfw_backward
 
-    def fwd(d):
+    def fwd(d, fl=None):
         _lib.check(lfw_forward(*[_lib.ptr(t) for t in d["ins"]], _lib.ptr(d["out"]), _lib.ptr(d["nxt"]),
-                               _lib.ptr(d.get("ckpt")), *dims, C, code, flags, _lib.ptr(d["ws"]), ws_bytes, stream))
+                               _lib.ptr(d.get("ckpt")), *dims, C, code, flags if fl is None else fl,
+                               _lib.ptr(d["ws"]), ws_bytes, stream))
 
-    def bwd(d):
+    def bwd(d, fl=None):
         i = d["ins"]
         g = d["grads"]
         _lib.check(lfw_backward(_lib.ptr(d["go"]), _lib.ptr(d["gs"]), *[_lib.ptr(t) for t in i],
                                 _lib.ptr(d["ckpt"]), *[_lib.ptr(t) for t in g], *dims, C, code,
-                                flags, _lib.ptr(d["ws"]), ws_bytes, stream))
+                                flags if fl is None else fl, _lib.ptr(d["ws"]), ws_bytes, stream))
 
     def step(i):
         d = sets[i % nsets]
@@ -149,69 +142,97 @@ def main():
         if backward:
             bwd(d)
 
-    for i in range(args.warmup):
+    # The timed region: the calls as the library ships them by default (flags 0: every decision about
+    # flagged rows is taken on the device, which for the backward includes its launch for flagged rows).
+    for i in range(warmup):
         step(i)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    for i in range(args.steps):
+    for i in range(steps):
         step(i)
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
-    ms_per_step = wall / args.steps * 1e3
-    mtok = B * T * args.steps / wall / 1e6
+    ms_per_step = wall / steps * 1e3
+    mtok = B * T * steps / wall / 1e6
 
     # per-call durations with events on the launch stream (same stream torch uses)
-    nrep = min(args.steps, 100)
+    nrep = min(steps, 100)
 
     def timed_calls(call_flags):
-        nonlocal flags
-        saved, flags = flags, call_flags
         ev = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(nrep)]
         for i in range(nrep):
             d = sets[i % nsets]
             ev[i][0].record()
-            fwd(d)
+            fwd(d, call_flags)
             ev[i][1].record()
             if backward:
-                bwd(d)
+                bwd(d, call_flags)
             ev[i][2].record()
         torch.cuda.synchronize()
-        flags = saved
-        return (sum(e[0].elapsed_time(e[1]) for e in ev) / nrep, sum(e[1].elapsed_time(e[2]) for e in ev) / nrep)
+        return [e[0].elapsed_time(e[1]) for e in ev], [e[1].elapsed_time(e[2]) for e in ev]
 
-    fwd_avg, bwd_avg = timed_calls(flags)
-    # the matrix-core kernel alone: the same calls without the exact-kernel launch that follows
-    # the backward (no row of this workload is flagged, so the results are the same)
-    fwd_kern, bwd_kern = (fwd_avg, bwd_avg) if args.force_scan else timed_calls(flags | _lib.FLAG_NO_FIXUP)
+    fwd_ms, bwd_ms = timed_calls(flags)
+    fwd_avg, bwd_avg = sum(fwd_ms) / nrep, sum(bwd_ms) / nrep
     fwd_bytes, bwd_bytes = algorithmic_bytes(B, T, D, K, es, C, backward)
-    if backward and bwd_kern >= fwd_kern:
-        dom, dom_bytes, dom_ms = "backward", bwd_bytes, bwd_kern
+    if backward and bwd_avg >= fwd_avg:
+        dom, dom_bytes, dom_ms, dom_all = "backward", bwd_bytes, bwd_avg, bwd_ms
     else:
-        dom, dom_bytes, dom_ms = "forward", fwd_bytes, fwd_kern
+        dom, dom_bytes, dom_ms, dom_all = "forward", fwd_bytes, fwd_avg, fwd_ms
     achieved = dom_bytes / (dom_ms * 1e-3) / 1e9
-    traffic = None
-    tpath = os.path.join(ROOT, "profiles", "traffic_%s.json" % args.workload)
-    if os.path.exists(tpath):
+    traffic, traffic_source = None, None
+    tpath = os.path.join(ROOT, "profiles", "traffic_%s.json" % name)
+    if os.path.exists(tpath) and gates == "config":
         try:
             traffic = json.load(open(tpath)).get(dom)
+            traffic_source = "profiles/traffic_%s.json (rocprofv3 FETCH_SIZE / WRITE_SIZE of the same launches, static: not measured in this run)" % name
         except Exception:
             traffic = None
-    # which launches `dom` stands for (the names under which rocprofv3 lists them)
-    flags_now = flags
+    chunk_parallel = C in (32, 64) and not flags & (_lib.FLAG_BLOCKWISE | _lib.FLAG_FP16_OPERANDS)
     if dom == "forward":
         launches = ["lfw_fwd_scan_kernel"] if args.force_scan else ["lfw_fwd_chunk_half_kernel" if 2 * ((B + 7) // 8 * 8) <= 256
                                                                     else "lfw_fwd_chunk_kernel"]
     elif args.force_scan:
         launches = ["lfw_bwd_scan_kernel (value side)", "lfw_bwd_scan_kernel (key side)"]
-    elif C in (32, 64) and not flags_now & (_lib.FLAG_BLOCKWISE | _lib.FLAG_FP16_OPERANDS):
-        launches = ["lfw_par_incr_kernel", "lfw_par_scan_kernel", "lfw_par_grads_kernel"]
+    elif chunk_parallel:
+        launches = ["lfw_par_incr_kernel", "lfw_par_scan_kernel", "lfw_par_grads_kernel",
+                    "lfw_bwd_chunk_kernel (rows the first three flagged)"]
     else:
         launches = ["lfw_bwd_chunk_kernel"]
     roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic, "kernel": dom, "launches": launches,
-                "call_with_fixup_launch_ms": round(bwd_avg if dom == "backward" else fwd_avg, 5),
-                "algorithmic_bytes": dom_bytes, "avg_launch_ms": round(dom_ms, 5)}
+                "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic, "traffic_source": traffic_source,
+                "kernel": dom, "launches": launches, "call": "as shipped (flags 0)",
+                "algorithmic_bytes": dom_bytes, "avg_launch_ms": round(dom_ms, 5), "launch_ms": percentiles(dom_all)}
+    if backward and not args.force_scan:
+        # the same calls when the caller knows that no row will be flagged (what LFWFunction passes once the
+        # forward's hints have reached the host): the backward's launch for flagged rows is left out
+        _, nf = timed_calls(flags | _lib.FLAG_NO_FIXUP)
+        roofline["backward_no_fixup_ms"] = round(sum(nf) / nrep, 5)
+        roofline["frac_no_fixup"] = round(bwd_bytes / (sum(nf) / nrep * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)
     whole = (fwd_bytes + bwd_bytes) / (ms_per_step * 1e-3) / 1e9
+
+    line = {
+        "metric": "fwd+bwd Mtokens/s + % HBM roofline, B*H=96 T=1024 d=kdim=64 fp16" if name == "cfg3" and gates == "config"
+                  else "Mtokens/s (%s)" % name,
+        "value": round(mtok, 1), "unit": "Mtokens/s", "n_gpus": 1, "steps": steps, "warmup": warmup,
+        "ms_per_step": round(ms_per_step, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": {"float16": "fp16", "bfloat16": "bf16"}[w["dtype"]] + (
+            " I/O, fp32 state" if args.force_scan else " I/O, bf16 MFMA operands, fp32 accumulate"),
+        "data": "synthetic",
+        "config": {"workload": "%s: B=%d T=%d D=%d K=%d %s %s, checkpoint interval %d%s" % (
+            name, B, T, D, K, w["dtype"], "fwd+bwd" if backward else "fwd", C,
+            ", gates as the reference's tests build them" if gates == "reference_test" else ""),
+            "input_sets_rotated": nsets, "path": "scan" if args.force_scan else "auto"},
+        "whole_step_algorithmic_GBs": round(whole, 1),
+        "whole_step_roofline_frac": round(whole / HBM_PEAK_GBS, 4),
+        "forward_avg_ms": round(fwd_avg, 5), "backward_avg_ms": round(bwd_avg, 5) if backward else None,
+        "forward_ms": percentiles(fwd_ms), "backward_ms": percentiles(bwd_ms) if backward else None,
+        "roofline": roofline,
+    }
+    if gates == "reference_test" and backward:
+        _, bw = timed_calls(flags | _lib.FLAG_BLOCKWISE)
+        line["backward_blockwise_ms"] = round(sum(bw) / nrep, 5)      # what the forward's hints make LFWFunction choose
+    if not extras:
+        return line
 
     # the same step through the autograd API (allocations and Python dispatch included)
     autograd = None
@@ -231,7 +252,7 @@ def main():
             astep(i)
         torch.cuda.synchronize()
         t0 = time.perf_counter()
-        n_a = min(args.steps, 50)
+        n_a = min(steps, 50)
         for i in range(n_a):
             astep(i)
         torch.cuda.synchronize()
@@ -258,6 +279,7 @@ def main():
         torch.cuda.synchronize()
         autograd["graph_replay_ms_per_step"] = round((time.perf_counter() - t0) / n_a * 1e3, 4)
         autograd["graph_replay_value"] = round(B * T / autograd["graph_replay_ms_per_step"] / 1e3, 1)
+    line["autograd_api"] = autograd
 
     cpu = None
     parity = None
@@ -265,36 +287,83 @@ def main():
         cpu = cpu_baseline(w, backward)
         if not H:
             parity = parity_report(sets[0], fwd, bwd if backward else None)
-
-    line = {
-        "metric": "fwd+bwd Mtokens/s + % HBM roofline, B*H=96 T=1024 d=kdim=64 fp16" if args.workload == "cfg3"
-                  else "Mtokens/s (%s)" % args.workload,
-        "value": round(mtok, 1), "unit": "Mtokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": round(ms_per_step, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": {"float16": "fp16", "bfloat16": "bf16"}[w["dtype"]] + (
-            " I/O, fp32 state" if args.force_scan else " I/O, bf16 MFMA operands, fp32 accumulate"),
-        "data": "synthetic",
-        "config": {"workload": "%s: B=%d T=%d D=%d K=%d %s %s, checkpoint interval %d" % (
-            args.workload, B, T, D, K, w["dtype"], "fwd+bwd" if backward else "fwd", C),
-            "input_sets_rotated": nsets, "path": "scan" if args.force_scan else "auto"},
-        "whole_step_algorithmic_GBs": round(whole, 1),
-        "whole_step_roofline_frac": round(whole / HBM_PEAK_GBS, 4),
-        "forward_avg_ms": round(fwd_avg, 5), "backward_avg_ms": round(bwd_avg, 5) if backward else None,
-        "autograd_api": autograd,
-        "roofline": roofline,
-        "cpu_baseline": cpu,
-        "parity": parity,
-    }
+    line["cpu_baseline"] = cpu
+    line["parity"] = parity
     if cpu:
         line["speedup_vs_cpu"] = round(mtok / cpu["value"], 1) if cpu["value"] else None
+    return line
+
+
+def brief(line):
+    """what `other_configs` keeps of a workload's line"""
+    r = line.get("roofline") or {}
+    out = {"value": line["value"], "unit": line["unit"], "ms_per_step": line["ms_per_step"], "steps": line["steps"],
+           "workload": line["config"]["workload"],
+           "whole_step_roofline_frac": line.get("whole_step_roofline_frac"),
+           "roofline": {k: r.get(k) for k in ("kernel", "frac", "achieved", "avg_launch_ms", "algorithmic_bytes")}}
+    for k in ("forward_avg_ms", "backward_avg_ms", "backward_blockwise_ms", "state_GBs"):
+        if line.get(k) is not None:
+            out[k] = line[k]
+    return out
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--workload", default="cfg3", choices=sorted(WORKLOADS) + ["dfw", "copy256", "copy64", "cfg3_refgates"])
+    ap.add_argument("--ckpt-interval", type=int, default=64)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-other-configs", action="store_true",
+                    help="headline workload only (default: cfg2, cfg4, cfg5 and the delta rule are run briefly afterwards)")
+    ap.add_argument("--force-scan", action="store_true", help="exact scan kernels only")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build measures one GPU only (the path shards over the batch with no "
+              "exchange); run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(1)
+    if args.workload == "cfg5":
+        line = bench_generation(args, args.steps, args.warmup)
+    elif args.workload in ("copy256", "copy64"):
+        line = bench_copy(args)
+    elif args.workload == "dfw":
+        line = bench_dfw(args, args.steps, args.warmup)
+    elif args.workload == "cfg3_refgates":
+        line = bench_lfw(args, "cfg3", args.steps, args.warmup, extras=False, gates="reference_test")
+    else:
+        line = bench_lfw(args, args.workload, args.steps, args.warmup, extras=True)
+        if args.workload == "cfg3" and not args.no_other_configs and not args.force_scan:
+            # the other configurations of the baseline, briefly, outside the headline's timed region
+            torch.cuda.empty_cache()
+            others = {}
+            for name, kw in (("cfg2", {}), ("cfg4", {"max_sets": 2}), ("cfg3_reference_test_gates", {"gates": "reference_test", "max_sets": 4})):
+                wl = "cfg3" if name.startswith("cfg3") else name
+                others[name] = brief(bench_lfw(args, wl, 20, 5, extras=False, **kw))
+                torch.cuda.empty_cache()
+            others["cfg5"] = brief(bench_generation(args, 50, 10))
+            torch.cuda.empty_cache()
+            others["dfw"] = brief(bench_dfw(args, 20, 5))
+            line["other_configs"] = others
     print(json.dumps(line))
 
 
 def parity_report(d, fwd, bwd, rows=3):
     """Part of the CPU leg: the GPU results of input set `d` (recomputed here, outside any timed
-    region) against the float64 oracle on the first `rows` batch rows (rows are independent)."""
+    region) against the float64 oracle on the first `rows` batch rows (rows are independent).
+    Next to each tensor's error stands the error of the reference's own arithmetic on the same
+    inputs: the recurrence of t2fw/torch.py:21-29 evaluated in the tensors' dtype on the CPU, with
+    gradients by autograd, which is what the reference's test compares its kernels against
+    (tests/test_lfw.py:30,48-53) and about what its kernels do (state and products in the tensor
+    dtype, t2fw/csrc/lfw_kernel.cu:38,46-50)."""
     import torch
-    from oracle import c_oracle
+    from oracle import c_oracle, lfw_ref
     from t2fw_amd.synthetic import err_stats
     fwd(d)
     if bwd is not None:
@@ -302,15 +371,37 @@ def parity_report(d, fwd, bwd, rows=3):
     torch.cuda.synchronize()
     ins = [t[:rows].cpu() for t in d["ins"]]
     r_out, r_nxt = c_oracle.lfw_forward(*ins)
-    pairs = [("outputs", d["out"][:rows], r_out), ("next_state", d["nxt"][:rows], r_nxt)]
+    names = ["outputs", "next_state"]
+    got = [d["out"][:rows], d["nxt"][:rows]]
+    ref = [r_out, r_nxt]
+    own = None
     if bwd is not None:
-        r_grads = c_oracle.lfw_backward(d["go"][:rows].cpu(), d["gs"][:rows].cpu(), *ins)
-        pairs += [(n, g[:rows], r) for n, g, r in zip(("d_x", "d_f", "d_q", "d_k", "d_f_key", "d_state"), d["grads"], r_grads)]
-    rep = {"reference": "float64 oracle (oracle/lfw_oracle.c) on the same quantised inputs", "rows": rows, "tensors": {}}
-    for name, got, ref in pairs:
-        mx, rel, mean_rel = err_stats(got, torch.as_tensor(ref))
+        go, gs = d["go"][:rows].cpu(), d["gs"][:rows].cpu()
+        names += ["d_x", "d_f", "d_q", "d_k", "d_f_key", "d_state"]
+        got += [g[:rows] for g in d["grads"]]
+        ref += list(c_oracle.lfw_backward(go, gs, *ins))
+        try:
+            o, n, g = lfw_ref.lfw_reference_grads(*ins, go, gs, dtype=ins[0].dtype)
+            own = [o, n] + list(g)
+        except Exception:                 # an op this torch build lacks for the dtype on the CPU
+            own = None
+    else:
+        try:
+            with torch.no_grad():
+                own = list(lfw_ref.lfw_reference(*ins))
+        except Exception:
+            own = None
+    rep = {"reference": "float64 oracle (oracle/lfw_oracle.c) on the same quantised inputs", "rows": rows,
+           "reference_arithmetic": "the recurrence of the reference evaluated in %s on the CPU (oracle/lfw_ref.py), "
+                                   "same inputs, against the same float64 oracle" % str(ins[0].dtype).replace("torch.", ""),
+           "tensors": {}}
+    for i, name in enumerate(names):
+        mx, rel, mean_rel = err_stats(got[i], torch.as_tensor(ref[i]))
         rep["tensors"][name] = {"max_abs": float("%.3e" % mx), "max_abs_over_max_ref": float("%.3e" % rel),
                                 "mean_rel": float("%.3e" % mean_rel)}
+        if own is not None:
+            omx, orel, _ = err_stats(own[i], torch.as_tensor(ref[i]))
+            rep["tensors"][name]["reference_arithmetic_max_abs_over_max_ref"] = float("%.3e" % orel)
     return rep
 
 
@@ -330,14 +421,14 @@ def bench_copy(args):
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
     gbs = 2 * n * args.steps / wall / 1e9
-    print(json.dumps({"metric": "device copy GB/s (read + write), %d MiB" % mib, "value": round(gbs, 1), "unit": "GB/s",
-                      "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-                      "ms_per_step": round(wall / args.steps * 1e3, 5), "higher_is_better": True, "scaling": "weak",
-                      "vs_baseline": None, "dtype": "u8", "data": "synthetic",
-                      "config": {"workload": "%s: torch copy_ of %d bytes, device to device" % (args.workload, n)}}))
+    return {"metric": "device copy GB/s (read + write), %d MiB" % mib, "value": round(gbs, 1), "unit": "GB/s",
+            "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+            "ms_per_step": round(wall / args.steps * 1e3, 5), "higher_is_better": True, "scaling": "weak",
+            "vs_baseline": None, "dtype": "u8", "data": "synthetic",
+            "config": {"workload": "%s: torch copy_ of %d bytes, device to device" % (args.workload, n)}}
 
 
-def bench_dfw(args):
+def bench_dfw(args, steps, warmup):
     """Delta rule (t2fw/functional_dfw.py:29-65) forward + backward through the C ABI: B=96, T=1024,
     D=M=64, fp32, keys built as the reference's test builds them (tests/test_dfw.py:45-46).  A step
     is one forward and one backward call; the backward call is two launches (value side, then
@@ -378,15 +469,15 @@ def bench_dfw(args):
         _lib.check(lib.t2fw_dfw_backward(P(d["go"]), P(d["gs"]), P(d["q"]), P(d["k"]), P(d["delta"]), P(d["fin"]),
                                          P(d["d_q"]), P(d["d_k"]), P(d["d_v"]), P(d["d_s0"]), B, T, D, M, code, stream))
 
-    for i in range(args.warmup):
+    for i in range(warmup):
         fwd(sets[i % nsets]); bwd(sets[i % nsets])
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    for i in range(args.steps):
+    for i in range(steps):
         fwd(sets[i % nsets]); bwd(sets[i % nsets])
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
-    nrep = min(args.steps, 100)
+    nrep = min(steps, 100)
     ev = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(nrep)]
     for i in range(nrep):
         d = sets[i % nsets]
@@ -397,11 +488,11 @@ def bench_dfw(args):
     tok = B * T
     fwd_bytes = (tok * (2 * M + 3 * D) + 2 * B * D * M) * es
     bwd_bytes = (tok * (2 * D + 2 * M + 2 * M + D) + 3 * B * D * M) * es
-    ms_per_step = wall / args.steps * 1e3
+    ms_per_step = wall / steps * 1e3
     achieved = bwd_bytes / (bwd_ms * 1e-3) / 1e9
     line = {
-        "metric": "delta rule fwd+bwd Mtokens/s, B=96 T=1024 D=M=64 fp32", "value": round(tok * args.steps / wall / 1e6, 1),
-        "unit": "Mtokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "metric": "delta rule fwd+bwd Mtokens/s, B=96 T=1024 D=M=64 fp32", "value": round(tok * steps / wall / 1e6, 1),
+        "unit": "Mtokens/s", "n_gpus": 1, "steps": steps, "warmup": warmup,
         "ms_per_step": round(ms_per_step, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f32", "data": "synthetic",
         "config": {"workload": "dfw: B=%d T=%d D=%d M=%d float32 fwd+bwd" % (B, T, D, M), "input_sets_rotated": nsets},
@@ -412,10 +503,10 @@ def bench_dfw(args):
                      "algorithmic_bytes": bwd_bytes, "avg_launch_ms": round(bwd_ms, 5)},
         "cpu_baseline": None,
     }
-    print(json.dumps(line))
+    return line
 
 
-def bench_generation(args):
+def bench_generation(args, steps, warmup):
     """cfg5: O(1) generation steps at serving batch, the state carried in place.  A "step" is
     one call of t2fw_lfw_step over the whole batch; bytes = state read + write + six vectors."""
     import torch
@@ -439,16 +530,16 @@ def bench_generation(args):
         v = vec[i % nvec]
         _lib.check(lib.t2fw_lfw_step(*[_lib.ptr(t) for t in v], _lib.ptr(state), _lib.ptr(out), _lib.ptr(state),
                                      B, D, K, code, stream))
-    for i in range(args.warmup):
+    for i in range(warmup):
         step(i)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    for i in range(args.steps):
+    for i in range(steps):
         step(i)
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
     ev = [torch.cuda.Event(enable_timing=True) for _ in range(2)]
-    nrep = min(args.steps, 100)
+    nrep = min(steps, 100)
     ev[0].record()
     for i in range(nrep):
         step(i)
@@ -459,9 +550,9 @@ def bench_generation(args):
     nbytes = B * (2 * D * K * es + (3 * D + 3 * K) * es)
     achieved = nbytes / (kern_ms * 1e-3) / 1e9
     line = {
-        "metric": "generation steps: Mtokens/s and state GB/s (cfg5)", "value": round(B * args.steps / wall / 1e6, 1),
-        "unit": "Mtokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": round(wall / args.steps * 1e3, 5), "higher_is_better": True, "scaling": "weak",
+        "metric": "generation steps: Mtokens/s and state GB/s (cfg5)", "value": round(B * steps / wall / 1e6, 1),
+        "unit": "Mtokens/s", "n_gpus": 1, "steps": steps, "warmup": warmup,
+        "ms_per_step": round(wall / steps * 1e3, 5), "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "fp16 I/O, fp32 arithmetic", "data": "synthetic",
         "config": {"workload": "cfg5: B=%d T=1 D=%d K=%d float16, state carried in place over consecutive calls" % (B, D, K)},
         "state_GBs": round(2 * B * D * K * es / (kern_ms * 1e-3) / 1e9, 1),
@@ -470,7 +561,7 @@ def bench_generation(args):
                      "algorithmic_bytes": nbytes, "avg_launch_ms": round(kern_ms, 5)},
         "cpu_baseline": None,
     }
-    print(json.dumps(line))
+    return line
 
 
 def cpu_baseline(w, backward):

@@ -150,8 +150,12 @@ int t2fw_lfw_forward(const void *x, const void *f, const void *q, const void *k,
  * (t2fw_lfw_workspace_bytes) exceeds the buffer is rejected with T2FW_ERR_WORKSPACE.  All calls
  * on one GPU share the buffer: calls that overlap in time on one GPU (different streams or
  * threads) race on it; calls on one stream do not.
+ * The first call on a GPU looks up the buffer's address, which may load the library's code onto that
+ * GPU: make that call, or t2fw_static_init() with the GPU current, before a stream capture begins.
  */
 #define T2FW_STATIC_SCRATCH_BYTES (1 << 20)
+/* Looks up the built-in buffer of the current GPU (once per GPU; later calls return at once). */
+int t2fw_static_init(void);
 int t2fw_lfw_forward_static(const void *x, const void *f, const void *q, const void *k,
                             const void *f_key, const void *s0,
                             void *out, void *next_state, void *ckpt,

@@ -35,6 +35,7 @@ SIGNATURES = {
     "t2fw_lfw_flag_regions": (ctypes.c_int, [_i64] * 4 + [_i32] * 3 + [ctypes.POINTER(ctypes.c_int64)]),
     "t2fw_host_workspace_device_pointer": (ctypes.c_int, [_vp, ctypes.POINTER(ctypes.c_void_p)]),
     "t2fw_lfw_forward": (ctypes.c_int, [_vp] * 9 + [_i64] * 4 + [_i32] * 3 + [_vp, _sz, _vp]),
+    "t2fw_static_init": (ctypes.c_int, []),
     "t2fw_lfw_forward_static": (ctypes.c_int, [_vp] * 9 + [_i64] * 4 + [_i32] * 3 + [_vp]),
     "t2fw_lfw_backward": (ctypes.c_int, [_vp] * 15 + [_i64] * 4 + [_i32] * 3 + [_vp, _sz, _vp]),
     "t2fw_lfw_forward_heads": (ctypes.c_int, [_vp] * 9 + [_i64] * 5 + [_i32] * 3 + [_vp, _sz, _vp]),

@@ -307,6 +307,11 @@ int t2fw_lfw_forward(const void *x, const void *f, const void *q, const void *k,
                             workspace_bytes, stream);
 }
 
+int t2fw_static_init(void) {
+    void *ws = nullptr;
+    return static_scratch(&ws);
+}
+
 int t2fw_lfw_forward_static(const void *x, const void *f, const void *q, const void *k, const void *f_key,
                             const void *s0, void *out, void *next_state, void *ckpt, int64_t B, int64_t T,
                             int64_t D, int64_t K, int32_t C, int32_t dtype, int32_t flags, void *stream) {

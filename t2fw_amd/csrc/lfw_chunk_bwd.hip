@@ -818,6 +818,11 @@ template <typename IOE, typename OPE, int NB, bool HEADS> int launch(const Chunk
         if (g.kg != 16 || g.kpl != 4) return fail(T2FW_ERR_UNSUPPORTED, "unexpected scan geometry for a 64 x 64 state");
         a2.scan_kg = g.kg;
         a2.scan_ntiles = (CH_N + g.rows - 1) / g.rows;
+        // the body runs in this kernel's LDS, below the verdict word
+        const size_t need = scan_bwd_lds_bytes(scan::SegLen<4>::value, g.kg, g.kpl, g.rows, a.C, true);
+        if (need > (size_t)OFF_VERDICT)
+            return fail(T2FW_ERR_UNSUPPORTED, "the exact scan body needs %zu bytes of LDS, the block-wise backward kernel has %d",
+                        need, OFF_VERDICT);
     }
     hipLaunchKernelGGL(kern, dim3(2u * (unsigned)rows_padded), dim3(BW_THREADS), BW_SMEM, stream, a2, rows_padded);
     return check_hip(hipGetLastError(), "lfw_bwd_chunk_kernel launch");

@@ -586,6 +586,11 @@ int chunk_forward(const ChunkFwdArgs &args, int dtype, int op, bool split, hipSt
         a.scan_ntiles = CH_N / g.rows;
         if (g.kpl != 4 || g.kg != 16 || a.scan_ntiles % 2 != 0)
             return fail(T2FW_ERR_UNSUPPORTED, "unexpected scan geometry for a 64 x 64 state");
+        // the body runs in this kernel's LDS, below the verdict word
+        const size_t need = scan_fwd_lds_bytes(tb, g.kg, g.kpl, g.rows);
+        if (need > (size_t)OFF_VERDICT)
+            return fail(T2FW_ERR_UNSUPPORTED, "the exact scan body needs %zu bytes of LDS, the forward kernel has %d", need,
+                        OFF_VERDICT);
     }
     if (a.heads == 1) {
         if (dtype == T2FW_F16)

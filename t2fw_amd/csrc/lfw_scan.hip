@@ -42,7 +42,7 @@ __global__ __launch_bounds__(SCAN_THREADS) void lfw_bwd_scan_kernel(ScanBwdArgs 
 template <typename IO, int KPL>
 int launch_fwd(const ScanFwdArgs &a, const ScanGeom &g, hipStream_t stream) {
     using Acc = typename AccOf<IO>::type;
-    const size_t smem = ((size_t)a.tb * 3 * g.kg * g.kpl + (size_t)a.tb * 3 * g.rows) * sizeof(Acc);
+    const size_t smem = scan_fwd_lds_bytes(a.tb, g.kg, g.kpl, g.rows) * sizeof(Acc) / 4;
     ScanFwdArgs a2 = a;
     a2.ntiles = (int)((a.D + g.rows - 1) / g.rows);
     const int64_t nblocks = a.B * a2.ntiles;
@@ -57,11 +57,10 @@ int launch_bwd(ScanBwdArgs a, const ScanGeom &g, hipStream_t stream) {
     using Acc = typename AccOf<IO>::type;
     constexpr int SEG = SegLen<KPL>::value;
     const int64_t nrows = SIDE == 0 ? a.D : a.K;
-    const size_t base = ((size_t)SEG * 3 * g.kg * g.kpl + (size_t)SEG * 6 * g.rows) * sizeof(Acc);
-    const size_t nseg = (size_t)(a.C + SEG - 1) / SEG;
-    const size_t sub = nseg * KPL * SCAN_THREADS * sizeof(Acc);
-    a.use_sub = (base + sub <= 64 * 1024) ? 1 : 0;
-    const size_t smem = base + (a.use_sub ? sub : 0);
+    const size_t base = scan_bwd_lds_bytes(SEG, g.kg, g.kpl, g.rows, a.C, false) * sizeof(Acc) / 4;
+    const size_t with_sub = scan_bwd_lds_bytes(SEG, g.kg, g.kpl, g.rows, a.C, true) * sizeof(Acc) / 4;
+    a.use_sub = (with_sub <= 64 * 1024) ? 1 : 0;
+    const size_t smem = a.use_sub ? with_sub : base;
     a.kg = g.kg;
     a.ntiles = (int)((nrows + g.rows - 1) / g.rows);
     const int64_t nblocks = a.B * a.ntiles;

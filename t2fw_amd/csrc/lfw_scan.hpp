@@ -30,6 +30,19 @@ struct ScanBwdArgs {
     int32_t accumulate;
 };
 
+// Dynamic LDS, in bytes, that the scan bodies use for a 32-bit accumulator (lfw_scan_body.hpp): the kernels
+// that run a scan body inside another kernel's allocation check their own size against these.
+//   forward: tb staged steps of the column inputs (kg * kpl columns) and the row inputs (rows per workgroup)
+inline size_t scan_fwd_lds_bytes(int tb, int kg, int kpl, int rows) {
+    return ((size_t)tb * 3 * kg * kpl + (size_t)tb * 3 * rows) * 4;
+}
+//   backward: seg staged steps of column inputs, row inputs and row outputs, plus (use_sub) the segment-start
+//   states of one chunk, kpl values per thread of the 256
+inline size_t scan_bwd_lds_bytes(int seg, int kg, int kpl, int rows, int C, bool use_sub) {
+    const size_t base = ((size_t)seg * 3 * kg * kpl + (size_t)seg * 6 * rows) * 4;
+    return base + (use_sub ? (size_t)((C + seg - 1) / seg) * kpl * 256 * 4 : 0);
+}
+
 int scan_forward(const ScanFwdArgs &a, int dtype, hipStream_t stream);
 int scan_backward(const ScanBwdArgs &a, int dtype, hipStream_t stream);
 

@@ -57,31 +57,40 @@ def count_hinted_rows(hints, rows):
     return int(np.count_nonzero(h[0] | h[1]))
 
 
+class _Slot:
+    """One pinned workspace: the tensor that owns it, the address the GPU sees it under, a view of its
+    hint region and the event recorded after the last launch that writes it."""
+    __slots__ = ("buf", "dptr", "view", "event")
+
+
 class _PinnedPool:
-    """Pinned host buffers of one size, handed out for one forward call each and taken back when the
-    GPU work that writes them has completed.  Grows to the number of calls in flight."""
+    """Pinned host workspaces, handed out for one forward call each and taken back once the GPU work that
+    writes them has completed.  Grows to the number of forward calls in flight."""
 
     def __init__(self):
         self.lock = threading.Lock()
-        self.free = {}          # (device index, nbytes) -> list of (tensor, device pointer, event that must have completed)
+        self.free = {}          # (device index, nbytes, hint offset, hint count) -> list of _Slot
 
-    def acquire(self, device, nbytes):
-        key = (device.index if device.index is not None else torch.cuda.current_device(), nbytes)
+    def acquire(self, key):
         with self.lock:
-            lst = self.free.get(key, [])
-            for i, (t, dptr, ev) in enumerate(lst):
-                if ev is None or ev.query():
-                    del lst[i]
-                    return t, dptr
-        t = torch.empty(nbytes, dtype=torch.uint8, pin_memory=True)
-        dptr = ctypes.c_void_p()
-        _lib.check(_lib.load().t2fw_host_workspace_device_pointer(ctypes.c_void_p(t.data_ptr()), ctypes.byref(dptr)))
-        return t, dptr
+            lst = self.free.get(key)
+            if lst:
+                for i in range(len(lst)):
+                    if lst[i].event.query():
+                        return lst.pop(i)
+        _, nbytes, hint_offset, hint_count = key
+        slot = _Slot()
+        slot.buf = torch.empty(nbytes, dtype=torch.uint8, pin_memory=True)
+        slot.dptr = ctypes.c_void_p()
+        _lib.check(_lib.load().t2fw_host_workspace_device_pointer(ctypes.c_void_p(slot.buf.data_ptr()),
+                                                                  ctypes.byref(slot.dptr)))
+        slot.view = slot.buf.numpy()[hint_offset:hint_offset + 4 * hint_count].view(np.int32)
+        slot.event = torch.cuda.Event()
+        return slot
 
-    def release(self, device, t, dptr, ev):
-        key = (device.index if device.index is not None else torch.cuda.current_device(), t.numel())
+    def release(self, key, slot):
         with self.lock:
-            self.free.setdefault(key, []).append((t, dptr, ev))
+            self.free.setdefault(key, []).append(slot)
 
 
 _POOL = _PinnedPool()
@@ -93,10 +102,11 @@ class ForwardHints:
     def __init__(self, device, nbytes, hint_offset, hint_count, rows):
         self.device = device
         self.rows = rows
-        self.buf, self.dptr = _POOL.acquire(device, nbytes)
         self.nbytes = nbytes
-        self.view = self.buf.numpy()[hint_offset:hint_offset + 4 * hint_count].view(np.int32)
-        self.event = None
+        self.key = (device.index if device.index is not None else torch.cuda.current_device(), nbytes, hint_offset,
+                    hint_count)
+        self.slot = _POOL.acquire(self.key)
+        self.launched_ = False
         self.count = None
 
     @staticmethod
@@ -105,26 +115,28 @@ class ForwardHints:
         return not torch.cuda.is_current_stream_capturing()
 
     def workspace(self):
-        return self.dptr, self.nbytes
+        return self.slot.dptr, self.nbytes
 
     def launched(self):
         """Call right after the forward launch, on the launch stream."""
-        self.event = torch.cuda.Event()
-        self.event.record(torch.cuda.current_stream(self.device))
+        self.slot.event.record(torch.cuda.current_stream(self.device))
+        self.launched_ = True
 
     def hinted_rows(self):
         """Rows hinted, or None while the forward call has not completed on the GPU.  The first answer is
         kept (a backward may be asked for twice) and the buffer goes back to the pool."""
-        if self.count is None and self.buf is not None and self.event is not None and self.event.query():
-            self.count = count_hinted_rows(self.view, self.rows)
+        slot = self.slot
+        if self.count is None and slot is not None and self.launched_ and slot.event.query():
+            self.count = count_hinted_rows(slot.view, self.rows) if slot.view.any() else 0
             self.close()
         return self.count
 
     def close(self):
-        if self.buf is not None:
-            self.view = None
-            _POOL.release(self.device, self.buf, self.dptr, self.event)
-            self.buf = None
+        slot, self.slot = self.slot, None
+        if slot is not None:
+            if not self.launched_:
+                slot.event.record(torch.cuda.current_stream(self.device))     # nothing pending: reusable at once
+            _POOL.release(self.key, slot)
 
     def __del__(self):
         try:

@@ -89,3 +89,40 @@ def test_static_forward_rejects_what_the_buffer_cannot_hold():
     rc = lib.t2fw_lfw_forward_static(p, p, p, p, p, p, p, p, None, B, 1, 64, 64, 64, code, 0, None)
     assert rc == 6                 # T2FW_ERR_WORKSPACE, before anything is launched
     assert b"built-in buffer" in lib.t2fw_last_error()
+
+
+def test_static_forward_under_graph_capture_allocates_nothing():
+    """after t2fw_static_init the call can be recorded into a HIP graph; replays on new inputs equal the
+    workspace call, and the device's free memory does not move across capture and replays"""
+    from t2fw_amd import _lib
+    lib = _lib.load()
+    _lib.check(lib.t2fw_static_init())
+    B, T, C = 6, 200, 64
+    code = _lib.DTYPE_CODE[torch.float16]
+    mk = lambda seed: [t.cuda() for t in make_config_inputs(B, T, 64, 64, torch.float16, seed=seed, state_std=0.2)[:6]]
+    static_ins = mk(11)
+    out, nxt = torch.empty_like(static_ins[0]), torch.empty_like(static_ins[5])
+    ckpt = torch.empty(B, lib.t2fw_lfw_num_ckpt(T, C), 64, 64, dtype=torch.float16, device="cuda")
+    ptrs = [_lib.ptr(t) for t in static_ins] + [_lib.ptr(out), _lib.ptr(nxt), _lib.ptr(ckpt)]
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):          # one eager call on the capture stream first
+        _lib.check(lib.t2fw_lfw_forward_static(*ptrs, B, T, 64, 64, C, code, 0, _lib.current_stream_handle(out.device)))
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    free_before = torch.cuda.mem_get_info()[0]
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        _lib.check(lib.t2fw_lfw_forward_static(*ptrs, B, T, 64, 64, C, code, 0, _lib.current_stream_handle(out.device)))
+    graph.replay()
+    torch.cuda.synchronize()
+    # nothing but the graph object itself may have taken device memory (no torch allocation happened in between)
+    assert torch.cuda.mem_get_info()[0] >= free_before - (8 << 20), "capture or replay allocated device memory"
+    for seed in (12, 13, 14):
+        fresh = mk(seed)
+        want = _forward(lib, _lib, fresh, C, static=False)      # eager work between the replays
+        for dst, src in zip(static_ins, fresh):
+            dst.copy_(src)
+        graph.replay()
+        torch.cuda.synchronize()
+        _same((out, nxt, ckpt), want)
