@@ -442,6 +442,7 @@ def bench_dfw(args, steps, warmup):
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     code = _lib.DTYPE_CODE[dtype]
+    flags = _lib.FLAG_FORCE_SCAN if args.force_scan else _lib.FLAG_AUTO
     stream = _lib.current_stream_handle(dev)
     per_set = (B * T * (3 * D + 2 * M) + B * T * (2 * D + 2 * M)) * es
     nsets = max(2, min(16, int(1.2e9 // per_set) + 1))
@@ -463,11 +464,11 @@ def bench_dfw(args, steps, warmup):
 
     def fwd(d):
         _lib.check(lib.t2fw_dfw_forward(P(d["q"]), P(d["k"]), P(d["v"]), P(d["s0"]), P(d["out"]), P(d["fin"]),
-                                        P(d["delta"]), B, T, D, M, code, stream))
+                                        P(d["delta"]), B, T, D, M, code, flags, stream))
 
     def bwd(d):
         _lib.check(lib.t2fw_dfw_backward(P(d["go"]), P(d["gs"]), P(d["q"]), P(d["k"]), P(d["delta"]), P(d["fin"]),
-                                         P(d["d_q"]), P(d["d_k"]), P(d["d_v"]), P(d["d_s0"]), B, T, D, M, code, stream))
+                                         P(d["d_q"]), P(d["d_k"]), P(d["d_v"]), P(d["d_s0"]), B, T, D, M, code, flags, stream))
 
     for i in range(warmup):
         fwd(sets[i % nsets]); bwd(sets[i % nsets])

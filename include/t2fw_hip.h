@@ -221,14 +221,14 @@ int t2fw_lfw_step(const void *x, const void *f, const void *q, const void *k,
 int t2fw_dfw_forward(const void *q, const void *k, const void *v, const void *s0,
                      void *out, void *final_state, void *delta,
                      int64_t B, int64_t T, int64_t D, int64_t M,
-                     int32_t dtype, void *stream);
+                     int32_t dtype, int32_t flags, void *stream);
 
 int t2fw_dfw_backward(const void *g_out, const void *g_state,
                       const void *q, const void *k, const void *delta,
                       const void *final_state,
                       void *d_q, void *d_k, void *d_v, void *d_s0,
                       int64_t B, int64_t T, int64_t D, int64_t M,
-                      int32_t dtype, void *stream);
+                      int32_t dtype, int32_t flags, void *stream);
 
 /*
  * Sigmoid gating of both forget gates in one launch: f = sigmoid(f_logit) [n_f elements],

@@ -43,8 +43,8 @@ SIGNATURES = {
     "t2fw_lfw_step": (ctypes.c_int, [_vp] * 8 + [_i64] * 3 + [_i32, _vp]),
     "t2fw_gate_forward": (ctypes.c_int, [_vp] * 4 + [_i64] * 2 + [_i32, _vp]),
     "t2fw_gate_backward": (ctypes.c_int, [_vp] * 6 + [_i64] * 2 + [_i32, _vp]),
-    "t2fw_dfw_forward": (ctypes.c_int, [_vp] * 7 + [_i64] * 4 + [_i32, _vp]),
-    "t2fw_dfw_backward": (ctypes.c_int, [_vp] * 10 + [_i64] * 4 + [_i32, _vp]),
+    "t2fw_dfw_forward": (ctypes.c_int, [_vp] * 7 + [_i64] * 4 + [_i32, _i32, _vp]),
+    "t2fw_dfw_backward": (ctypes.c_int, [_vp] * 10 + [_i64] * 4 + [_i32, _i32, _vp]),
 }
 
 _lib = None

@@ -461,8 +461,14 @@ int t2fw_lfw_step(const void *x, const void *f, const void *q, const void *k, co
                             T2FW_FLAG_FORCE_SCAN, nullptr, 0, stream);
 }
 
+// The block-wise matrix-core kernels of the delta rule cover D = M = 64 with fp32 tensors.
+static bool dfw_chunk_ok(int64_t D, int64_t M, int32_t dtype, int32_t flags) {
+    return (flags & T2FW_FLAG_FORCE_SCAN) == 0 && D == 64 && M == 64 && dtype == T2FW_F32;
+}
+
 int t2fw_dfw_forward(const void *q, const void *k, const void *v, const void *s0, void *out, void *final_state,
-                     void *delta, int64_t B, int64_t T, int64_t D, int64_t M, int32_t dtype, void *stream) {
+                     void *delta, int64_t B, int64_t T, int64_t D, int64_t M, int32_t dtype, int32_t flags,
+                     void *stream) {
     const size_t es = elem_size(dtype);
     if (es == 0) return fail(T2FW_ERR_BAD_DTYPE, "unknown dtype code %d", dtype);
     int rc = check_dims(B, T, D, M);
@@ -484,12 +490,14 @@ int t2fw_dfw_forward(const void *q, const void *k, const void *v, const void *s0
     DfwFwdArgs a{};
     a.q = q; a.k = k; a.v = v; a.s0 = s0; a.out = out; a.final_state = final_state; a.delta = delta;
     a.B = B; a.T = T; a.D = D; a.M = M;
+    if (dfw_chunk_ok(D, M, dtype, flags) && T * CH_N < 0x7fffffffLL && aligned16({q, k, v, s0, out, final_state, delta}))
+        return dfw_chunk_forward(a, st);
     return dfw_forward(a, dtype, st);
 }
 
 int t2fw_dfw_backward(const void *g_out, const void *g_state, const void *q, const void *k, const void *delta,
                       const void *final_state, void *d_q, void *d_k, void *d_v, void *d_s0, int64_t B, int64_t T,
-                      int64_t D, int64_t M, int32_t dtype, void *stream) {
+                      int64_t D, int64_t M, int32_t dtype, int32_t flags, void *stream) {
     const size_t es = elem_size(dtype);
     if (es == 0) return fail(T2FW_ERR_BAD_DTYPE, "unknown dtype code %d", dtype);
     int rc = check_dims(B, T, D, M);

@@ -1,0 +1,214 @@
+// Block-wise matrix-core form of the delta rule for D = M = 64, fp32 tensors (dfw_chunk_fwd.hip,
+// dfw_chunk_bwd.hip): shared layout constants and device helpers.
+//
+// Inside a block of L = 16 steps that starts from the state S0 (all matrices with one row per step):
+//   A  = strictly lower triangle of K K^T        Bq = strictly lower triangle of Q K^T
+//   Delta = Tm (V - K S0^T),  Tm = (I + A)^-1    (the block's delta_t = v_t - S_{t-1} k_t)
+//   O  = Q S0^T + Bq Delta                       S_L = S0 + Delta^T K
+// A is nilpotent (A^16 = 0), so Tm = (I - A)(I + A^2)(I + A^4)(I + A^8): three squarings and a few more
+// 16 x 16 products on the matrix cores instead of a 16-step substitution.  Tm and the transformed keys
+// K' = Tm K do not depend on the state, so they are prepared ahead of the sequential pass, whose chain per
+// block is then only  S0 -> Delta = Tm V - K' S0^T -> S_L.  The backward pass uses Tm transposed the same way.
+//
+// Precision: the tensors are fp32 and the matrix cores take bf16, so every operand is split into a bf16
+// head and a bf16 remainder (x = hi + lo up to 2^-17 of x) and a product runs as three MFMAs
+// (hi*hi + hi*lo + lo*hi) with fp32 accumulation: results carry fp32-level rounding (measured against the
+// fp64 oracle: 1e-5 of max|ref|), not the 2^-9 of a single bf16 operand.
+#pragma once
+
+#include "lfw_chunk.hpp"
+#include "lfw_chunk_bwd_dev.hpp"
+
+namespace t2fw {
+
+#if defined(__HIPCC__)
+namespace dfwc {
+
+using namespace bwd;
+
+constexpr int DL = 16;                        // block length
+constexpr int DNB = 2;                        // blocks per stage (one workgroup barrier per stage)
+constexpr int DTS = 72;                       // row stride (elements) of token-major tiles [16 tokens][64 channels]
+constexpr int DCS = 20;                       // row stride of channel-major tiles [64 channels][16 tokens]
+constexpr int TM_TILE = DL * DTS * 2;         // bytes of one token-major tile (one of hi / lo)
+constexpr int CM_TILE = CH_N * DCS * 2;       // bytes of one channel-major tile
+constexpr int ST_TILE = 64 * 8;               // a 16 x 16 matrix as a packed MFMA operand: 8 bytes per lane
+
+// an operand of a 16-deep (Sp2) or 32-deep (Sp4) contraction as bf16 head and remainder
+struct Sp2 {
+    uint2 hi, lo;
+};
+struct Sp4 {
+    uint4 hi, lo;
+};
+
+__device__ __forceinline__ Sp2 split4(float a, float b, float c, float d) {
+    Sp2 o;
+    o.hi = packq<Bf16>(a, b, c, d);
+    o.lo = packq<Bf16>(a - Bf16::to_f32((u16)(o.hi.x & 0xffffu)), b - Bf16::to_f32((u16)(o.hi.x >> 16)),
+                       c - Bf16::to_f32((u16)(o.hi.y & 0xffffu)), d - Bf16::to_f32((u16)(o.hi.y >> 16)));
+    return o;
+}
+__device__ __forceinline__ Sp2 split4(const floatx4 &v) { return split4(v[0], v[1], v[2], v[3]); }
+__device__ __forceinline__ Sp4 cat(const Sp2 &a, const Sp2 &b) {
+    Sp4 o;
+    o.hi = bwd::cat(a.hi, b.hi);
+    o.lo = bwd::cat(a.lo, b.lo);
+    return o;
+}
+
+// c + a b with split operands (the smaller terms first); chains of one MFMA form only
+__device__ __forceinline__ floatx4 mma16(const Sp2 &a, const Sp2 &b, floatx4 c) {
+    c = Bf16::mfma16(a.lo, b.hi, c);
+    c = Bf16::mfma16(a.hi, b.lo, c);
+    return Bf16::mfma16(a.hi, b.hi, c);
+}
+__device__ __forceinline__ floatx4 mma32(const Sp4 &a, const Sp4 &b, floatx4 c) {
+    c = Bf16::mfma32(a.lo, b.hi, c);
+    c = Bf16::mfma32(a.hi, b.lo, c);
+    return Bf16::mfma32(a.hi, b.hi, c);
+}
+
+// ---- tiles in LDS: a head tile followed by a remainder tile of the same shape ----------------------
+// token-major [16][DTS]: channel c of a token sits at tm_pos(c), so that the sixteen channels a matrix lane
+// (r, g) pairs with its accumulators (16 j + 4 g + e) are contiguous at 16 g
+struct TmTile {
+    const u16 *hi, *lo;
+    __device__ __forceinline__ TmTile(const unsigned char *base) : hi(reinterpret_cast<const u16 *>(base)), lo(reinterpret_cast<const u16 *>(base + TM_TILE)) {}
+    // A / B operand "row `row`, the lane's accumulator channels", halves h = 0, 1 of the 64-deep contraction
+    __device__ __forceinline__ Sp4 acc_order(int row, int g, int h) const {
+        Sp4 o;
+        o.hi = ld4(hi + row * DTS + 16 * g + 8 * h);
+        o.lo = ld4(lo + row * DTS + 16 * g + 8 * h);
+        return o;
+    }
+    // A / B operand "row `row`" for products of two token-major tiles (any fixed channel order)
+    __device__ __forceinline__ Sp4 any_order(int row, int g, int h) const {
+        Sp4 o;
+        o.hi = ld4(hi + row * DTS + 8 * g + 32 * h);
+        o.lo = ld4(lo + row * DTS + 8 * g + 32 * h);
+        return o;
+    }
+};
+// channel-major [64][DCS]: A operand "channel `ch`, tokens 4 g .. 4 g + 3"
+struct CmTile {
+    const u16 *hi, *lo;
+    __device__ __forceinline__ CmTile(const unsigned char *base) : hi(reinterpret_cast<const u16 *>(base)), lo(reinterpret_cast<const u16 *>(base + CM_TILE)) {}
+    __device__ __forceinline__ Sp2 tokens(int ch, int g) const {
+        Sp2 o;
+        o.hi = ld2(hi + ch * DCS + 4 * g);
+        o.lo = ld2(lo + ch * DCS + 4 * g);
+        return o;
+    }
+};
+// Four result tiles [channel 16 j + 4 g + e][token r] (j = 0 .. 3) of a lane are the sixteen channels that
+// tm_pos puts at 16 g of token row r: stored as head and remainder of a token-major tile
+__device__ __forceinline__ void store_tm_from_acc(unsigned char *tile, int r, int g, const floatx4 (&v)[4]) {
+    u16 *hi = reinterpret_cast<u16 *>(tile), *lo = reinterpret_cast<u16 *>(tile + TM_TILE);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const Sp2 s = split4(v[j]);
+        *reinterpret_cast<uint2 *>(hi + r * DTS + 16 * g + 4 * j) = s.hi;
+        *reinterpret_cast<uint2 *>(lo + r * DTS + 16 * g + 4 * j) = s.lo;
+    }
+}
+
+// a 16 x 16 matrix in the accumulator layout (lane (r, g): rows 4 g + e of column r), packed: read back by
+// the same lane it is at once the B operand "X" and the A operand "X transposed" of a 16-deep product
+__device__ __forceinline__ void st_store(unsigned char *tile, int lane, const Sp2 &v) {
+    reinterpret_cast<uint2 *>(tile)[lane] = v.hi;
+    reinterpret_cast<uint2 *>(tile + ST_TILE)[lane] = v.lo;
+}
+__device__ __forceinline__ Sp2 st_load(const unsigned char *tile, int lane) {
+    Sp2 o;
+    o.hi = reinterpret_cast<const uint2 *>(tile)[lane];
+    o.lo = reinterpret_cast<const uint2 *>(tile + ST_TILE)[lane];
+    return o;
+}
+
+// ---- the state-independent 16 x 16 algebra of a block ------------------------------------------------
+// In the accumulator layout lane (r, g) holds rows 4 g + e of column r.  From the symmetric K K^T (`kk`) both
+// triangles: acc(A) (column < row) and acc(A^T) (row < column).  A matrix held in the accumulator layout is the
+// B operand "X" and the A operand "X^T" of a 16-deep product, so acc(X Y) = mfma(acc(X^T), acc(Y)) without any
+// data movement; squaring X and X^T side by side gives the powers 2, 4, 8 of A and of A^T, then
+//   P1 = (I + A^4)(I + A^8) = I + A^4 + A^8 + A^12,   P2^T = ((I - A)(I + A^2))^T = I - A^T + (A^2)^T - (A^3)^T,
+//   Tm = P2 P1:   acc(Tm^T) = mfma(acc(P1), acc(P2^T)),   acc(Tm) = mfma(acc(P2^T), acc(P1)).
+struct BlockInverse {
+    Sp2 p1, p2t;
+    __device__ __forceinline__ BlockInverse(const floatx4 &kk, int r, int g) {
+        const floatx4 zero = {0.f, 0.f, 0.f, 0.f};
+        floatx4 a, at, eye;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const int row = 4 * g + e;
+            a[e] = r < row ? kk[e] : 0.f;
+            at[e] = row < r ? kk[e] : 0.f;
+            eye[e] = row == r ? 1.f : 0.f;
+        }
+        const Sp2 x1 = split4(a), x1t = split4(at);
+        const floatx4 a2 = mma16(x1t, x1, zero), a2t = mma16(x1, x1t, zero);
+        const Sp2 x2 = split4(a2), x2t = split4(a2t);
+        const floatx4 a3t = mma16(x1, x2t, zero);                       // (A^3)^T = A^T (A^2)^T
+        const floatx4 a4 = mma16(x2t, x2, zero), a4t = mma16(x2, x2t, zero);
+        const Sp2 x4 = split4(a4), x4t = split4(a4t);
+        const floatx4 a8 = mma16(x4t, x4, zero);
+        const floatx4 a12 = mma16(x4t, split4(a8), zero);               // A^12 = A^4 A^8
+        p1 = split4(eye + a4 + a8 + a12);
+        p2t = split4(eye - at + a2t - a3t);
+    }
+    __device__ __forceinline__ floatx4 acc_tm_transposed() const { return mma16(p1, p2t, floatx4{0.f, 0.f, 0.f, 0.f}); }
+    __device__ __forceinline__ floatx4 acc_tm() const { return mma16(p2t, p1, floatx4{0.f, 0.f, 0.f, 0.f}); }
+};
+
+// ---- staging of an fp32 [T, 64] array into tiles (one wave per array and layout) -------------------
+// sixteen floats of one lane: token-major staging takes token lane >> 2, channels 16 (lane & 3) .. + 15;
+// channel-major staging takes channel `lane`, tokens 0 .. 15 of the block.  Rows at or past T read as zero.
+struct Raw16 {
+    float4 v[4];
+};
+// Loads are issued unconditionally (rows at or past T are read from row T - 1 and zeroed when the tile is
+// built): a load inside a branch would make every later wait for a load a wait for all of them.
+__device__ __forceinline__ Raw16 load_tm(const float *row0, int tok0, int T, int lane) {
+    Raw16 r;
+    const int t = min(tok0 + (lane >> 2), T - 1);
+    const float4 *p = reinterpret_cast<const float4 *>(row0 + (size_t)t * CH_N + 16 * (lane & 3));
+#pragma unroll
+    for (int a = 0; a < 4; ++a) r.v[a] = p[a];
+    return r;
+}
+__device__ __forceinline__ void store_tm(unsigned char *tile, int lane, const Raw16 &r, int tok0, int T) {
+    u16 *hi = reinterpret_cast<u16 *>(tile), *lo = reinterpret_cast<u16 *>(tile + TM_TILE);
+    const int o = (lane >> 2) * DTS + 4 * (lane & 3);
+    const float keep = tok0 + (lane >> 2) < T ? 1.f : 0.f;
+#pragma unroll
+    for (int a = 0; a < 4; ++a) {          // channels 16 q + 4 a + e sit at 16 a + 4 q + e
+        const Sp2 s = split4(r.v[a].x * keep, r.v[a].y * keep, r.v[a].z * keep, r.v[a].w * keep);
+        *reinterpret_cast<uint2 *>(hi + o + 16 * a) = s.hi;
+        *reinterpret_cast<uint2 *>(lo + o + 16 * a) = s.lo;
+    }
+}
+__device__ __forceinline__ Raw16 load_cm(const float *row0, int tok0, int T, int lane) {
+    Raw16 r;
+    float f[16];
+#pragma unroll
+    for (int t = 0; t < 16; ++t) f[t] = row0[(size_t)min(tok0 + t, T - 1) * CH_N + lane];
+#pragma unroll
+    for (int a = 0; a < 4; ++a) r.v[a] = make_float4(f[4 * a], f[4 * a + 1], f[4 * a + 2], f[4 * a + 3]);
+    return r;
+}
+__device__ __forceinline__ void store_cm(unsigned char *tile, int lane, const Raw16 &r, int tok0, int T, float sign = 1.f) {
+    u16 *hi = reinterpret_cast<u16 *>(tile), *lo = reinterpret_cast<u16 *>(tile + CM_TILE);
+#pragma unroll
+    for (int a = 0; a < 4; ++a) {
+        const int t = tok0 + 4 * a;
+        const Sp2 s = split4(t < T ? r.v[a].x * sign : 0.f, t + 1 < T ? r.v[a].y * sign : 0.f, t + 2 < T ? r.v[a].z * sign : 0.f,
+                             t + 3 < T ? r.v[a].w * sign : 0.f);
+        *reinterpret_cast<uint2 *>(hi + lane * DCS + 4 * a) = s.hi;
+        *reinterpret_cast<uint2 *>(lo + lane * DCS + 4 * a) = s.lo;
+    }
+}
+
+}  // namespace dfwc
+#endif  // __HIPCC__
+
+}  // namespace t2fw

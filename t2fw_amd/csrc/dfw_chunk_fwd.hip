@@ -1,0 +1,237 @@
+// Forward pass of the delta rule on the matrix cores, D = M = 64, fp32 tensors (algebra and precision:
+// dfw_chunk.hpp).  Two workgroups per batch row, one per half of the value channels: the rows S[d, :] of the
+// state, and with them the columns of V, Delta and O, never interact.  A workgroup has seven waves:
+//   two slab waves    each keeps 16 rows of the state in fp32 accumulators for the whole sequence; per block:
+//                     Delta = Tm V - K' S0^T, O = Q S0^T + Bq Delta, S += Delta^T K; they load V and store O
+//                     and Delta themselves (64 contiguous bytes per token)
+//   two matrix waves  everything that does not depend on the state, one stage ahead of the slab waves, one
+//                     block of the stage each: K K^T and K Q^T, the triangular masks, Tm = (I + A)^-1 by
+//                     squarings, K' = Tm K; they leave Tm^T and Bq^T as ready operands and K' as a tile in LDS
+//   three prep waves  K and Q token-major and K channel-major as bf16 head / remainder tiles, two stages ahead
+// One workgroup barrier per stage of two blocks.
+//
+// Replaces lfw_cuda_fwd_kernel of the reference's delta rule (t2fw/csrc/dfw_kernel.cu:105-196), semantics
+// t2fw/torch.py:44-53; `delta` is the tensor that kernel emits for its backward (dfw_kernel.cu:176-183).
+#include "common.hpp"
+#include "dfw_chunk.hpp"
+#include "dfw_scan.hpp"
+
+namespace t2fw {
+namespace {
+
+using namespace dfwc;
+
+constexpr int FW_THREADS = 512;
+// per block: raw tiles K token-major, Q token-major, K channel-major (head + remainder each) ...
+constexpr int FW_KT = 0, FW_QT = FW_KT + 2 * TM_TILE, FW_KC = FW_QT + 2 * TM_TILE, FW_RAW_BLOCK = FW_KC + 2 * CM_TILE;
+// ... and what the matrix waves make of them: K' token-major, Tm^T and Bq^T as operands
+constexpr int FW_KP = 0, FW_TT = FW_KP + 2 * TM_TILE, FW_BQT = FW_TT + 2 * ST_TILE, FW_ST_BLOCK = FW_BQT + 2 * ST_TILE;
+constexpr int FW_RAW = 0;                                        // three stages of raw tiles
+constexpr int FW_ST = FW_RAW + 3 * DNB * FW_RAW_BLOCK;           // two stages of the matrix waves' results
+constexpr int FW_SMEM = FW_ST + 2 * DNB * FW_ST_BLOCK;
+static_assert(FW_SMEM <= 160 * 1024, "forward tiles exceed the LDS of one CU");
+
+__device__ __forceinline__ unsigned char *raw_block(unsigned char *smem, int stage, int bb) {
+    return smem + FW_RAW + ((stage % 3) * DNB + bb) * FW_RAW_BLOCK;
+}
+__device__ __forceinline__ unsigned char *st_block(unsigned char *smem, int stage, int bb) {
+    return smem + FW_ST + ((stage & 1) * DNB + bb) * FW_ST_BLOCK;
+}
+
+// One array into one kind of tile, for every stage of the sequence, two stages ahead of the slab waves.  The
+// loads of a stage are issued one stage before its tiles are built, into the register set that the stage
+// before last has left: two sets in turn, so that nothing waits for a load in the stage that issued it.
+template <bool CHANNEL_MAJOR, int NARR>
+__device__ __forceinline__ void prep_wave(unsigned char *smem, const float *row0, const float *row1, int off0, int off1, int T,
+                                          int nstages, int lane) {
+    Raw16 set_a[NARR][DNB], set_b[NARR][DNB];
+    auto load = [&](Raw16 (&r)[NARR][DNB], int stage) {
+#pragma unroll
+        for (int a = 0; a < NARR; ++a)
+#pragma unroll
+            for (int bb = 0; bb < DNB; ++bb) {
+                const int tok0 = (stage * DNB + bb) * DL;
+                r[a][bb] = CHANNEL_MAJOR ? load_cm(a ? row1 : row0, tok0, T, lane) : load_tm(a ? row1 : row0, tok0, T, lane);
+            }
+    };
+    auto tick_body = [&](int tick, Raw16 (&cur)[NARR][DNB], Raw16 (&nxt)[NARR][DNB]) {
+        load(nxt, min(tick + 1, nstages - 1));          // unconditional: the same loads in flight on every path
+        if (tick < nstages) {
+#pragma unroll
+            for (int a = 0; a < NARR; ++a)
+#pragma unroll
+                for (int bb = 0; bb < DNB; ++bb) {
+                    unsigned char *tile = raw_block(smem, tick, bb) + (a ? off1 : off0);
+                    const int tok0 = (tick * DNB + bb) * DL;
+                    if (CHANNEL_MAJOR)
+                        store_cm(tile, lane, cur[a][bb], tok0, T);
+                    else
+                        store_tm(tile, lane, cur[a][bb], tok0, T);
+                }
+        }
+        __syncthreads();
+    };
+    load(set_a, 0);
+    const int nticks = nstages + 2;
+    for (int tick = 0; tick < nticks; tick += 2) {
+        tick_body(tick, set_a, set_b);
+        if (tick + 1 < nticks) tick_body(tick + 1, set_b, set_a);
+    }
+}
+
+// The state-independent part of block `bb` of every stage, one stage ahead of the slab waves.
+__device__ __forceinline__ void structure_wave(unsigned char *smem, int nstages, int bb, int lane) {
+    const int r = lane & 15, g = lane >> 4;
+    const floatx4 zero = {0.f, 0.f, 0.f, 0.f};
+    for (int tick = 0; tick < nstages + 2; ++tick) {
+        const int stage = tick - 1;
+        if (stage >= 0 && stage < nstages) {
+            const unsigned char *raw = raw_block(smem, stage, bb);
+            const TmTile KT(raw + FW_KT), QT(raw + FW_QT);
+            const CmTile KC(raw + FW_KC);
+            const Sp4 k0 = KT.any_order(r, g, 0), k1 = KT.any_order(r, g, 1);
+            const Sp4 q0 = QT.any_order(r, g, 0), q1 = QT.any_order(r, g, 1);
+            const floatx4 kk = mma32(k1, k1, mma32(k0, k0, zero));      // [s = 4g+e][t = r] = k_s . k_t
+            const floatx4 kq = mma32(k1, q1, mma32(k0, q0, zero));      // [s = 4g+e][t = r] = k_s . q_t
+            floatx4 bqt;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) bqt[e] = 4 * g + e < r ? kq[e] : 0.f;      // Bq^T[s][t] = k_s . q_t for s < t
+            const BlockInverse inv(kk, r, g);
+            const Sp2 tt = split4(inv.acc_tm_transposed());
+            unsigned char *st = st_block(smem, stage, bb);
+            st_store(st + FW_TT, lane, tt);
+            st_store(st + FW_BQT, lane, split4(bqt));
+            // K'^T tile j: [m = 16 j + 4 g + e][t = r] = sum_s K[s][m] Tm[t][s]
+            floatx4 kp[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) kp[j] = mma16(KC.tokens(16 * j + r, g), tt, zero);
+            store_tm_from_acc(st + FW_KP, r, g, kp);
+        }
+        __syncthreads();
+    }
+}
+
+__device__ __forceinline__ void slab_wave(const DfwFwdArgs &p, unsigned char *smem, int64_t b, int d0, int nstages, int lane) {
+    const int r = lane & 15, g = lane >> 4, d = d0 + r, T = (int)p.T;
+    const floatx4 zero = {0.f, 0.f, 0.f, 0.f};
+    // token addresses: a wave-uniform base per block plus the lane's fixed offset (first token 4 g, channel d)
+    const float *const v = reinterpret_cast<const float *>(p.v) + b * p.T * CH_N;
+    float *const out = reinterpret_cast<float *>(p.out) + b * p.T * CH_N;
+    float *const delta = reinterpret_cast<float *>(p.delta) + b * p.T * CH_N;
+    const u32 lane_off = (u32)(4 * g * CH_N + d);
+    // S[j][e] = S[d][16 j + 4 g + e]
+    floatx4 S[4];
+    {
+        const float *s0 = reinterpret_cast<const float *>(p.s0) + (b * CH_N + d) * CH_N + 4 * g;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const float4 t = *reinterpret_cast<const float4 *>(s0 + 16 * j);
+            S[j] = floatx4{t.x, t.y, t.z, t.w};
+        }
+    }
+    // V of a stage: element [bb][e] is token (stage * DNB + bb) * 16 + 4 g + e; loaded one stage ahead into the
+    // register set the stage before has left
+    // (unconditional loads: tokens at or past T are read from token T - 1 and zeroed where they are used)
+    auto load_v = [&](floatx4 (&x)[DNB], int stage) {
+#pragma unroll
+        for (int bb = 0; bb < DNB; ++bb)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) x[bb][e] = v[(size_t)min((stage * DNB + bb) * DL + 4 * g + e, T - 1) * CH_N + d];
+    };
+    auto tick_body = [&](int tick, floatx4 (&vcur)[DNB], floatx4 (&vnxt)[DNB]) {
+        const int stage = tick - 2;
+        load_v(vnxt, min(max(stage + 1, 0), nstages - 1));
+        if (stage >= 0) {
+#pragma unroll
+            for (int bb = 0; bb < DNB; ++bb) {
+                const int tok0 = (stage * DNB + bb) * DL;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) vcur[bb][e] = tok0 + 4 * g + e < T ? vcur[bb][e] : 0.f;
+                const unsigned char *raw = raw_block(smem, stage, bb);
+                const unsigned char *st = st_block(smem, stage, bb);
+                const TmTile QT(raw + FW_QT), KP(st + FW_KP);
+                const CmTile KC(raw + FW_KC);
+                // Delta[tok 4g+e][d] = Tm V - K' S0^T: only the second term waits for the state
+                const floatx4 tv = mma16(st_load(st + FW_TT, lane), split4(vcur[bb]), zero);
+                const Sp4 sb0 = cat(split4(S[0]), split4(S[1])), sb1 = cat(split4(S[2]), split4(S[3]));
+                const floatx4 ks = mma32(KP.acc_order(r, g, 1), sb1, mma32(KP.acc_order(r, g, 0), sb0, zero));
+                const floatx4 dl = tv - ks;
+                const Sp2 dls = split4(dl);
+                // O = Q S0^T + Bq Delta
+                const floatx4 qs = mma32(QT.acc_order(r, g, 1), sb1, mma32(QT.acc_order(r, g, 0), sb0, zero));
+                const floatx4 o = qs + mma16(st_load(st + FW_BQT, lane), dls, zero);
+                float *const ob = out + (size_t)tok0 * CH_N, *const db = delta + (size_t)tok0 * CH_N;      // wave-uniform
+                if (tok0 + DL <= T) {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        ob[lane_off + e * CH_N] = o[e];
+                        db[lane_off + e * CH_N] = dl[e];
+                    }
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e)
+                        if (tok0 + 4 * g + e < T) {
+                            ob[lane_off + e * CH_N] = o[e];
+                            db[lane_off + e * CH_N] = dl[e];
+                        }
+                }
+                // S += Delta^T K
+#pragma unroll
+                for (int j = 0; j < 4; ++j) S[j] = mma16(KC.tokens(16 * j + r, g), dls, S[j]);
+            }
+        }
+        __syncthreads();
+    };
+    floatx4 v_a[DNB], v_b[DNB];
+    load_v(v_a, 0);
+    const int nticks = nstages + 2;
+    for (int tick = 0; tick < nticks; tick += 2) {      // stage 0 runs in tick 2: the even ticks use set a
+        tick_body(tick, v_a, v_b);
+        if (tick + 1 < nticks) tick_body(tick + 1, v_b, v_a);
+    }
+    float *fin = reinterpret_cast<float *>(p.final_state) + (b * CH_N + d) * CH_N + 4 * g;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) *reinterpret_cast<float4 *>(fin + 16 * j) = make_float4(S[j][0], S[j][1], S[j][2], S[j][3]);
+}
+
+// blockIdx = half * rows_padded + row with rows_padded a multiple of 8: the two halves of a row land on the
+// same XCD and share its L2 for K and Q, which both read
+__global__ __launch_bounds__(FW_THREADS) void dfw_chunk_fwd_kernel(DfwFwdArgs p, int rows_padded) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    const int half = (int)blockIdx.x >= rows_padded ? 1 : 0;
+    const int64_t b = (int)blockIdx.x - half * rows_padded;
+    if (b >= p.B) return;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
+    const int T = (int)p.T, nstages = (T + DL * DNB - 1) / (DL * DNB);
+    const float *const k = reinterpret_cast<const float *>(p.k) + b * p.T * CH_N;
+    const float *const q = reinterpret_cast<const float *>(p.q) + b * p.T * CH_N;
+    // Every wave that stays executes nstages + 2 workgroup barriers.  Wave i runs on SIMD i % 4: the slab waves,
+    // whose chain of dependent steps sets the kernel's duration, get SIMDs 0 and 1 to themselves (waves 4 and 5
+    // leave at once; a workgroup barrier waits only for the waves that are left), the matrix waves and the
+    // prep waves share SIMDs 2 and 3.
+    static_assert(DNB == 2, "one matrix wave per block of a stage");
+    if (wave < 2)
+        slab_wave(p, smem, b, 32 * half + 16 * wave, nstages, lane);
+    else if (wave < 4)
+        structure_wave(smem, nstages, wave - 2, lane);
+    else if (wave == 6)
+        prep_wave<false, 2>(smem, k, q, FW_KT, FW_QT, T, nstages, lane);
+    else if (wave == 7)
+        prep_wave<true, 1>(smem, k, k, FW_KC, FW_KC, T, nstages, lane);
+}
+
+}  // namespace
+
+int dfw_chunk_forward(const DfwFwdArgs &a, hipStream_t stream) {
+    if (a.D != CH_N || a.M != CH_N) return fail(T2FW_ERR_UNSUPPORTED, "the block-wise delta-rule kernels take D = M = 64");
+    if (a.T * CH_N >= 0x7fffffffLL || a.B > 0x1fffffffLL)
+        return fail(T2FW_ERR_UNSUPPORTED, "B=%lld T=%lld is too large for the block-wise delta-rule kernels", (long long)a.B, (long long)a.T);
+    auto kern = dfw_chunk_fwd_kernel;
+    int rc = enable_lds(reinterpret_cast<const void *>(kern), FW_SMEM, "hipFuncSetAttribute(delta-rule forward kernel)");
+    if (rc) return rc;
+    const int rows_padded = (int)((a.B + 7) / 8 * 8);
+    hipLaunchKernelGGL(kern, dim3(2u * (unsigned)rows_padded), dim3(FW_THREADS), FW_SMEM, stream, a, rows_padded);
+    return check_hip(hipGetLastError(), "dfw_chunk_fwd_kernel launch");
+}
+
+}  // namespace t2fw

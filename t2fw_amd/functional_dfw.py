@@ -5,7 +5,7 @@ and the final state saved by forward (t2fw/functional_dfw.py:46-51)."""
 import torch
 
 from . import _lib
-from .functional_lfw import _check_input, _dtype_code, _on_device
+from .functional_lfw import _check_input, _dtype_code, _flags, _on_device
 
 
 class DFWFunction(torch.autograd.Function):
@@ -38,7 +38,7 @@ class DFWFunction(torch.autograd.Function):
             delta = torch.empty_like(value)
             _lib.check(lib.t2fw_dfw_forward(
                 _lib.ptr(query), _lib.ptr(key), _lib.ptr(value), _lib.ptr(state), _lib.ptr(outputs),
-                _lib.ptr(final_state), _lib.ptr(delta), B, T, D, M, code, _lib.current_stream_handle(dev)))
+                _lib.ptr(final_state), _lib.ptr(delta), B, T, D, M, code, _flags(), _lib.current_stream_handle(dev)))
         ctx.save_for_backward(query, key, delta, final_state)
         return outputs, final_state
 
@@ -60,6 +60,6 @@ class DFWFunction(torch.autograd.Function):
             _lib.check(lib.t2fw_dfw_backward(
                 _lib.ptr(grad_output), _lib.ptr(grad_state), _lib.ptr(query), _lib.ptr(key), _lib.ptr(delta),
                 _lib.ptr(final_state), _lib.ptr(d_q), _lib.ptr(d_k), _lib.ptr(d_v), _lib.ptr(d_s),
-                B, T, D, M, _dtype_code(delta.dtype), _lib.current_stream_handle(dev)))
+                B, T, D, M, _dtype_code(delta.dtype), _flags(), _lib.current_stream_handle(dev)))
         # order of t2fw/csrc/dfw_kernel.cu:557
         return d_q, d_k, d_v, d_s

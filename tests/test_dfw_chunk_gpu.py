@@ -1,0 +1,94 @@
+"""GPU parity of the block-wise matrix-core kernels of the delta rule (D = M = 64, fp32 tensors) against
+the CPU oracle (fp64, same inputs), through the C ABI.  The operands of every contraction are split into a
+bf16 head and remainder, so the results are held to the tolerance of the exact per-step kernels
+(tests/test_dfw_gpu.py), not to a 16-bit one; the exact kernels (flag 1) are run on the same inputs."""
+import pytest
+import torch
+
+from oracle.dfw_ref import dfw_deltas, dfw_reference_grads
+from tests.test_dfw_gpu import NAMES, TOL_DFW, make_inputs
+from tests.test_lfw_gpu import assert_close
+
+pytestmark = pytest.mark.gpu
+TOL = TOL_DFW[torch.float32]
+
+
+def run_abi(q, k, v, s, go, gs, flags=0, backward=True):
+    from t2fw_amd import _lib
+    lib = _lib.load()
+    q, k, v, s = [t.cuda() for t in (q, k, v, s)]
+    B, T, D = v.shape
+    M = q.shape[2]
+    code = _lib.DTYPE_CODE[v.dtype]
+    st = _lib.current_stream_handle(v.device)
+    out, delta, fin = torch.empty_like(v), torch.empty_like(v), torch.empty_like(s)
+    P = _lib.ptr
+    _lib.check(lib.t2fw_dfw_forward(P(q), P(k), P(v), P(s), P(out), P(fin), P(delta), B, T, D, M, code, flags, st))
+    grads = None
+    if backward:
+        go_d, gs_d = go.cuda(), gs.cuda()
+        grads = [torch.empty_like(q), torch.empty_like(k), torch.empty_like(v), torch.empty_like(s)]
+        _lib.check(lib.t2fw_dfw_backward(P(go_d), P(gs_d), P(q), P(k), P(delta), P(fin), *[P(t) for t in grads],
+                                         B, T, D, M, code, flags, st))
+    torch.cuda.synchronize()
+    return out, fin, delta, grads
+
+
+def check(B, T, seed, key_scale=None, backward=True):
+    q, k, v, s, go, gs = make_inputs(B, T, 64, 64, torch.float32, seed)
+    if key_scale is not None:          # unnormalised keys of a chosen size instead of the reference test's
+        g = torch.Generator().manual_seed(seed + 1)
+        k = torch.randn(B, T, 64, generator=g) * key_scale
+    r_out, r_fin, r_grads = dfw_reference_grads(q, k, v, s, go, gs)
+    r_delta = dfw_deltas(q.double(), k.double(), v.double(), s.double())
+    for flags in (0, 1):
+        tag = " (flags %d)" % flags
+        out, fin, delta, grads = run_abi(q, k, v, s, go, gs, flags, backward)
+        assert_close(out, r_out, torch.float32, "outputs" + tag, tol=TOL)
+        assert_close(fin, r_fin, torch.float32, "final_state" + tag, tol=TOL)
+        assert_close(delta, r_delta, torch.float32, "delta" + tag, tol=TOL)
+        if backward:
+            for n, g, r in zip(NAMES, grads, r_grads):
+                assert_close(g, r, torch.float32, n + tag, tol=TOL)
+
+
+@pytest.mark.parametrize("T", [1, 15, 16, 17, 31, 32, 33, 47, 48, 64, 65, 100, 257, 1024])
+def test_sequence_lengths_around_block_and_stage_boundaries(T):
+    check(3, T, seed=100 + T)
+
+
+@pytest.mark.parametrize("B", [1, 8, 9, 130, 300])
+def test_batch_sizes_around_the_grid_padding(B):
+    check(B, 70, seed=200 + B)
+
+
+@pytest.mark.parametrize("scale", [0.05, 0.125, 0.2])
+def test_unnormalised_keys(scale):
+    """|k|^2 up to about 2.5: the triangular factors are far from the identity"""
+    check(2, 200, seed=300, key_scale=scale)
+
+
+def test_headline_shape_rows_against_the_oracle():
+    """B = 96, T = 1024 as the benchmark runs it; the oracle on three rows"""
+    q, k, v, s, go, gs = make_inputs(96, 1024, 64, 64, torch.float32, seed=5)
+    out, fin, delta, grads = run_abi(q, k, v, s, go, gs)
+    rows = [0, 47, 95]
+    r_out, r_fin, r_grads = dfw_reference_grads(q[rows], k[rows], v[rows], s[rows], go[rows], gs[rows])
+    assert_close(out[rows], r_out, torch.float32, "outputs", tol=TOL)
+    assert_close(fin[rows], r_fin, torch.float32, "final_state", tol=TOL)
+    for n, g, r in zip(NAMES, grads, r_grads):
+        assert_close(g[rows], r, torch.float32, n, tol=TOL)
+
+
+def test_autograd_function_uses_the_block_wise_kernels():
+    from t2fw.functional_dfw import DFWFunction
+    q, k, v, s, go, gs = make_inputs(4, 130, 64, 64, torch.float32, seed=9)
+    ins = [t.cuda().requires_grad_(True) for t in (q, k, v, s)]
+    out, fin = DFWFunction.apply(*ins)
+    out.backward(go.cuda(), retain_graph=True)
+    fin.backward(gs.cuda())
+    torch.cuda.synchronize()
+    r_out, r_fin, r_grads = dfw_reference_grads(q, k, v, s, go, gs)
+    assert_close(out, r_out, torch.float32, "outputs", tol=TOL)
+    for n, t, r in zip(NAMES, ins, r_grads):
+        assert_close(t.grad, r, torch.float32, n, tol=TOL)
