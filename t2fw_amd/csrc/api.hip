@@ -521,6 +521,9 @@ int t2fw_dfw_backward(const void *g_out, const void *g_state, const void *q, con
     a.g_out = g_out; a.g_state = g_state; a.q = q; a.k = k; a.delta = delta; a.final_state = final_state;
     a.d_q = d_q; a.d_k = d_k; a.d_v = d_v; a.d_s0 = d_s0;
     a.B = B; a.T = T; a.D = D; a.M = M;
+    if (dfw_chunk_ok(D, M, dtype, flags) && T * CH_N < 0x7fffffffLL &&
+        aligned16({g_out, g_state, q, k, delta, final_state, d_q, d_k, d_v, d_s0}))
+        return dfw_chunk_backward(a, st);
     return dfw_backward(a, dtype, st);
 }
 

@@ -176,10 +176,10 @@ __device__ __forceinline__ Raw16 load_tm(const float *row0, int tok0, int T, int
     for (int a = 0; a < 4; ++a) r.v[a] = p[a];
     return r;
 }
-__device__ __forceinline__ void store_tm(unsigned char *tile, int lane, const Raw16 &r, int tok0, int T) {
+__device__ __forceinline__ void store_tm(unsigned char *tile, int lane, const Raw16 &r, int tok0, int T, float sign = 1.f) {
     u16 *hi = reinterpret_cast<u16 *>(tile), *lo = reinterpret_cast<u16 *>(tile + TM_TILE);
     const int o = (lane >> 2) * DTS + 4 * (lane & 3);
-    const float keep = tok0 + (lane >> 2) < T ? 1.f : 0.f;
+    const float keep = tok0 + (lane >> 2) < T ? sign : 0.f;
 #pragma unroll
     for (int a = 0; a < 4; ++a) {          // channels 16 q + 4 a + e sit at 16 a + 4 q + e
         const Sp2 s = split4(r.v[a].x * keep, r.v[a].y * keep, r.v[a].z * keep, r.v[a].w * keep);
@@ -205,6 +205,67 @@ __device__ __forceinline__ void store_cm(unsigned char *tile, int lane, const Ra
                              t + 3 < T ? r.v[a].w * sign : 0.f);
         *reinterpret_cast<uint2 *>(hi + lane * DCS + 4 * a) = s.hi;
         *reinterpret_cast<uint2 *>(lo + lane * DCS + 4 * a) = s.lo;
+    }
+}
+
+// ---- staging pipeline shared by the backward kernels ---------------------------------------------------
+// LDS as rings of stages: raw tiles live three stages (built two stages ahead of the slab waves, read by the
+// matrix waves one stage ahead and by the slab waves), the matrix waves' results two.
+template <int RAW_BLOCK, int ST_BLOCK, int NBLK> struct Ring {
+    static constexpr int ST = 3 * NBLK * RAW_BLOCK;
+    static constexpr int SMEM = ST + 2 * NBLK * ST_BLOCK;
+    static __device__ __forceinline__ unsigned char *raw(unsigned char *smem, int stage, int bb) {
+        return smem + ((stage % 3) * NBLK + bb) * RAW_BLOCK;
+    }
+    static __device__ __forceinline__ unsigned char *st(unsigned char *smem, int stage, int bb) {
+        return smem + ST + ((stage & 1) * NBLK + bb) * ST_BLOCK;
+    }
+};
+
+// One wave stages NJOBS arrays (all token-major or all channel-major) for every stage, two stages ahead of the
+// slab waves.  Loads of a stage are issued, unconditionally, one stage before its tiles are built, into the
+// register set the stage before last has left.  tok0_of(stage, bb): first token of a block (at or past T: a
+// block of zeros).
+struct PrepJob {
+    const float *src;       // token 0 of the batch row
+    int off;                // byte offset of the tile inside a block's raw tiles
+    float sign;             // the tile holds sign * src
+};
+template <typename RING, int NBLK, bool CHANNEL_MAJOR, int NJOBS, typename TOK0>
+__device__ __forceinline__ void prep_wave_jobs(unsigned char *smem, const PrepJob (&jobs)[NJOBS], int T, int nstages, int lane,
+                                               TOK0 tok0_of) {
+    Raw16 set_a[NJOBS][NBLK], set_b[NJOBS][NBLK];
+    auto load = [&](Raw16 (&r)[NJOBS][NBLK], int stage) {
+#pragma unroll
+        for (int a = 0; a < NJOBS; ++a)
+#pragma unroll
+            for (int bb = 0; bb < NBLK; ++bb) {
+                const int tok0 = tok0_of(stage, bb);
+                r[a][bb] = CHANNEL_MAJOR ? load_cm(jobs[a].src, tok0, T, lane) : load_tm(jobs[a].src, tok0, T, lane);
+            }
+    };
+    auto tick_body = [&](int tick, Raw16 (&cur)[NJOBS][NBLK], Raw16 (&nxt)[NJOBS][NBLK]) {
+        load(nxt, min(tick + 1, nstages - 1));
+        if (tick < nstages) {
+#pragma unroll
+            for (int a = 0; a < NJOBS; ++a)
+#pragma unroll
+                for (int bb = 0; bb < NBLK; ++bb) {
+                    unsigned char *tile = RING::raw(smem, tick, bb) + jobs[a].off;
+                    const int tok0 = tok0_of(tick, bb);
+                    if (CHANNEL_MAJOR)
+                        store_cm(tile, lane, cur[a][bb], tok0, T, jobs[a].sign);
+                    else
+                        store_tm(tile, lane, cur[a][bb], tok0, T, jobs[a].sign);
+                }
+        }
+        __syncthreads();
+    };
+    load(set_a, 0);
+    const int nticks = nstages + 2;
+    for (int tick = 0; tick < nticks; tick += 2) {
+        tick_body(tick, set_a, set_b);
+        if (tick + 1 < nticks) tick_body(tick + 1, set_b, set_a);
     }
 }
 

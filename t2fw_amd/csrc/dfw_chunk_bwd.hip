@@ -1,0 +1,329 @@
+// Backward pass of the delta rule on the matrix cores, D = M = 64, fp32 tensors (block algebra, precision
+// and staging: dfw_chunk.hpp).  Blocks of 16 steps are visited last to first.  With g = dL/dO of the block,
+// G_end the adjoint of the state after it, Delta the block's saved deltas and Tm = (I + A)^-1:
+//   dDelta = Bq^T g + K G_end^T            dU = Tm^T dDelta  (= d_value)
+//   G_start = G_end + g^T Q - dU^T K       (d_state = G before the first block)
+//   S0 = S_end - Delta^T K                 (the state walked backwards from final_state, as the reference does)
+//   d_query = g S0 + X1 K                  X1[t][s] = g_t . delta_s   (s < t)
+//   d_key   = X1^T Q + Delta G_end - dU S0 + (X2 + X2^T) K            X2[t][s] = -dU_t . delta_s  (s < t)
+// Two launches, as in the reference (t2fw/csrc/dfw_kernel.cu:203-283 and :290-384):
+//   value side  one workgroup per (row, half of the value channels): G rows in fp32 accumulators; writes d_value
+//               and d_state.  Its chain per block is  G_end -> dU = Tm^T Bq^T g + (Tm^T K) G_end^T -> G_start,
+//               with Tm, Bq and K'' = Tm^T K prepared ahead by the matrix waves.
+//   key side    one workgroup per (row, half of the key channels): columns of S and of G in fp32 accumulators,
+//               both plain running sums (it reads d_value from the first launch); writes d_query and d_key.
+#include "common.hpp"
+#include "dfw_chunk.hpp"
+#include "dfw_scan.hpp"
+
+namespace t2fw {
+namespace {
+
+using namespace dfwc;
+
+constexpr int BW_THREADS = 512;
+
+// ---- value side -----------------------------------------------------------------------------------------
+constexpr int VS_KT = 0, VS_QT = VS_KT + 2 * TM_TILE, VS_KC = VS_QT + 2 * TM_TILE, VS_QC = VS_KC + 2 * CM_TILE,
+              VS_RAW_BLOCK = VS_QC + 2 * CM_TILE;
+constexpr int VS_KPP = 0, VS_TM = VS_KPP + 2 * TM_TILE, VS_BQ = VS_TM + 2 * ST_TILE, VS_ST_BLOCK = VS_BQ + 2 * ST_TILE;
+using VsRing = Ring<VS_RAW_BLOCK, VS_ST_BLOCK, DNB>;
+static_assert(VsRing::SMEM <= 160 * 1024, "value-side tiles exceed the LDS of one CU");
+
+// first token of block `bb` of a stage when the blocks are visited last to first
+__device__ __forceinline__ int reverse_tok0(int nblocks, int nblk_per_stage, int stage, int bb) {
+    return (nblocks - 1 - (stage * nblk_per_stage + bb)) * DL;
+}
+
+__device__ __forceinline__ void vs_structure_wave(unsigned char *smem, int nstages, int bb, int lane) {
+    const int r = lane & 15, g = lane >> 4;
+    const floatx4 zero = {0.f, 0.f, 0.f, 0.f};
+    for (int tick = 0; tick < nstages + 2; ++tick) {
+        const int stage = tick - 1;
+        if (stage >= 0 && stage < nstages) {
+            const unsigned char *raw = VsRing::raw(smem, stage, bb);
+            const TmTile KT(raw + VS_KT), QT(raw + VS_QT);
+            const CmTile KC(raw + VS_KC);
+            const Sp4 k0 = KT.any_order(r, g, 0), k1 = KT.any_order(r, g, 1);
+            const Sp4 q0 = QT.any_order(r, g, 0), q1 = QT.any_order(r, g, 1);
+            const floatx4 kk = mma32(k1, k1, mma32(k0, k0, zero));
+            const floatx4 qk = mma32(q1, k1, mma32(q0, k0, zero));      // [t = 4g+e][s = r] = q_t . k_s
+            floatx4 bq;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) bq[e] = r < 4 * g + e ? qk[e] : 0.f;       // Bq[t][s] for s < t
+            const BlockInverse inv(kk, r, g);
+            const Sp2 tm = split4(inv.acc_tm());
+            unsigned char *st = VsRing::st(smem, stage, bb);
+            st_store(st + VS_TM, lane, tm);
+            st_store(st + VS_BQ, lane, split4(bq));
+            // K''^T tile j: [m = 16 j + 4 g + e][t = r] = sum_s K[s][m] Tm[s][t]   (K'' = Tm^T K)
+            floatx4 kpp[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) kpp[j] = mma16(KC.tokens(16 * j + r, g), tm, zero);
+            store_tm_from_acc(st + VS_KPP, r, g, kpp);
+        }
+        __syncthreads();
+    }
+}
+
+__device__ __forceinline__ void vs_slab_wave(const DfwBwdArgs &p, unsigned char *smem, int64_t b, int d0, int nstages, int lane) {
+    const int r = lane & 15, g = lane >> 4, d = d0 + r, T = (int)p.T, nblocks = nstages * DNB;
+    const floatx4 zero = {0.f, 0.f, 0.f, 0.f};
+    const float *const go = reinterpret_cast<const float *>(p.g_out) + b * p.T * CH_N;
+    float *const d_v = reinterpret_cast<float *>(p.d_v) + b * p.T * CH_N;
+    const u32 lane_off = (u32)(4 * g * CH_N + d);
+    // G[j][e] = G[d][16 j + 4 g + e]
+    floatx4 G[4];
+    {
+        const float *gs = reinterpret_cast<const float *>(p.g_state) + (b * CH_N + d) * CH_N + 4 * g;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const float4 t = *reinterpret_cast<const float4 *>(gs + 16 * j);
+            G[j] = floatx4{t.x, t.y, t.z, t.w};
+        }
+    }
+    auto load_g = [&](floatx4 (&x)[DNB], int stage) {
+#pragma unroll
+        for (int bb = 0; bb < DNB; ++bb)
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+                x[bb][e] = go[(size_t)min(reverse_tok0(nblocks, DNB, stage, bb) + 4 * g + e, T - 1) * CH_N + d];
+    };
+    auto tick_body = [&](int tick, floatx4 (&gcur)[DNB], floatx4 (&gnxt)[DNB]) {
+        const int stage = tick - 2;
+        load_g(gnxt, min(max(stage + 1, 0), nstages - 1));
+        if (stage >= 0) {
+#pragma unroll
+            for (int bb = 0; bb < DNB; ++bb) {
+                const int tok0 = reverse_tok0(nblocks, DNB, stage, bb);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) gcur[bb][e] = tok0 + 4 * g + e < T ? gcur[bb][e] : 0.f;
+                const unsigned char *raw = VsRing::raw(smem, stage, bb);
+                const unsigned char *st = VsRing::st(smem, stage, bb);
+                const TmTile KPP(st + VS_KPP);
+                const CmTile KC(raw + VS_KC), QC(raw + VS_QC);
+                // dU[tok 4g+e][d] = Tm^T (Bq^T g) + K'' G_end^T: only the second term waits for the adjoint
+                const Sp2 gs = split4(gcur[bb]);
+                const floatx4 bg = mma16(st_load(st + VS_BQ, lane), gs, zero);
+                const floatx4 tbg = mma16(st_load(st + VS_TM, lane), split4(bg), zero);
+                const Sp4 gb0 = cat(split4(G[0]), split4(G[1])), gb1 = cat(split4(G[2]), split4(G[3]));
+                const floatx4 kg = mma32(KPP.acc_order(r, g, 1), gb1, mma32(KPP.acc_order(r, g, 0), gb0, zero));
+                const floatx4 du = tbg + kg;
+                float *const vb = d_v + (size_t)tok0 * CH_N;        // wave-uniform
+                if (tok0 + DL <= T) {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) vb[lane_off + e * CH_N] = du[e];
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e)
+                        if (tok0 + 4 * g + e < T) vb[lane_off + e * CH_N] = du[e];
+                }
+                // G += g^T Q - dU^T K
+                const Sp2 ndu = split4(-du);
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    G[j] = mma16(QC.tokens(16 * j + r, g), gs, G[j]);
+                    G[j] = mma16(KC.tokens(16 * j + r, g), ndu, G[j]);
+                }
+            }
+        }
+        __syncthreads();
+    };
+    floatx4 g_a[DNB], g_b[DNB];
+    load_g(g_a, 0);
+    const int nticks = nstages + 2;
+    for (int tick = 0; tick < nticks; tick += 2) {
+        tick_body(tick, g_a, g_b);
+        if (tick + 1 < nticks) tick_body(tick + 1, g_b, g_a);
+    }
+    float *ds0 = reinterpret_cast<float *>(p.d_s0) + (b * CH_N + d) * CH_N + 4 * g;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) *reinterpret_cast<float4 *>(ds0 + 16 * j) = make_float4(G[j][0], G[j][1], G[j][2], G[j][3]);
+}
+
+// blockIdx = half * rows_padded + row (rows_padded a multiple of 8: both halves of a row on one XCD).  Waves 0, 1:
+// slab waves, alone on SIMDs 0 and 1; waves 2, 3: matrix waves; waves 6, 7: prep waves; waves 4, 5 leave at once.
+__global__ __launch_bounds__(BW_THREADS) void dfw_chunk_bwd_value_kernel(DfwBwdArgs p, int rows_padded) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    const int half = (int)blockIdx.x >= rows_padded ? 1 : 0;
+    const int64_t b = (int)blockIdx.x - half * rows_padded;
+    if (b >= p.B) return;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
+    const int T = (int)p.T, nstages = (T + DL * DNB - 1) / (DL * DNB), nblocks = nstages * DNB;
+    const float *const k = reinterpret_cast<const float *>(p.k) + b * p.T * CH_N;
+    const float *const q = reinterpret_cast<const float *>(p.q) + b * p.T * CH_N;
+    auto tok0_of = [=](int stage, int bb) { return reverse_tok0(nblocks, DNB, stage, bb); };
+    static_assert(DNB == 2, "one matrix wave per block of a stage");
+    if (wave < 2) {
+        vs_slab_wave(p, smem, b, 32 * half + 16 * wave, nstages, lane);
+    } else if (wave < 4) {
+        vs_structure_wave(smem, nstages, wave - 2, lane);
+    } else if (wave == 6) {
+        const PrepJob jobs[2] = {{k, VS_KT, 1.f}, {q, VS_QT, 1.f}};
+        prep_wave_jobs<VsRing, DNB, false, 2>(smem, jobs, T, nstages, lane, tok0_of);
+    } else if (wave == 7) {
+        const PrepJob jobs[2] = {{k, VS_KC, 1.f}, {q, VS_QC, 1.f}};
+        prep_wave_jobs<VsRing, DNB, true, 2>(smem, jobs, T, nstages, lane, tok0_of);
+    }
+}
+
+// ---- key side -------------------------------------------------------------------------------------------
+// one block per stage: eight raw tiles per block leave no room for more
+constexpr int KS_DT = 0, KS_GT = KS_DT + 2 * TM_TILE, KS_NUT = KS_GT + 2 * TM_TILE, KS_NDC = KS_NUT + 2 * TM_TILE,
+              KS_GC = KS_NDC + 2 * CM_TILE, KS_NUC = KS_GC + 2 * CM_TILE, KS_KC = KS_NUC + 2 * CM_TILE,
+              KS_QC = KS_KC + 2 * CM_TILE, KS_RAW_BLOCK = KS_QC + 2 * CM_TILE;
+constexpr int KS_X1 = 0, KS_X1T = KS_X1 + 2 * ST_TILE, KS_X2S = KS_X1T + 2 * ST_TILE, KS_ST_BLOCK = KS_X2S + 2 * ST_TILE;
+using KsRing = Ring<KS_RAW_BLOCK, KS_ST_BLOCK, 1>;
+static_assert(KsRing::SMEM <= 160 * 1024, "key-side tiles exceed the LDS of one CU");
+
+__device__ __forceinline__ void ks_structure_wave(unsigned char *smem, int nstages, int lane) {
+    const int r = lane & 15, g = lane >> 4;
+    const floatx4 zero = {0.f, 0.f, 0.f, 0.f};
+    for (int tick = 0; tick < nstages + 2; ++tick) {
+        const int stage = tick - 1;
+        if (stage >= 0 && stage < nstages) {
+            const unsigned char *raw = KsRing::raw(smem, stage, 0);
+            const TmTile DT(raw + KS_DT), GT(raw + KS_GT), NUT(raw + KS_NUT);
+            const Sp4 d0 = DT.any_order(r, g, 0), d1 = DT.any_order(r, g, 1);
+            const Sp4 g0 = GT.any_order(r, g, 0), g1 = GT.any_order(r, g, 1);
+            const Sp4 u0 = NUT.any_order(r, g, 0), u1 = NUT.any_order(r, g, 1);
+            const floatx4 z = mma32(g1, d1, mma32(g0, d0, zero));       // [t = 4g+e][s = r] =  g_t . delta_s
+            const floatx4 zt = mma32(d1, g1, mma32(d0, g0, zero));      // [s = 4g+e][t = r] =  delta_s . g_t
+            const floatx4 y = mma32(u1, d1, mma32(u0, d0, zero));       // [t = 4g+e][s = r] = -dU_t . delta_s
+            const floatx4 yt = mma32(d1, u1, mma32(d0, u0, zero));      // [s = 4g+e][t = r] = -delta_s . dU_t
+            floatx4 x1, x1t, x2s;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const int row = 4 * g + e;
+                x1[e] = r < row ? z[e] : 0.f;                 // X1[t][s], s < t
+                x1t[e] = row < r ? zt[e] : 0.f;               // X1^T[s][t], s < t
+                x2s[e] = r < row ? y[e] : (row < r ? yt[e] : 0.f);      // X2 + X2^T
+            }
+            unsigned char *st = KsRing::st(smem, stage, 0);
+            st_store(st + KS_X1, lane, split4(x1));
+            st_store(st + KS_X1T, lane, split4(x1t));
+            st_store(st + KS_X2S, lane, split4(x2s));
+        }
+        __syncthreads();
+    }
+}
+
+__device__ __forceinline__ void ks_slab_wave(const DfwBwdArgs &p, unsigned char *smem, int64_t b, int m0, int nstages, int lane) {
+    const int r = lane & 15, g = lane >> 4, m = m0 + r, T = (int)p.T, nblocks = nstages;
+    const floatx4 zero = {0.f, 0.f, 0.f, 0.f};
+    float *const d_q = reinterpret_cast<float *>(p.d_q) + b * p.T * CH_N;
+    float *const d_k = reinterpret_cast<float *>(p.d_k) + b * p.T * CH_N;
+    const u32 lane_off = (u32)(4 * g * CH_N + m);
+    // S[j][e] = S[d = 16 j + 4 g + e][m], G likewise: columns of the state and of its adjoint
+    floatx4 S[4], G[4];
+    {
+        const float *fs = reinterpret_cast<const float *>(p.final_state) + b * CH_N * CH_N + m;
+        const float *gs = reinterpret_cast<const float *>(p.g_state) + b * CH_N * CH_N + m;
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                S[j][e] = fs[(16 * j + 4 * g + e) * CH_N];
+                G[j][e] = gs[(16 * j + 4 * g + e) * CH_N];
+            }
+    }
+    for (int tick = 0; tick < nstages + 2; ++tick) {
+        const int stage = tick - 2;
+        if (stage >= 0) {
+            const int tok0 = reverse_tok0(nblocks, 1, stage, 0);
+            const unsigned char *raw = KsRing::raw(smem, stage, 0);
+            const unsigned char *st = KsRing::st(smem, stage, 0);
+            const TmTile DT(raw + KS_DT), GT(raw + KS_GT), NUT(raw + KS_NUT);
+            const CmTile NDC(raw + KS_NDC), GC(raw + KS_GC), NUC(raw + KS_NUC), KC(raw + KS_KC), QC(raw + KS_QC);
+            const Sp2 kb = KC.tokens(m, g), qb = QC.tokens(m, g);          // K[t = 4g+e][m], Q[t][m]
+            // the adjoint after the block, before it takes the block in
+            const Sp4 gb0 = cat(split4(G[0]), split4(G[1])), gb1 = cat(split4(G[2]), split4(G[3]));
+            // S0 = S_end - Delta^T K
+#pragma unroll
+            for (int j = 0; j < 4; ++j) S[j] = mma16(NDC.tokens(16 * j + r, g), kb, S[j]);
+            const Sp4 sb0 = cat(split4(S[0]), split4(S[1])), sb1 = cat(split4(S[2]), split4(S[3]));
+            // d_query[t][m] = g S0 + X1 K
+            const floatx4 dq = mma32(GT.acc_order(r, g, 1), sb1, mma32(GT.acc_order(r, g, 0), sb0, zero)) +
+                               mma16(st_load(st + KS_X1T, lane), kb, zero);
+            // d_key[s][m] = Delta G_end - dU S0 + X1^T Q + (X2 + X2^T) K
+            const floatx4 dk = mma32(NUT.acc_order(r, g, 1), sb1,
+                                     mma32(NUT.acc_order(r, g, 0), sb0,
+                                           mma32(DT.acc_order(r, g, 1), gb1, mma32(DT.acc_order(r, g, 0), gb0, zero)))) +
+                               mma16(st_load(st + KS_X2S, lane), kb, mma16(st_load(st + KS_X1, lane), qb, zero));
+            float *const qo = d_q + (size_t)tok0 * CH_N, *const ko = d_k + (size_t)tok0 * CH_N;      // wave-uniform
+            if (tok0 + DL <= T) {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    qo[lane_off + e * CH_N] = dq[e];
+                    ko[lane_off + e * CH_N] = dk[e];
+                }
+            } else {
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                    if (tok0 + 4 * g + e < T) {
+                        qo[lane_off + e * CH_N] = dq[e];
+                        ko[lane_off + e * CH_N] = dk[e];
+                    }
+            }
+            // G_start = G_end + g^T Q - dU^T K
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                G[j] = mma16(GC.tokens(16 * j + r, g), qb, G[j]);
+                G[j] = mma16(NUC.tokens(16 * j + r, g), kb, G[j]);
+            }
+        }
+        __syncthreads();
+    }
+}
+
+// Waves 0, 1: slab waves (16 key channels each), alone on SIMDs 0 and 1; wave 2: matrix wave; waves 3, 6, 7: prep
+// waves; waves 4, 5 leave at once.
+__global__ __launch_bounds__(BW_THREADS) void dfw_chunk_bwd_key_kernel(DfwBwdArgs p, int rows_padded) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    const int half = (int)blockIdx.x >= rows_padded ? 1 : 0;
+    const int64_t b = (int)blockIdx.x - half * rows_padded;
+    if (b >= p.B) return;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
+    const int T = (int)p.T, nstages = (T + DL - 1) / DL;
+    const int64_t row = b * p.T * CH_N;
+    const float *const k = reinterpret_cast<const float *>(p.k) + row;
+    const float *const q = reinterpret_cast<const float *>(p.q) + row;
+    const float *const dl = reinterpret_cast<const float *>(p.delta) + row;
+    const float *const go = reinterpret_cast<const float *>(p.g_out) + row;
+    const float *const dv = reinterpret_cast<const float *>(p.d_v) + row;
+    auto tok0_of = [=](int stage, int bb) { return reverse_tok0(nstages, 1, stage, bb); };
+    if (wave < 2) {
+        ks_slab_wave(p, smem, b, 32 * half + 16 * wave, nstages, lane);
+    } else if (wave == 2) {
+        ks_structure_wave(smem, nstages, lane);
+    } else if (wave == 3) {
+        const PrepJob jobs[3] = {{dl, KS_DT, 1.f}, {go, KS_GT, 1.f}, {dv, KS_NUT, -1.f}};
+        prep_wave_jobs<KsRing, 1, false, 3>(smem, jobs, T, nstages, lane, tok0_of);
+    } else if (wave == 6) {
+        const PrepJob jobs[3] = {{dl, KS_NDC, -1.f}, {go, KS_GC, 1.f}, {dv, KS_NUC, -1.f}};
+        prep_wave_jobs<KsRing, 1, true, 3>(smem, jobs, T, nstages, lane, tok0_of);
+    } else if (wave == 7) {
+        const PrepJob jobs[2] = {{k, KS_KC, 1.f}, {q, KS_QC, 1.f}};
+        prep_wave_jobs<KsRing, 1, true, 2>(smem, jobs, T, nstages, lane, tok0_of);
+    }
+}
+
+}  // namespace
+
+int dfw_chunk_backward(const DfwBwdArgs &a, hipStream_t stream) {
+    if (a.D != CH_N || a.M != CH_N) return fail(T2FW_ERR_UNSUPPORTED, "the block-wise delta-rule kernels take D = M = 64");
+    if (a.T * CH_N >= 0x7fffffffLL || a.B > 0x1fffffffLL)
+        return fail(T2FW_ERR_UNSUPPORTED, "B=%lld T=%lld is too large for the block-wise delta-rule kernels", (long long)a.B, (long long)a.T);
+    auto value_side = dfw_chunk_bwd_value_kernel;
+    auto key_side = dfw_chunk_bwd_key_kernel;
+    int rc = enable_lds(reinterpret_cast<const void *>(value_side), VsRing::SMEM, "hipFuncSetAttribute(delta-rule backward kernel, value side)");
+    if (rc) return rc;
+    if ((rc = enable_lds(reinterpret_cast<const void *>(key_side), KsRing::SMEM, "hipFuncSetAttribute(delta-rule backward kernel, key side)"))) return rc;
+    const int rows_padded = (int)((a.B + 7) / 8 * 8);
+    hipLaunchKernelGGL(value_side, dim3(2u * (unsigned)rows_padded), dim3(BW_THREADS), VsRing::SMEM, stream, a, rows_padded);
+    if ((rc = check_hip(hipGetLastError(), "dfw_chunk_bwd_value_kernel launch"))) return rc;
+    hipLaunchKernelGGL(key_side, dim3(2u * (unsigned)rows_padded), dim3(BW_THREADS), KsRing::SMEM, stream, a, rows_padded);
+    return check_hip(hipGetLastError(), "dfw_chunk_bwd_key_kernel launch");
+}
+
+}  // namespace t2fw
