@@ -127,9 +127,34 @@ size_t forward_workspace_bytes(int64_t B, int64_t D, int64_t K, int32_t dtype, i
     return 0;
 }
 
+// Checkpoint intervals that are a multiple of 32 other than 32 and 64 (the forward takes them, the backward
+// kernels do not): the backward call first runs the forward kernel once more at an interval the backward takes,
+// into checkpoints of its own in the workspace, and then proceeds as for that interval.
+int32_t backward_interval(int32_t C) {
+    if (C == 32 || C == 64 || C < 32 || C % 32 != 0) return C;
+    return C % 64 == 0 ? 64 : 32;
+}
+size_t align256(size_t n) { return (n + 255) / 256 * 256; }
+
+struct DenseScratch {
+    size_t ckpt, out, next, total;      // byte offsets from the start of the workspace
+};
+DenseScratch dense_scratch(size_t inner, int64_t B, int64_t T, int32_t Cd, size_t es) {
+    const int64_t nc = T <= 0 ? 1 : (T + Cd - 1) / Cd;
+    DenseScratch d;
+    d.ckpt = align256(inner);
+    d.out = d.ckpt + align256((size_t)(B * nc) * CH_N * CH_N * es);
+    d.next = d.out + align256((size_t)(B * (T > 0 ? T : 1)) * CH_N * es);
+    d.total = d.next + align256((size_t)B * CH_N * CH_N * es);
+    return d;
+}
+
 size_t backward_workspace_bytes(int64_t B, int64_t T, int64_t D, int64_t K, int32_t C, int32_t dtype, int32_t flags) {
-    if (B > 0 && chunk_shape_ok(D, K, dtype, flags))
-        return par_ok(B, T, C, flags) ? par_scratch(B, T, C).total : 2 * row_flag_bytes(B);
+    if (B > 0 && chunk_shape_ok(D, K, dtype, flags)) {
+        const int32_t Cd = backward_interval(C);
+        const size_t inner = par_ok(B, T, Cd, flags) ? par_scratch(B, T, Cd).total : 2 * row_flag_bytes(B);
+        return Cd == C ? inner : dense_scratch(inner, B, T, Cd, elem_size(dtype)).total;
+    }
     return 0;
 }
 
@@ -219,8 +244,9 @@ int t2fw_lfw_flag_regions(int64_t B, int64_t T, int64_t D, int64_t K, int32_t C,
     const int64_t slots = 2 * chunk_rows_padded(B), region = (int64_t)row_flag_bytes(B);
     regions[0] = 0; regions[1] = slots;                  // forward verdicts
     regions[2] = region; regions[3] = slots;             // forward hints for the backward
-    if (C == 32 || C == 64) {                            // else the backward runs on the exact kernels
-        if (par_ok(B, T, C, flags)) {
+    const int32_t Cd = backward_interval(C);
+    if (Cd == 32 || Cd == 64) {                          // else the backward runs on the exact kernels
+        if (par_ok(B, T, Cd, flags)) {
             regions[4] = region; regions[5] = B;
         } else {
             regions[4] = 0; regions[5] = slots;
@@ -341,9 +367,9 @@ int t2fw_lfw_forward_heads(const void *x, const void *f, const void *q, const vo
 }
 
 static int lfw_backward_rows(const void *g_out, const void *g_state, const void *x, const void *f, const void *q,
-                             const void *k, const void *f_key, const void *ckpt, void *d_x, void *d_f, void *d_q,
-                             void *d_k, void *d_f_key, void *d_s0, int64_t B, int64_t T, int64_t heads, int64_t D,
-                             int64_t K, int32_t C, int32_t dtype, int32_t flags, void *workspace,
+                             const void *k, const void *f_key, const void *s0, const void *ckpt, void *d_x, void *d_f,
+                             void *d_q, void *d_k, void *d_f_key, void *d_s0, int64_t B, int64_t T, int64_t heads,
+                             int64_t D, int64_t K, int32_t C, int32_t dtype, int32_t flags, void *workspace,
                              size_t workspace_bytes, void *stream) {
     const size_t es = elem_size(dtype);
     if (es == 0) return fail(T2FW_ERR_BAD_DTYPE, "unknown dtype code %d", dtype);
@@ -374,12 +400,27 @@ static int lfw_backward_rows(const void *g_out, const void *g_state, const void 
     a.heads = (int32_t)heads;
     a.NC = t2fw_lfw_num_ckpt(T, C);
 
+    const int32_t C_given = C;
+    C = backward_interval(C);
     if (chunk_shape_ok(D, K, dtype, flags) && (C == 32 || C == 64) && T * heads < CHUNK_MAX_T &&
-        aligned16({g_out, g_state, x, f, q, k, f_key, ckpt, d_x, d_f, d_q, d_k, d_f_key, d_s0})) {
-        const size_t need = backward_workspace_bytes(B, T, D, K, C, dtype, flags);
+        aligned16({g_out, g_state, x, f, q, k, f_key, ckpt, d_x, d_f, d_q, d_k, d_f_key, d_s0}) &&
+        (C == C_given || (s0 != nullptr && aligned16({s0})))) {
+        const size_t need = backward_workspace_bytes(B, T, D, K, C_given, dtype, flags);
         if (workspace == nullptr || workspace_bytes < need)
             return fail(T2FW_ERR_WORKSPACE, "workspace of %zu bytes needed, %zu given", need, workspace_bytes);
         if (!aligned16({workspace})) return fail(T2FW_ERR_MISALIGNED, "the workspace must be 16-byte aligned");
+        a.C = C;
+        a.NC = t2fw_lfw_num_ckpt(T, C);
+        if (C != C_given) {
+            // checkpoints at the interval the backward kernels take: the forward kernel once more, from s0
+            const size_t inner = par_ok(B, T, C, flags) ? par_scratch(B, T, C).total : 2 * row_flag_bytes(B);
+            const DenseScratch ds = dense_scratch(inner, B, T, C, es);
+            unsigned char *const ws = static_cast<unsigned char *>(workspace);
+            rc = lfw_forward_rows(x, f, q, k, f_key, s0, ws + ds.out, ws + ds.next, ws + ds.ckpt, B, T, heads, D, K, C,
+                                  dtype, flags & T2FW_FLAG_FP16_OPERANDS, workspace, inner, stream);
+            if (rc) return rc;
+            ckpt = ws + ds.ckpt;
+        }
         ChunkBwdArgs c{};
         c.g_out = g_out; c.g_state = g_state; c.x = x; c.f = f; c.q = q; c.k = k; c.f_key = f_key; c.ckpt = ckpt;
         c.d_x = d_x; c.d_f = d_f; c.d_q = d_q; c.d_k = d_k; c.d_f_key = d_f_key; c.d_s0 = d_s0;
@@ -413,6 +454,8 @@ static int lfw_backward_rows(const void *g_out, const void *g_state, const void 
         c.redo = (flags & T2FW_FLAG_NO_FIXUP) ? 0 : 1;
         return chunk_backward(c, dtype, op, st);
     }
+    a.C = C_given;
+    a.NC = t2fw_lfw_num_ckpt(T, C_given);
     return scan_backward(a, dtype, st);
 }
 
@@ -421,8 +464,7 @@ int t2fw_lfw_backward(const void *g_out, const void *g_state, const void *x, con
                       void *d_f, void *d_q, void *d_k, void *d_f_key, void *d_s0, int64_t B, int64_t T,
                       int64_t D, int64_t K, int32_t C, int32_t dtype, int32_t flags, void *workspace,
                       size_t workspace_bytes, void *stream) {
-    (void)s0;
-    return lfw_backward_rows(g_out, g_state, x, f, q, k, f_key, ckpt, d_x, d_f, d_q, d_k, d_f_key, d_s0, B, T, 1, D, K, C,
+    return lfw_backward_rows(g_out, g_state, x, f, q, k, f_key, s0, ckpt, d_x, d_f, d_q, d_k, d_f_key, d_s0, B, T, 1, D, K, C,
                              dtype, flags, workspace, workspace_bytes, stream);
 }
 
@@ -431,10 +473,9 @@ int t2fw_lfw_backward_heads(const void *g_out, const void *g_state, const void *
                             void *d_q, void *d_k, void *d_f_key, void *d_s0, int64_t B, int64_t T, int64_t H,
                             int64_t D, int64_t K, int32_t C, int32_t dtype, int32_t flags, void *workspace,
                             size_t workspace_bytes, void *stream) {
-    (void)s0;
     const int rc = check_heads(B, H);
     if (rc) return rc;
-    return lfw_backward_rows(g_out, g_state, x, f, q, k, f_key, ckpt, d_x, d_f, d_q, d_k, d_f_key, d_s0, B * H, T, H, D, K,
+    return lfw_backward_rows(g_out, g_state, x, f, q, k, f_key, s0, ckpt, d_x, d_f, d_q, d_k, d_f_key, d_s0, B * H, T, H, D, K,
                              C, dtype, flags, workspace, workspace_bytes, stream);
 }
 

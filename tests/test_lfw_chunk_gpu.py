@@ -39,7 +39,7 @@ class Flagged(tuple):
 def chunk_parallel_backward(C, flags):
     """the backward runs the chunk-parallel kernels unless a flag asks for the block-wise ones"""
     from t2fw_amd import _lib
-    return C in (32, 64) and not flags & (_lib.FLAG_BLOCKWISE | 2 | 1)
+    return C >= 32 and C % 32 == 0 and not flags & (_lib.FLAG_BLOCKWISE | 2 | 1)
 
 
 def run_abi(inputs, go, gs, C, flags=0, with_backward=True):
@@ -323,3 +323,29 @@ def test_random_lengths_and_intervals(seed):
     dtype = (torch.float16, torch.bfloat16)[int(torch.randint(0, 2, (1,), generator=g))]
     x, f, q, k, fk, s, go, gs = make_config_inputs(B, T, 64, 64, dtype, seed=seed, gate_mean=2.5, state_std=0.3)
     check_against_oracle((x, f, q, k, fk, s), go, gs, C, dtype, expect_flagged=0)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("C,T", [(96, 300), (128, 1024), (128, 130), (256, 700), (1024, 1000), (160, 161)])
+def test_checkpoint_intervals_that_are_other_multiples_of_32(C, T, dtype):
+    """The forward takes any multiple of 32; the backward kernels take 32 and 64 and get there by running the
+    forward kernel once more into checkpoints of their own (in the workspace), from s0."""
+    x, f, q, k, fk, s, go, gs = make_config_inputs(3, T, 64, 64, dtype, seed=C + T, gate_mean=2.5, state_std=0.3)
+    out, nxt, ckpt, grads = check_against_oracle((x, f, q, k, fk, s), go, gs, C, dtype, expect_flagged=0)
+    # the caller's checkpoints are at the interval it asked for
+    from t2fw_amd import _lib
+    assert ckpt.shape[1] == _lib.load().t2fw_lfw_num_ckpt(T, C)
+
+
+def test_sparse_checkpoints_with_rows_that_fall_back():
+    B, T, C = 4, 400, 128
+    x, f, q, k, fk, s, go, gs = make_config_inputs(B, T, 64, 64, torch.float16, seed=77, state_std=0.3)
+    f, fk = f.clone(), fk.clone()
+    f[1, 200, 5] = -0.5                 # the exact recurrence, forward and backward
+    fk[2, 64:96, 9] = 0.15              # declined by the chunk-parallel backward only
+    out, nxt, ckpt, grads, flagged = run_abi((x, f, q, k, fk, s), go, gs, C)
+    assert flagged == (1, 2) and flagged.exact == 1, (flagged, flagged.exact)
+    r_grads = c_oracle.lfw_backward(go, gs, x, f, q, k, fk, s)
+    for n, g, r in zip(NAMES, grads, r_grads):
+        assert_close(g, r, torch.float16, n, tol=TOL_CHUNK_GATE if n in ("d_f", "d_f_key") else TOL_CHUNK)
+        assert_close(g[1:2], r[1:2], torch.float16, n + "[row on the exact scan]")
