@@ -318,6 +318,8 @@ def main():
     ap.add_argument("--no-other-configs", action="store_true",
                     help="headline workload only (default: cfg2, cfg4, cfg5 and the delta rule are run briefly afterwards)")
     ap.add_argument("--force-scan", action="store_true", help="exact scan kernels only")
+    ap.add_argument("--dfw-bf16-operands", action="store_true",
+                    help="--workload dfw: the opt-in single-bf16 operand mode (flag 16)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU only (the path shards over the batch with no "
@@ -334,7 +336,7 @@ def main():
     elif args.workload in ("copy256", "copy64"):
         line = bench_copy(args)
     elif args.workload == "dfw":
-        line = bench_dfw(args, args.steps, args.warmup)
+        line = bench_dfw(args, args.steps, args.warmup, args.dfw_bf16_operands)
     elif args.workload == "cfg3_refgates":
         line = bench_lfw(args, "cfg3", args.steps, args.warmup, extras=False, gates="reference_test")
     else:
@@ -350,6 +352,7 @@ def main():
             others["cfg5"] = brief(bench_generation(args, 50, 10))
             torch.cuda.empty_cache()
             others["dfw"] = brief(bench_dfw(args, 20, 5))
+            others["dfw_bf16_operands"] = brief(bench_dfw(args, 20, 5, bf16_operands=True))
             line["other_configs"] = others
     print(json.dumps(line))
 
@@ -428,11 +431,12 @@ def bench_copy(args):
             "config": {"workload": "%s: torch copy_ of %d bytes, device to device" % (args.workload, n)}}
 
 
-def bench_dfw(args, steps, warmup):
+def bench_dfw(args, steps, warmup, bf16_operands=False):
     """Delta rule (t2fw/functional_dfw.py:29-65) forward + backward through the C ABI: B=96, T=1024,
     D=M=64, fp32, keys built as the reference's test builds them (tests/test_dfw.py:45-46).  A step
     is one forward and one backward call; the backward call is two launches (value side, then
-    query/key side).  Bytes: forward reads q,k,v,s0 and writes out,delta,final_state; backward
+    query/key side).  bf16_operands: the opt-in single-bf16 mode of the matrix-core kernels (flag 16)
+    instead of their default split operands.  Bytes: forward reads q,k,v,s0 and writes out,delta,final_state; backward
     reads g_out,g_state,q,k,delta,final_state and writes d_q,d_k,d_v,d_s0."""
     import torch
     from t2fw_amd import _lib
@@ -442,7 +446,7 @@ def bench_dfw(args, steps, warmup):
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     code = _lib.DTYPE_CODE[dtype]
-    flags = _lib.FLAG_FORCE_SCAN if args.force_scan else _lib.FLAG_AUTO
+    flags = _lib.FLAG_FORCE_SCAN if args.force_scan else (_lib.FLAG_BF16_OPERANDS if bf16_operands else _lib.FLAG_AUTO)
     stream = _lib.current_stream_handle(dev)
     per_set = (B * T * (3 * D + 2 * M) + B * T * (2 * D + 2 * M)) * es
     nsets = max(2, min(16, int(1.2e9 // per_set) + 1))
@@ -496,7 +500,9 @@ def bench_dfw(args, steps, warmup):
         "unit": "Mtokens/s", "n_gpus": 1, "steps": steps, "warmup": warmup,
         "ms_per_step": round(ms_per_step, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f32", "data": "synthetic",
-        "config": {"workload": "dfw: B=%d T=%d D=%d M=%d float32 fwd+bwd" % (B, T, D, M), "input_sets_rotated": nsets},
+        "config": {"workload": "dfw: B=%d T=%d D=%d M=%d float32 fwd+bwd" % (B, T, D, M), "input_sets_rotated": nsets,
+                   "operands": "exact per-step kernels" if args.force_scan else
+                               ("single bf16 (flag 16)" if bf16_operands else "bf16 head + remainder (default)")},
         "forward_avg_ms": round(fwd_ms, 5), "backward_avg_ms": round(bwd_ms, 5),
         "whole_step_algorithmic_GBs": round((fwd_bytes + bwd_bytes) / (ms_per_step * 1e-3) / 1e9, 1),
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",

@@ -91,6 +91,12 @@ extern "C" {
                                      instead of the chunk-parallel ones (every chunk of every row at once;
                                      gate products over half a chunk down to 2^-80)                  */
 
+#define T2FW_FLAG_BF16_OPERANDS 16 /* delta rule, matrix-core path: single bf16 operands (2^-9 per operand;
+                                     results within 1e-2 of max|ref| like the LFW kernels') instead of
+                                     operands split into bf16 head + remainder (fp32-level results, three
+                                     matrix-core products per product): for callers that train in reduced
+                                     precision anyway.  Off by default.                               */
+
 int t2fw_abi_version(void);
 const char *t2fw_last_error(void);
 

@@ -22,6 +22,7 @@ FLAG_FORCE_SCAN = 1
 FLAG_FP16_OPERANDS = 2
 FLAG_NO_FIXUP = 4
 FLAG_BLOCKWISE = 8
+FLAG_BF16_OPERANDS = 16
 
 _vp, _i64, _i32, _sz = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int32, ctypes.c_size_t
 

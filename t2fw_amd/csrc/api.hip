@@ -532,7 +532,7 @@ int t2fw_dfw_forward(const void *q, const void *k, const void *v, const void *s0
     a.q = q; a.k = k; a.v = v; a.s0 = s0; a.out = out; a.final_state = final_state; a.delta = delta;
     a.B = B; a.T = T; a.D = D; a.M = M;
     if (dfw_chunk_ok(D, M, dtype, flags) && T * CH_N < 0x7fffffffLL && aligned16({q, k, v, s0, out, final_state, delta}))
-        return dfw_chunk_forward(a, st);
+        return dfw_chunk_forward(a, (flags & T2FW_FLAG_BF16_OPERANDS) == 0, st);
     return dfw_forward(a, dtype, st);
 }
 
@@ -564,7 +564,7 @@ int t2fw_dfw_backward(const void *g_out, const void *g_state, const void *q, con
     a.B = B; a.T = T; a.D = D; a.M = M;
     if (dfw_chunk_ok(D, M, dtype, flags) && T * CH_N < 0x7fffffffLL &&
         aligned16({g_out, g_state, q, k, delta, final_state, d_q, d_k, d_v, d_s0}))
-        return dfw_chunk_backward(a, st);
+        return dfw_chunk_backward(a, (flags & T2FW_FLAG_BF16_OPERANDS) == 0, st);
     return dfw_backward(a, dtype, st);
 }
 

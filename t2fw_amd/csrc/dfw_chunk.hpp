@@ -13,7 +13,8 @@
 // Precision: the tensors are fp32 and the matrix cores take bf16, so every operand is split into a bf16
 // head and a bf16 remainder (x = hi + lo up to 2^-17 of x) and a product runs as three MFMAs
 // (hi*hi + hi*lo + lo*hi) with fp32 accumulation: results carry fp32-level rounding (measured against the
-// fp64 oracle: 1e-5 of max|ref|), not the 2^-9 of a single bf16 operand.
+// fp64 oracle: 3e-5 of max|ref|), not the 2^-9 of a single bf16 operand.  A caller that prefers speed asks for
+// the heads alone (T2FW_FLAG_BF16_OPERANDS; template parameter SP = false below).
 #pragma once
 
 #include "lfw_chunk.hpp"
@@ -34,95 +35,103 @@ constexpr int TM_TILE = DL * DTS * 2;         // bytes of one token-major tile (
 constexpr int CM_TILE = CH_N * DCS * 2;       // bytes of one channel-major tile
 constexpr int ST_TILE = 64 * 8;               // a 16 x 16 matrix as a packed MFMA operand: 8 bytes per lane
 
-// an operand of a 16-deep (Sp2) or 32-deep (Sp4) contraction as bf16 head and remainder
-struct Sp2 {
+// An operand of a 16-deep (Sp2) or 32-deep (Sp4) contraction as bf16 head and remainder.  SP = false (the
+// caller asked for T2FW_FLAG_BF16_OPERANDS): the head alone, one MFMA per product, 2^-9 per operand.
+template <bool SP> struct Sp2 {
     uint2 hi, lo;
 };
-struct Sp4 {
+template <bool SP> struct Sp4 {
     uint4 hi, lo;
 };
 
-__device__ __forceinline__ Sp2 split4(float a, float b, float c, float d) {
-    Sp2 o;
+template <bool SP> __device__ __forceinline__ Sp2<SP> split4(float a, float b, float c, float d) {
+    Sp2<SP> o;
     o.hi = packq<Bf16>(a, b, c, d);
-    o.lo = packq<Bf16>(a - Bf16::to_f32((u16)(o.hi.x & 0xffffu)), b - Bf16::to_f32((u16)(o.hi.x >> 16)),
-                       c - Bf16::to_f32((u16)(o.hi.y & 0xffffu)), d - Bf16::to_f32((u16)(o.hi.y >> 16)));
+    if constexpr (SP)
+        o.lo = packq<Bf16>(a - Bf16::to_f32((u16)(o.hi.x & 0xffffu)), b - Bf16::to_f32((u16)(o.hi.x >> 16)),
+                           c - Bf16::to_f32((u16)(o.hi.y & 0xffffu)), d - Bf16::to_f32((u16)(o.hi.y >> 16)));
+    else
+        o.lo = make_uint2(0u, 0u);
     return o;
 }
-__device__ __forceinline__ Sp2 split4(const floatx4 &v) { return split4(v[0], v[1], v[2], v[3]); }
-__device__ __forceinline__ Sp4 cat(const Sp2 &a, const Sp2 &b) {
-    Sp4 o;
+template <bool SP> __device__ __forceinline__ Sp2<SP> split4(const floatx4 &v) { return split4<SP>(v[0], v[1], v[2], v[3]); }
+template <bool SP> __device__ __forceinline__ Sp4<SP> cat(const Sp2<SP> &a, const Sp2<SP> &b) {
+    Sp4<SP> o;
     o.hi = bwd::cat(a.hi, b.hi);
     o.lo = bwd::cat(a.lo, b.lo);
     return o;
 }
 
 // c + a b with split operands (the smaller terms first); chains of one MFMA form only
-__device__ __forceinline__ floatx4 mma16(const Sp2 &a, const Sp2 &b, floatx4 c) {
-    c = Bf16::mfma16(a.lo, b.hi, c);
-    c = Bf16::mfma16(a.hi, b.lo, c);
+template <bool SP> __device__ __forceinline__ floatx4 mma16(const Sp2<SP> &a, const Sp2<SP> &b, floatx4 c) {
+    if constexpr (SP) {
+        c = Bf16::mfma16(a.lo, b.hi, c);
+        c = Bf16::mfma16(a.hi, b.lo, c);
+    }
     return Bf16::mfma16(a.hi, b.hi, c);
 }
-__device__ __forceinline__ floatx4 mma32(const Sp4 &a, const Sp4 &b, floatx4 c) {
-    c = Bf16::mfma32(a.lo, b.hi, c);
-    c = Bf16::mfma32(a.hi, b.lo, c);
+template <bool SP> __device__ __forceinline__ floatx4 mma32(const Sp4<SP> &a, const Sp4<SP> &b, floatx4 c) {
+    if constexpr (SP) {
+        c = Bf16::mfma32(a.lo, b.hi, c);
+        c = Bf16::mfma32(a.hi, b.lo, c);
+    }
     return Bf16::mfma32(a.hi, b.hi, c);
 }
 
 // ---- tiles in LDS: a head tile followed by a remainder tile of the same shape ----------------------
 // token-major [16][DTS]: channel c of a token sits at tm_pos(c), so that the sixteen channels a matrix lane
 // (r, g) pairs with its accumulators (16 j + 4 g + e) are contiguous at 16 g
-struct TmTile {
+template <bool SP> struct TmTile {
     const u16 *hi, *lo;
     __device__ __forceinline__ TmTile(const unsigned char *base) : hi(reinterpret_cast<const u16 *>(base)), lo(reinterpret_cast<const u16 *>(base + TM_TILE)) {}
     // A / B operand "row `row`, the lane's accumulator channels", halves h = 0, 1 of the 64-deep contraction
-    __device__ __forceinline__ Sp4 acc_order(int row, int g, int h) const {
-        Sp4 o;
+    __device__ __forceinline__ Sp4<SP> acc_order(int row, int g, int h) const {
+        Sp4<SP> o;
         o.hi = ld4(hi + row * DTS + 16 * g + 8 * h);
-        o.lo = ld4(lo + row * DTS + 16 * g + 8 * h);
+        o.lo = SP ? ld4(lo + row * DTS + 16 * g + 8 * h) : make_uint4(0u, 0u, 0u, 0u);
         return o;
     }
     // A / B operand "row `row`" for products of two token-major tiles (any fixed channel order)
-    __device__ __forceinline__ Sp4 any_order(int row, int g, int h) const {
-        Sp4 o;
+    __device__ __forceinline__ Sp4<SP> any_order(int row, int g, int h) const {
+        Sp4<SP> o;
         o.hi = ld4(hi + row * DTS + 8 * g + 32 * h);
-        o.lo = ld4(lo + row * DTS + 8 * g + 32 * h);
+        o.lo = SP ? ld4(lo + row * DTS + 8 * g + 32 * h) : make_uint4(0u, 0u, 0u, 0u);
         return o;
     }
 };
 // channel-major [64][DCS]: A operand "channel `ch`, tokens 4 g .. 4 g + 3"
-struct CmTile {
+template <bool SP> struct CmTile {
     const u16 *hi, *lo;
     __device__ __forceinline__ CmTile(const unsigned char *base) : hi(reinterpret_cast<const u16 *>(base)), lo(reinterpret_cast<const u16 *>(base + CM_TILE)) {}
-    __device__ __forceinline__ Sp2 tokens(int ch, int g) const {
-        Sp2 o;
+    __device__ __forceinline__ Sp2<SP> tokens(int ch, int g) const {
+        Sp2<SP> o;
         o.hi = ld2(hi + ch * DCS + 4 * g);
-        o.lo = ld2(lo + ch * DCS + 4 * g);
+        o.lo = SP ? ld2(lo + ch * DCS + 4 * g) : make_uint2(0u, 0u);
         return o;
     }
 };
 // Four result tiles [channel 16 j + 4 g + e][token r] (j = 0 .. 3) of a lane are the sixteen channels that
 // tm_pos puts at 16 g of token row r: stored as head and remainder of a token-major tile
-__device__ __forceinline__ void store_tm_from_acc(unsigned char *tile, int r, int g, const floatx4 (&v)[4]) {
+template <bool SP> __device__ __forceinline__ void store_tm_from_acc(unsigned char *tile, int r, int g, const floatx4 (&v)[4]) {
     u16 *hi = reinterpret_cast<u16 *>(tile), *lo = reinterpret_cast<u16 *>(tile + TM_TILE);
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-        const Sp2 s = split4(v[j]);
+        const Sp2<SP> s = split4<SP>(v[j]);
         *reinterpret_cast<uint2 *>(hi + r * DTS + 16 * g + 4 * j) = s.hi;
-        *reinterpret_cast<uint2 *>(lo + r * DTS + 16 * g + 4 * j) = s.lo;
+        if constexpr (SP) *reinterpret_cast<uint2 *>(lo + r * DTS + 16 * g + 4 * j) = s.lo;
     }
 }
 
 // a 16 x 16 matrix in the accumulator layout (lane (r, g): rows 4 g + e of column r), packed: read back by
 // the same lane it is at once the B operand "X" and the A operand "X transposed" of a 16-deep product
-__device__ __forceinline__ void st_store(unsigned char *tile, int lane, const Sp2 &v) {
+template <bool SP> __device__ __forceinline__ void st_store(unsigned char *tile, int lane, const Sp2<SP> &v) {
     reinterpret_cast<uint2 *>(tile)[lane] = v.hi;
-    reinterpret_cast<uint2 *>(tile + ST_TILE)[lane] = v.lo;
+    if constexpr (SP) reinterpret_cast<uint2 *>(tile + ST_TILE)[lane] = v.lo;
 }
-__device__ __forceinline__ Sp2 st_load(const unsigned char *tile, int lane) {
-    Sp2 o;
+template <bool SP> __device__ __forceinline__ Sp2<SP> st_load(const unsigned char *tile, int lane) {
+    Sp2<SP> o;
     o.hi = reinterpret_cast<const uint2 *>(tile)[lane];
-    o.lo = reinterpret_cast<const uint2 *>(tile + ST_TILE)[lane];
+    o.lo = SP ? reinterpret_cast<const uint2 *>(tile + ST_TILE)[lane] : make_uint2(0u, 0u);
     return o;
 }
 
@@ -133,8 +142,8 @@ __device__ __forceinline__ Sp2 st_load(const unsigned char *tile, int lane) {
 // data movement; squaring X and X^T side by side gives the powers 2, 4, 8 of A and of A^T, then
 //   P1 = (I + A^4)(I + A^8) = I + A^4 + A^8 + A^12,   P2^T = ((I - A)(I + A^2))^T = I - A^T + (A^2)^T - (A^3)^T,
 //   Tm = P2 P1:   acc(Tm^T) = mfma(acc(P1), acc(P2^T)),   acc(Tm) = mfma(acc(P2^T), acc(P1)).
-struct BlockInverse {
-    Sp2 p1, p2t;
+template <bool SP> struct BlockInverse {
+    Sp2<SP> p1, p2t;
     __device__ __forceinline__ BlockInverse(const floatx4 &kk, int r, int g) {
         const floatx4 zero = {0.f, 0.f, 0.f, 0.f};
         floatx4 a, at, eye;
@@ -145,16 +154,16 @@ struct BlockInverse {
             at[e] = row < r ? kk[e] : 0.f;
             eye[e] = row == r ? 1.f : 0.f;
         }
-        const Sp2 x1 = split4(a), x1t = split4(at);
+        const Sp2<SP> x1 = split4<SP>(a), x1t = split4<SP>(at);
         const floatx4 a2 = mma16(x1t, x1, zero), a2t = mma16(x1, x1t, zero);
-        const Sp2 x2 = split4(a2), x2t = split4(a2t);
+        const Sp2<SP> x2 = split4<SP>(a2), x2t = split4<SP>(a2t);
         const floatx4 a3t = mma16(x1, x2t, zero);                       // (A^3)^T = A^T (A^2)^T
         const floatx4 a4 = mma16(x2t, x2, zero), a4t = mma16(x2, x2t, zero);
-        const Sp2 x4 = split4(a4), x4t = split4(a4t);
+        const Sp2<SP> x4 = split4<SP>(a4), x4t = split4<SP>(a4t);
         const floatx4 a8 = mma16(x4t, x4, zero);
-        const floatx4 a12 = mma16(x4t, split4(a8), zero);               // A^12 = A^4 A^8
-        p1 = split4(eye + a4 + a8 + a12);
-        p2t = split4(eye - at + a2t - a3t);
+        const floatx4 a12 = mma16(x4t, split4<SP>(a8), zero);               // A^12 = A^4 A^8
+        p1 = split4<SP>(eye + a4 + a8 + a12);
+        p2t = split4<SP>(eye - at + a2t - a3t);
     }
     __device__ __forceinline__ floatx4 acc_tm_transposed() const { return mma16(p1, p2t, floatx4{0.f, 0.f, 0.f, 0.f}); }
     __device__ __forceinline__ floatx4 acc_tm() const { return mma16(p2t, p1, floatx4{0.f, 0.f, 0.f, 0.f}); }
@@ -176,15 +185,15 @@ __device__ __forceinline__ Raw16 load_tm(const float *row0, int tok0, int T, int
     for (int a = 0; a < 4; ++a) r.v[a] = p[a];
     return r;
 }
-__device__ __forceinline__ void store_tm(unsigned char *tile, int lane, const Raw16 &r, int tok0, int T, float sign = 1.f) {
+template <bool SP> __device__ __forceinline__ void store_tm(unsigned char *tile, int lane, const Raw16 &r, int tok0, int T, float sign = 1.f) {
     u16 *hi = reinterpret_cast<u16 *>(tile), *lo = reinterpret_cast<u16 *>(tile + TM_TILE);
     const int o = (lane >> 2) * DTS + 4 * (lane & 3);
     const float keep = tok0 + (lane >> 2) < T ? sign : 0.f;
 #pragma unroll
     for (int a = 0; a < 4; ++a) {          // channels 16 q + 4 a + e sit at 16 a + 4 q + e
-        const Sp2 s = split4(r.v[a].x * keep, r.v[a].y * keep, r.v[a].z * keep, r.v[a].w * keep);
+        const Sp2<SP> s = split4<SP>(r.v[a].x * keep, r.v[a].y * keep, r.v[a].z * keep, r.v[a].w * keep);
         *reinterpret_cast<uint2 *>(hi + o + 16 * a) = s.hi;
-        *reinterpret_cast<uint2 *>(lo + o + 16 * a) = s.lo;
+        if constexpr (SP) *reinterpret_cast<uint2 *>(lo + o + 16 * a) = s.lo;
     }
 }
 __device__ __forceinline__ Raw16 load_cm(const float *row0, int tok0, int T, int lane) {
@@ -196,15 +205,15 @@ __device__ __forceinline__ Raw16 load_cm(const float *row0, int tok0, int T, int
     for (int a = 0; a < 4; ++a) r.v[a] = make_float4(f[4 * a], f[4 * a + 1], f[4 * a + 2], f[4 * a + 3]);
     return r;
 }
-__device__ __forceinline__ void store_cm(unsigned char *tile, int lane, const Raw16 &r, int tok0, int T, float sign = 1.f) {
+template <bool SP> __device__ __forceinline__ void store_cm(unsigned char *tile, int lane, const Raw16 &r, int tok0, int T, float sign = 1.f) {
     u16 *hi = reinterpret_cast<u16 *>(tile), *lo = reinterpret_cast<u16 *>(tile + CM_TILE);
 #pragma unroll
     for (int a = 0; a < 4; ++a) {
         const int t = tok0 + 4 * a;
-        const Sp2 s = split4(t < T ? r.v[a].x * sign : 0.f, t + 1 < T ? r.v[a].y * sign : 0.f, t + 2 < T ? r.v[a].z * sign : 0.f,
-                             t + 3 < T ? r.v[a].w * sign : 0.f);
+        const Sp2<SP> s = split4<SP>(t < T ? r.v[a].x * sign : 0.f, t + 1 < T ? r.v[a].y * sign : 0.f, t + 2 < T ? r.v[a].z * sign : 0.f,
+                                     t + 3 < T ? r.v[a].w * sign : 0.f);
         *reinterpret_cast<uint2 *>(hi + lane * DCS + 4 * a) = s.hi;
-        *reinterpret_cast<uint2 *>(lo + lane * DCS + 4 * a) = s.lo;
+        if constexpr (SP) *reinterpret_cast<uint2 *>(lo + lane * DCS + 4 * a) = s.lo;
     }
 }
 
@@ -231,7 +240,7 @@ struct PrepJob {
     int off;                // byte offset of the tile inside a block's raw tiles
     float sign;             // the tile holds sign * src
 };
-template <typename RING, int NBLK, bool CHANNEL_MAJOR, int NJOBS, typename TOK0>
+template <typename RING, int NBLK, bool CHANNEL_MAJOR, int NJOBS, bool SP, typename TOK0>
 __device__ __forceinline__ void prep_wave_jobs(unsigned char *smem, const PrepJob (&jobs)[NJOBS], int T, int nstages, int lane,
                                                TOK0 tok0_of) {
     Raw16 set_a[NJOBS][NBLK], set_b[NJOBS][NBLK];
@@ -254,9 +263,9 @@ __device__ __forceinline__ void prep_wave_jobs(unsigned char *smem, const PrepJo
                     unsigned char *tile = RING::raw(smem, tick, bb) + jobs[a].off;
                     const int tok0 = tok0_of(tick, bb);
                     if (CHANNEL_MAJOR)
-                        store_cm(tile, lane, cur[a][bb], tok0, T, jobs[a].sign);
+                        store_cm<SP>(tile, lane, cur[a][bb], tok0, T, jobs[a].sign);
                     else
-                        store_tm(tile, lane, cur[a][bb], tok0, T, jobs[a].sign);
+                        store_tm<SP>(tile, lane, cur[a][bb], tok0, T, jobs[a].sign);
                 }
         }
         __syncthreads();

@@ -35,38 +35,38 @@ __device__ __forceinline__ int reverse_tok0(int nblocks, int nblk_per_stage, int
     return (nblocks - 1 - (stage * nblk_per_stage + bb)) * DL;
 }
 
-__device__ __forceinline__ void vs_structure_wave(unsigned char *smem, int nstages, int bb, int lane) {
+template <bool SP> __device__ __forceinline__ void vs_structure_wave(unsigned char *smem, int nstages, int bb, int lane) {
     const int r = lane & 15, g = lane >> 4;
     const floatx4 zero = {0.f, 0.f, 0.f, 0.f};
     for (int tick = 0; tick < nstages + 2; ++tick) {
         const int stage = tick - 1;
         if (stage >= 0 && stage < nstages) {
             const unsigned char *raw = VsRing::raw(smem, stage, bb);
-            const TmTile KT(raw + VS_KT), QT(raw + VS_QT);
-            const CmTile KC(raw + VS_KC);
-            const Sp4 k0 = KT.any_order(r, g, 0), k1 = KT.any_order(r, g, 1);
-            const Sp4 q0 = QT.any_order(r, g, 0), q1 = QT.any_order(r, g, 1);
+            const TmTile<SP> KT(raw + VS_KT), QT(raw + VS_QT);
+            const CmTile<SP> KC(raw + VS_KC);
+            const Sp4<SP> k0 = KT.any_order(r, g, 0), k1 = KT.any_order(r, g, 1);
+            const Sp4<SP> q0 = QT.any_order(r, g, 0), q1 = QT.any_order(r, g, 1);
             const floatx4 kk = mma32(k1, k1, mma32(k0, k0, zero));
             const floatx4 qk = mma32(q1, k1, mma32(q0, k0, zero));      // [t = 4g+e][s = r] = q_t . k_s
             floatx4 bq;
 #pragma unroll
             for (int e = 0; e < 4; ++e) bq[e] = r < 4 * g + e ? qk[e] : 0.f;       // Bq[t][s] for s < t
-            const BlockInverse inv(kk, r, g);
-            const Sp2 tm = split4(inv.acc_tm());
+            const BlockInverse<SP> inv(kk, r, g);
+            const Sp2<SP> tm = split4<SP>(inv.acc_tm());
             unsigned char *st = VsRing::st(smem, stage, bb);
-            st_store(st + VS_TM, lane, tm);
-            st_store(st + VS_BQ, lane, split4(bq));
+            st_store<SP>(st + VS_TM, lane, tm);
+            st_store<SP>(st + VS_BQ, lane, split4<SP>(bq));
             // K''^T tile j: [m = 16 j + 4 g + e][t = r] = sum_s K[s][m] Tm[s][t]   (K'' = Tm^T K)
             floatx4 kpp[4];
 #pragma unroll
             for (int j = 0; j < 4; ++j) kpp[j] = mma16(KC.tokens(16 * j + r, g), tm, zero);
-            store_tm_from_acc(st + VS_KPP, r, g, kpp);
+            store_tm_from_acc<SP>(st + VS_KPP, r, g, kpp);
         }
         __syncthreads();
     }
 }
 
-__device__ __forceinline__ void vs_slab_wave(const DfwBwdArgs &p, unsigned char *smem, int64_t b, int d0, int nstages, int lane) {
+template <bool SP> __device__ __forceinline__ void vs_slab_wave(const DfwBwdArgs &p, unsigned char *smem, int64_t b, int d0, int nstages, int lane) {
     const int r = lane & 15, g = lane >> 4, d = d0 + r, T = (int)p.T, nblocks = nstages * DNB;
     const floatx4 zero = {0.f, 0.f, 0.f, 0.f};
     const float *const go = reinterpret_cast<const float *>(p.g_out) + b * p.T * CH_N;
@@ -100,13 +100,13 @@ __device__ __forceinline__ void vs_slab_wave(const DfwBwdArgs &p, unsigned char 
                 for (int e = 0; e < 4; ++e) gcur[bb][e] = tok0 + 4 * g + e < T ? gcur[bb][e] : 0.f;
                 const unsigned char *raw = VsRing::raw(smem, stage, bb);
                 const unsigned char *st = VsRing::st(smem, stage, bb);
-                const TmTile KPP(st + VS_KPP);
-                const CmTile KC(raw + VS_KC), QC(raw + VS_QC);
+                const TmTile<SP> KPP(st + VS_KPP);
+                const CmTile<SP> KC(raw + VS_KC), QC(raw + VS_QC);
                 // dU[tok 4g+e][d] = Tm^T (Bq^T g) + K'' G_end^T: only the second term waits for the adjoint
-                const Sp2 gs = split4(gcur[bb]);
-                const floatx4 bg = mma16(st_load(st + VS_BQ, lane), gs, zero);
-                const floatx4 tbg = mma16(st_load(st + VS_TM, lane), split4(bg), zero);
-                const Sp4 gb0 = cat(split4(G[0]), split4(G[1])), gb1 = cat(split4(G[2]), split4(G[3]));
+                const Sp2<SP> gs = split4<SP>(gcur[bb]);
+                const floatx4 bg = mma16(st_load<SP>(st + VS_BQ, lane), gs, zero);
+                const floatx4 tbg = mma16(st_load<SP>(st + VS_TM, lane), split4<SP>(bg), zero);
+                const Sp4<SP> gb0 = cat(split4<SP>(G[0]), split4<SP>(G[1])), gb1 = cat(split4<SP>(G[2]), split4<SP>(G[3]));
                 const floatx4 kg = mma32(KPP.acc_order(r, g, 1), gb1, mma32(KPP.acc_order(r, g, 0), gb0, zero));
                 const floatx4 du = tbg + kg;
                 float *const vb = d_v + (size_t)tok0 * CH_N;        // wave-uniform
@@ -119,7 +119,7 @@ __device__ __forceinline__ void vs_slab_wave(const DfwBwdArgs &p, unsigned char 
                         if (tok0 + 4 * g + e < T) vb[lane_off + e * CH_N] = du[e];
                 }
                 // G += g^T Q - dU^T K
-                const Sp2 ndu = split4(-du);
+                const Sp2<SP> ndu = split4<SP>(-du);
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
                     G[j] = mma16(QC.tokens(16 * j + r, g), gs, G[j]);
@@ -143,7 +143,7 @@ __device__ __forceinline__ void vs_slab_wave(const DfwBwdArgs &p, unsigned char 
 
 // blockIdx = half * rows_padded + row (rows_padded a multiple of 8: both halves of a row on one XCD).  Waves 0, 1:
 // slab waves, alone on SIMDs 0 and 1; waves 2, 3: matrix waves; waves 6, 7: prep waves; waves 4, 5 leave at once.
-__global__ __launch_bounds__(BW_THREADS) void dfw_chunk_bwd_value_kernel(DfwBwdArgs p, int rows_padded) {
+template <bool SP> __global__ __launch_bounds__(BW_THREADS) void dfw_chunk_bwd_value_kernel(DfwBwdArgs p, int rows_padded) {
     extern __shared__ __align__(16) unsigned char smem[];
     const int half = (int)blockIdx.x >= rows_padded ? 1 : 0;
     const int64_t b = (int)blockIdx.x - half * rows_padded;
@@ -155,15 +155,15 @@ __global__ __launch_bounds__(BW_THREADS) void dfw_chunk_bwd_value_kernel(DfwBwdA
     auto tok0_of = [=](int stage, int bb) { return reverse_tok0(nblocks, DNB, stage, bb); };
     static_assert(DNB == 2, "one matrix wave per block of a stage");
     if (wave < 2) {
-        vs_slab_wave(p, smem, b, 32 * half + 16 * wave, nstages, lane);
+        vs_slab_wave<SP>(p, smem, b, 32 * half + 16 * wave, nstages, lane);
     } else if (wave < 4) {
-        vs_structure_wave(smem, nstages, wave - 2, lane);
+        vs_structure_wave<SP>(smem, nstages, wave - 2, lane);
     } else if (wave == 6) {
         const PrepJob jobs[2] = {{k, VS_KT, 1.f}, {q, VS_QT, 1.f}};
-        prep_wave_jobs<VsRing, DNB, false, 2>(smem, jobs, T, nstages, lane, tok0_of);
+        prep_wave_jobs<VsRing, DNB, false, 2, SP>(smem, jobs, T, nstages, lane, tok0_of);
     } else if (wave == 7) {
         const PrepJob jobs[2] = {{k, VS_KC, 1.f}, {q, VS_QC, 1.f}};
-        prep_wave_jobs<VsRing, DNB, true, 2>(smem, jobs, T, nstages, lane, tok0_of);
+        prep_wave_jobs<VsRing, DNB, true, 2, SP>(smem, jobs, T, nstages, lane, tok0_of);
     }
 }
 
@@ -176,17 +176,17 @@ constexpr int KS_X1 = 0, KS_X1T = KS_X1 + 2 * ST_TILE, KS_X2S = KS_X1T + 2 * ST_
 using KsRing = Ring<KS_RAW_BLOCK, KS_ST_BLOCK, 1>;
 static_assert(KsRing::SMEM <= 160 * 1024, "key-side tiles exceed the LDS of one CU");
 
-__device__ __forceinline__ void ks_structure_wave(unsigned char *smem, int nstages, int lane) {
+template <bool SP> __device__ __forceinline__ void ks_structure_wave(unsigned char *smem, int nstages, int lane) {
     const int r = lane & 15, g = lane >> 4;
     const floatx4 zero = {0.f, 0.f, 0.f, 0.f};
     for (int tick = 0; tick < nstages + 2; ++tick) {
         const int stage = tick - 1;
         if (stage >= 0 && stage < nstages) {
             const unsigned char *raw = KsRing::raw(smem, stage, 0);
-            const TmTile DT(raw + KS_DT), GT(raw + KS_GT), NUT(raw + KS_NUT);
-            const Sp4 d0 = DT.any_order(r, g, 0), d1 = DT.any_order(r, g, 1);
-            const Sp4 g0 = GT.any_order(r, g, 0), g1 = GT.any_order(r, g, 1);
-            const Sp4 u0 = NUT.any_order(r, g, 0), u1 = NUT.any_order(r, g, 1);
+            const TmTile<SP> DT(raw + KS_DT), GT(raw + KS_GT), NUT(raw + KS_NUT);
+            const Sp4<SP> d0 = DT.any_order(r, g, 0), d1 = DT.any_order(r, g, 1);
+            const Sp4<SP> g0 = GT.any_order(r, g, 0), g1 = GT.any_order(r, g, 1);
+            const Sp4<SP> u0 = NUT.any_order(r, g, 0), u1 = NUT.any_order(r, g, 1);
             const floatx4 z = mma32(g1, d1, mma32(g0, d0, zero));       // [t = 4g+e][s = r] =  g_t . delta_s
             const floatx4 zt = mma32(d1, g1, mma32(d0, g0, zero));      // [s = 4g+e][t = r] =  delta_s . g_t
             const floatx4 y = mma32(u1, d1, mma32(u0, d0, zero));       // [t = 4g+e][s = r] = -dU_t . delta_s
@@ -200,15 +200,15 @@ __device__ __forceinline__ void ks_structure_wave(unsigned char *smem, int nstag
                 x2s[e] = r < row ? y[e] : (row < r ? yt[e] : 0.f);      // X2 + X2^T
             }
             unsigned char *st = KsRing::st(smem, stage, 0);
-            st_store(st + KS_X1, lane, split4(x1));
-            st_store(st + KS_X1T, lane, split4(x1t));
-            st_store(st + KS_X2S, lane, split4(x2s));
+            st_store<SP>(st + KS_X1, lane, split4<SP>(x1));
+            st_store<SP>(st + KS_X1T, lane, split4<SP>(x1t));
+            st_store<SP>(st + KS_X2S, lane, split4<SP>(x2s));
         }
         __syncthreads();
     }
 }
 
-__device__ __forceinline__ void ks_slab_wave(const DfwBwdArgs &p, unsigned char *smem, int64_t b, int m0, int nstages, int lane) {
+template <bool SP> __device__ __forceinline__ void ks_slab_wave(const DfwBwdArgs &p, unsigned char *smem, int64_t b, int m0, int nstages, int lane) {
     const int r = lane & 15, g = lane >> 4, m = m0 + r, T = (int)p.T, nblocks = nstages;
     const floatx4 zero = {0.f, 0.f, 0.f, 0.f};
     float *const d_q = reinterpret_cast<float *>(p.d_q) + b * p.T * CH_N;
@@ -233,23 +233,23 @@ __device__ __forceinline__ void ks_slab_wave(const DfwBwdArgs &p, unsigned char 
             const int tok0 = reverse_tok0(nblocks, 1, stage, 0);
             const unsigned char *raw = KsRing::raw(smem, stage, 0);
             const unsigned char *st = KsRing::st(smem, stage, 0);
-            const TmTile DT(raw + KS_DT), GT(raw + KS_GT), NUT(raw + KS_NUT);
-            const CmTile NDC(raw + KS_NDC), GC(raw + KS_GC), NUC(raw + KS_NUC), KC(raw + KS_KC), QC(raw + KS_QC);
-            const Sp2 kb = KC.tokens(m, g), qb = QC.tokens(m, g);          // K[t = 4g+e][m], Q[t][m]
+            const TmTile<SP> DT(raw + KS_DT), GT(raw + KS_GT), NUT(raw + KS_NUT);
+            const CmTile<SP> NDC(raw + KS_NDC), GC(raw + KS_GC), NUC(raw + KS_NUC), KC(raw + KS_KC), QC(raw + KS_QC);
+            const Sp2<SP> kb = KC.tokens(m, g), qb = QC.tokens(m, g);          // K[t = 4g+e][m], Q[t][m]
             // the adjoint after the block, before it takes the block in
-            const Sp4 gb0 = cat(split4(G[0]), split4(G[1])), gb1 = cat(split4(G[2]), split4(G[3]));
+            const Sp4<SP> gb0 = cat(split4<SP>(G[0]), split4<SP>(G[1])), gb1 = cat(split4<SP>(G[2]), split4<SP>(G[3]));
             // S0 = S_end - Delta^T K
 #pragma unroll
             for (int j = 0; j < 4; ++j) S[j] = mma16(NDC.tokens(16 * j + r, g), kb, S[j]);
-            const Sp4 sb0 = cat(split4(S[0]), split4(S[1])), sb1 = cat(split4(S[2]), split4(S[3]));
+            const Sp4<SP> sb0 = cat(split4<SP>(S[0]), split4<SP>(S[1])), sb1 = cat(split4<SP>(S[2]), split4<SP>(S[3]));
             // d_query[t][m] = g S0 + X1 K
             const floatx4 dq = mma32(GT.acc_order(r, g, 1), sb1, mma32(GT.acc_order(r, g, 0), sb0, zero)) +
-                               mma16(st_load(st + KS_X1T, lane), kb, zero);
+                               mma16(st_load<SP>(st + KS_X1T, lane), kb, zero);
             // d_key[s][m] = Delta G_end - dU S0 + X1^T Q + (X2 + X2^T) K
             const floatx4 dk = mma32(NUT.acc_order(r, g, 1), sb1,
                                      mma32(NUT.acc_order(r, g, 0), sb0,
                                            mma32(DT.acc_order(r, g, 1), gb1, mma32(DT.acc_order(r, g, 0), gb0, zero)))) +
-                               mma16(st_load(st + KS_X2S, lane), kb, mma16(st_load(st + KS_X1, lane), qb, zero));
+                               mma16(st_load<SP>(st + KS_X2S, lane), kb, mma16(st_load<SP>(st + KS_X1, lane), qb, zero));
             float *const qo = d_q + (size_t)tok0 * CH_N, *const ko = d_k + (size_t)tok0 * CH_N;      // wave-uniform
             if (tok0 + DL <= T) {
 #pragma unroll
@@ -278,7 +278,7 @@ __device__ __forceinline__ void ks_slab_wave(const DfwBwdArgs &p, unsigned char 
 
 // Waves 0, 1: slab waves (16 key channels each), alone on SIMDs 0 and 1; wave 2: matrix wave; waves 3, 6, 7: prep
 // waves; waves 4, 5 leave at once.
-__global__ __launch_bounds__(BW_THREADS) void dfw_chunk_bwd_key_kernel(DfwBwdArgs p, int rows_padded) {
+template <bool SP> __global__ __launch_bounds__(BW_THREADS) void dfw_chunk_bwd_key_kernel(DfwBwdArgs p, int rows_padded) {
     extern __shared__ __align__(16) unsigned char smem[];
     const int half = (int)blockIdx.x >= rows_padded ? 1 : 0;
     const int64_t b = (int)blockIdx.x - half * rows_padded;
@@ -293,29 +293,26 @@ __global__ __launch_bounds__(BW_THREADS) void dfw_chunk_bwd_key_kernel(DfwBwdArg
     const float *const dv = reinterpret_cast<const float *>(p.d_v) + row;
     auto tok0_of = [=](int stage, int bb) { return reverse_tok0(nstages, 1, stage, bb); };
     if (wave < 2) {
-        ks_slab_wave(p, smem, b, 32 * half + 16 * wave, nstages, lane);
+        ks_slab_wave<SP>(p, smem, b, 32 * half + 16 * wave, nstages, lane);
     } else if (wave == 2) {
-        ks_structure_wave(smem, nstages, lane);
+        ks_structure_wave<SP>(smem, nstages, lane);
     } else if (wave == 3) {
         const PrepJob jobs[3] = {{dl, KS_DT, 1.f}, {go, KS_GT, 1.f}, {dv, KS_NUT, -1.f}};
-        prep_wave_jobs<KsRing, 1, false, 3>(smem, jobs, T, nstages, lane, tok0_of);
+        prep_wave_jobs<KsRing, 1, false, 3, SP>(smem, jobs, T, nstages, lane, tok0_of);
     } else if (wave == 6) {
         const PrepJob jobs[3] = {{dl, KS_NDC, -1.f}, {go, KS_GC, 1.f}, {dv, KS_NUC, -1.f}};
-        prep_wave_jobs<KsRing, 1, true, 3>(smem, jobs, T, nstages, lane, tok0_of);
+        prep_wave_jobs<KsRing, 1, true, 3, SP>(smem, jobs, T, nstages, lane, tok0_of);
     } else if (wave == 7) {
         const PrepJob jobs[2] = {{k, KS_KC, 1.f}, {q, KS_QC, 1.f}};
-        prep_wave_jobs<KsRing, 1, true, 2>(smem, jobs, T, nstages, lane, tok0_of);
+        prep_wave_jobs<KsRing, 1, true, 2, SP>(smem, jobs, T, nstages, lane, tok0_of);
     }
 }
 
 }  // namespace
 
-int dfw_chunk_backward(const DfwBwdArgs &a, hipStream_t stream) {
-    if (a.D != CH_N || a.M != CH_N) return fail(T2FW_ERR_UNSUPPORTED, "the block-wise delta-rule kernels take D = M = 64");
-    if (a.T * CH_N >= 0x7fffffffLL || a.B > 0x1fffffffLL)
-        return fail(T2FW_ERR_UNSUPPORTED, "B=%lld T=%lld is too large for the block-wise delta-rule kernels", (long long)a.B, (long long)a.T);
-    auto value_side = dfw_chunk_bwd_value_kernel;
-    auto key_side = dfw_chunk_bwd_key_kernel;
+template <bool SP> static int launch_backward(const DfwBwdArgs &a, hipStream_t stream) {
+    auto value_side = dfw_chunk_bwd_value_kernel<SP>;
+    auto key_side = dfw_chunk_bwd_key_kernel<SP>;
     int rc = enable_lds(reinterpret_cast<const void *>(value_side), VsRing::SMEM, "hipFuncSetAttribute(delta-rule backward kernel, value side)");
     if (rc) return rc;
     if ((rc = enable_lds(reinterpret_cast<const void *>(key_side), KsRing::SMEM, "hipFuncSetAttribute(delta-rule backward kernel, key side)"))) return rc;
@@ -324,6 +321,13 @@ int dfw_chunk_backward(const DfwBwdArgs &a, hipStream_t stream) {
     if ((rc = check_hip(hipGetLastError(), "dfw_chunk_bwd_value_kernel launch"))) return rc;
     hipLaunchKernelGGL(key_side, dim3(2u * (unsigned)rows_padded), dim3(BW_THREADS), KsRing::SMEM, stream, a, rows_padded);
     return check_hip(hipGetLastError(), "dfw_chunk_bwd_key_kernel launch");
+}
+
+int dfw_chunk_backward(const DfwBwdArgs &a, bool split_operands, hipStream_t stream) {
+    if (a.D != CH_N || a.M != CH_N) return fail(T2FW_ERR_UNSUPPORTED, "the block-wise delta-rule kernels take D = M = 64");
+    if (a.T * CH_N >= 0x7fffffffLL || a.B > 0x1fffffffLL)
+        return fail(T2FW_ERR_UNSUPPORTED, "B=%lld T=%lld is too large for the block-wise delta-rule kernels", (long long)a.B, (long long)a.T);
+    return split_operands ? launch_backward<true>(a, stream) : launch_backward<false>(a, stream);
 }
 
 }  // namespace t2fw

@@ -41,7 +41,7 @@ __device__ __forceinline__ unsigned char *st_block(unsigned char *smem, int stag
 // One array into one kind of tile, for every stage of the sequence, two stages ahead of the slab waves.  The
 // loads of a stage are issued one stage before its tiles are built, into the register set that the stage
 // before last has left: two sets in turn, so that nothing waits for a load in the stage that issued it.
-template <bool CHANNEL_MAJOR, int NARR>
+template <bool CHANNEL_MAJOR, int NARR, bool SP>
 __device__ __forceinline__ void prep_wave(unsigned char *smem, const float *row0, const float *row1, int off0, int off1, int T,
                                           int nstages, int lane) {
     Raw16 set_a[NARR][DNB], set_b[NARR][DNB];
@@ -64,9 +64,9 @@ __device__ __forceinline__ void prep_wave(unsigned char *smem, const float *row0
                     unsigned char *tile = raw_block(smem, tick, bb) + (a ? off1 : off0);
                     const int tok0 = (tick * DNB + bb) * DL;
                     if (CHANNEL_MAJOR)
-                        store_cm(tile, lane, cur[a][bb], tok0, T);
+                        store_cm<SP>(tile, lane, cur[a][bb], tok0, T);
                     else
-                        store_tm(tile, lane, cur[a][bb], tok0, T);
+                        store_tm<SP>(tile, lane, cur[a][bb], tok0, T);
                 }
         }
         __syncthreads();
@@ -80,38 +80,38 @@ __device__ __forceinline__ void prep_wave(unsigned char *smem, const float *row0
 }
 
 // The state-independent part of block `bb` of every stage, one stage ahead of the slab waves.
-__device__ __forceinline__ void structure_wave(unsigned char *smem, int nstages, int bb, int lane) {
+template <bool SP> __device__ __forceinline__ void structure_wave(unsigned char *smem, int nstages, int bb, int lane) {
     const int r = lane & 15, g = lane >> 4;
     const floatx4 zero = {0.f, 0.f, 0.f, 0.f};
     for (int tick = 0; tick < nstages + 2; ++tick) {
         const int stage = tick - 1;
         if (stage >= 0 && stage < nstages) {
             const unsigned char *raw = raw_block(smem, stage, bb);
-            const TmTile KT(raw + FW_KT), QT(raw + FW_QT);
-            const CmTile KC(raw + FW_KC);
-            const Sp4 k0 = KT.any_order(r, g, 0), k1 = KT.any_order(r, g, 1);
-            const Sp4 q0 = QT.any_order(r, g, 0), q1 = QT.any_order(r, g, 1);
+            const TmTile<SP> KT(raw + FW_KT), QT(raw + FW_QT);
+            const CmTile<SP> KC(raw + FW_KC);
+            const Sp4<SP> k0 = KT.any_order(r, g, 0), k1 = KT.any_order(r, g, 1);
+            const Sp4<SP> q0 = QT.any_order(r, g, 0), q1 = QT.any_order(r, g, 1);
             const floatx4 kk = mma32(k1, k1, mma32(k0, k0, zero));      // [s = 4g+e][t = r] = k_s . k_t
             const floatx4 kq = mma32(k1, q1, mma32(k0, q0, zero));      // [s = 4g+e][t = r] = k_s . q_t
             floatx4 bqt;
 #pragma unroll
             for (int e = 0; e < 4; ++e) bqt[e] = 4 * g + e < r ? kq[e] : 0.f;      // Bq^T[s][t] = k_s . q_t for s < t
-            const BlockInverse inv(kk, r, g);
-            const Sp2 tt = split4(inv.acc_tm_transposed());
+            const BlockInverse<SP> inv(kk, r, g);
+            const Sp2<SP> tt = split4<SP>(inv.acc_tm_transposed());
             unsigned char *st = st_block(smem, stage, bb);
-            st_store(st + FW_TT, lane, tt);
-            st_store(st + FW_BQT, lane, split4(bqt));
+            st_store<SP>(st + FW_TT, lane, tt);
+            st_store<SP>(st + FW_BQT, lane, split4<SP>(bqt));
             // K'^T tile j: [m = 16 j + 4 g + e][t = r] = sum_s K[s][m] Tm[t][s]
             floatx4 kp[4];
 #pragma unroll
             for (int j = 0; j < 4; ++j) kp[j] = mma16(KC.tokens(16 * j + r, g), tt, zero);
-            store_tm_from_acc(st + FW_KP, r, g, kp);
+            store_tm_from_acc<SP>(st + FW_KP, r, g, kp);
         }
         __syncthreads();
     }
 }
 
-__device__ __forceinline__ void slab_wave(const DfwFwdArgs &p, unsigned char *smem, int64_t b, int d0, int nstages, int lane) {
+template <bool SP> __device__ __forceinline__ void slab_wave(const DfwFwdArgs &p, unsigned char *smem, int64_t b, int d0, int nstages, int lane) {
     const int r = lane & 15, g = lane >> 4, d = d0 + r, T = (int)p.T;
     const floatx4 zero = {0.f, 0.f, 0.f, 0.f};
     // token addresses: a wave-uniform base per block plus the lane's fixed offset (first token 4 g, channel d)
@@ -149,17 +149,17 @@ __device__ __forceinline__ void slab_wave(const DfwFwdArgs &p, unsigned char *sm
                 for (int e = 0; e < 4; ++e) vcur[bb][e] = tok0 + 4 * g + e < T ? vcur[bb][e] : 0.f;
                 const unsigned char *raw = raw_block(smem, stage, bb);
                 const unsigned char *st = st_block(smem, stage, bb);
-                const TmTile QT(raw + FW_QT), KP(st + FW_KP);
-                const CmTile KC(raw + FW_KC);
+                const TmTile<SP> QT(raw + FW_QT), KP(st + FW_KP);
+                const CmTile<SP> KC(raw + FW_KC);
                 // Delta[tok 4g+e][d] = Tm V - K' S0^T: only the second term waits for the state
-                const floatx4 tv = mma16(st_load(st + FW_TT, lane), split4(vcur[bb]), zero);
-                const Sp4 sb0 = cat(split4(S[0]), split4(S[1])), sb1 = cat(split4(S[2]), split4(S[3]));
+                const floatx4 tv = mma16(st_load<SP>(st + FW_TT, lane), split4<SP>(vcur[bb]), zero);
+                const Sp4<SP> sb0 = cat(split4<SP>(S[0]), split4<SP>(S[1])), sb1 = cat(split4<SP>(S[2]), split4<SP>(S[3]));
                 const floatx4 ks = mma32(KP.acc_order(r, g, 1), sb1, mma32(KP.acc_order(r, g, 0), sb0, zero));
                 const floatx4 dl = tv - ks;
-                const Sp2 dls = split4(dl);
+                const Sp2<SP> dls = split4<SP>(dl);
                 // O = Q S0^T + Bq Delta
                 const floatx4 qs = mma32(QT.acc_order(r, g, 1), sb1, mma32(QT.acc_order(r, g, 0), sb0, zero));
-                const floatx4 o = qs + mma16(st_load(st + FW_BQT, lane), dls, zero);
+                const floatx4 o = qs + mma16(st_load<SP>(st + FW_BQT, lane), dls, zero);
                 float *const ob = out + (size_t)tok0 * CH_N, *const db = delta + (size_t)tok0 * CH_N;      // wave-uniform
                 if (tok0 + DL <= T) {
 #pragma unroll
@@ -196,7 +196,7 @@ __device__ __forceinline__ void slab_wave(const DfwFwdArgs &p, unsigned char *sm
 
 // blockIdx = half * rows_padded + row with rows_padded a multiple of 8: the two halves of a row land on the
 // same XCD and share its L2 for K and Q, which both read
-__global__ __launch_bounds__(FW_THREADS) void dfw_chunk_fwd_kernel(DfwFwdArgs p, int rows_padded) {
+template <bool SP> __global__ __launch_bounds__(FW_THREADS) void dfw_chunk_fwd_kernel(DfwFwdArgs p, int rows_padded) {
     extern __shared__ __align__(16) unsigned char smem[];
     const int half = (int)blockIdx.x >= rows_padded ? 1 : 0;
     const int64_t b = (int)blockIdx.x - half * rows_padded;
@@ -211,27 +211,31 @@ __global__ __launch_bounds__(FW_THREADS) void dfw_chunk_fwd_kernel(DfwFwdArgs p,
     // prep waves share SIMDs 2 and 3.
     static_assert(DNB == 2, "one matrix wave per block of a stage");
     if (wave < 2)
-        slab_wave(p, smem, b, 32 * half + 16 * wave, nstages, lane);
+        slab_wave<SP>(p, smem, b, 32 * half + 16 * wave, nstages, lane);
     else if (wave < 4)
-        structure_wave(smem, nstages, wave - 2, lane);
+        structure_wave<SP>(smem, nstages, wave - 2, lane);
     else if (wave == 6)
-        prep_wave<false, 2>(smem, k, q, FW_KT, FW_QT, T, nstages, lane);
+        prep_wave<false, 2, SP>(smem, k, q, FW_KT, FW_QT, T, nstages, lane);
     else if (wave == 7)
-        prep_wave<true, 1>(smem, k, k, FW_KC, FW_KC, T, nstages, lane);
+        prep_wave<true, 1, SP>(smem, k, k, FW_KC, FW_KC, T, nstages, lane);
 }
 
 }  // namespace
 
-int dfw_chunk_forward(const DfwFwdArgs &a, hipStream_t stream) {
-    if (a.D != CH_N || a.M != CH_N) return fail(T2FW_ERR_UNSUPPORTED, "the block-wise delta-rule kernels take D = M = 64");
-    if (a.T * CH_N >= 0x7fffffffLL || a.B > 0x1fffffffLL)
-        return fail(T2FW_ERR_UNSUPPORTED, "B=%lld T=%lld is too large for the block-wise delta-rule kernels", (long long)a.B, (long long)a.T);
-    auto kern = dfw_chunk_fwd_kernel;
+template <bool SP> static int launch_forward(const DfwFwdArgs &a, hipStream_t stream) {
+    auto kern = dfw_chunk_fwd_kernel<SP>;
     int rc = enable_lds(reinterpret_cast<const void *>(kern), FW_SMEM, "hipFuncSetAttribute(delta-rule forward kernel)");
     if (rc) return rc;
     const int rows_padded = (int)((a.B + 7) / 8 * 8);
     hipLaunchKernelGGL(kern, dim3(2u * (unsigned)rows_padded), dim3(FW_THREADS), FW_SMEM, stream, a, rows_padded);
     return check_hip(hipGetLastError(), "dfw_chunk_fwd_kernel launch");
+}
+
+int dfw_chunk_forward(const DfwFwdArgs &a, bool split_operands, hipStream_t stream) {
+    if (a.D != CH_N || a.M != CH_N) return fail(T2FW_ERR_UNSUPPORTED, "the block-wise delta-rule kernels take D = M = 64");
+    if (a.T * CH_N >= 0x7fffffffLL || a.B > 0x1fffffffLL)
+        return fail(T2FW_ERR_UNSUPPORTED, "B=%lld T=%lld is too large for the block-wise delta-rule kernels", (long long)a.B, (long long)a.T);
+    return split_operands ? launch_forward<true>(a, stream) : launch_forward<false>(a, stream);
 }
 
 }  // namespace t2fw

@@ -80,6 +80,22 @@ def test_headline_shape_rows_against_the_oracle():
         assert_close(g[rows], r, torch.float32, n, tol=TOL)
 
 
+@pytest.mark.parametrize("B,T", [(3, 100), (9, 257), (2, 1024)])
+def test_single_bf16_operand_mode(B, T):
+    """flag 16: one bf16 operand per product instead of head + remainder.  Held to 1e-2 of max|ref| per result,
+    the bound of the other 16-bit-operand kernels of this library; different from the default's results (so the
+    flag is seen to select other kernels), and the default's stay inside the fp32 tolerance."""
+    q, k, v, s, go, gs = make_inputs(B, T, 64, 64, torch.float32, seed=400 + T)
+    r_out, r_fin, r_grads = dfw_reference_grads(q, k, v, s, go, gs)
+    out, fin, delta, grads = run_abi(q, k, v, s, go, gs, flags=16)
+    out0 = run_abi(q, k, v, s, go, gs, flags=0)[0]
+    assert not torch.equal(out, out0)
+    for n, got, ref in [("outputs", out, r_out), ("final_state", fin, r_fin)] + [(n, g, r) for n, g, r in zip(NAMES, grads, r_grads)]:
+        err = (got.double().cpu() - ref.double()).abs().max().item()
+        scale = ref.double().abs().max().item()
+        assert err <= 1e-2 * scale, "%s: max error %.3e against max|ref| %.3e" % (n, err, scale)
+
+
 def test_autograd_function_uses_the_block_wise_kernels():
     from t2fw.functional_dfw import DFWFunction
     q, k, v, s, go, gs = make_inputs(4, 130, 64, 64, torch.float32, seed=9)

@@ -203,10 +203,12 @@ def test_wide_gate_distribution_stays_on_the_chunked_path():
                          gate_tol=(2e-1, 4e-2))
 
 
-def test_reference_test_gates_stay_on_the_chunked_path():
+def test_reference_test_gates_stay_on_the_matrix_cores_via_the_block_wise_backward():
     # per-channel constant gates in (1/64, 1-1/64) as the reference's tests build them
-    # (16-step products down to 2^-96).  The chunk-parallel backward scales by products over half a
-    # chunk, which these gates take below its range in every row: it hands the rows to the exact scan.
+    # (16-step products down to 2^-96).  The forward takes them.  The chunk-parallel backward scales by
+    # products over half a chunk, which these gates take below its range in every row: it declines both rows
+    # and the block-wise kernel that follows computes them (nothing reaches the exact scan; a caller that
+    # reads the forward's hints goes to the block-wise kernel directly, tests/test_zero_gates_gpu.py).
     # Unit-variance inputs over 256 steps give outputs up to 6, so atol = 1e-2 of the reference's test
     # is below the bf16 rounding of the forward's operands: chunk tolerance only.
     x, f, q, k, fk, s, go, gs = make_reference_test_inputs(2, 256, 64, 64, torch.float16, seed=1)
