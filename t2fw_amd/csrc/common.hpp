@@ -81,6 +81,10 @@ __device__ __forceinline__ double group_sum(double v, int group) {
     return v;
 }
 
+// Wait until none of this wave's global loads and stores is outstanding (s_waitcnt vmcnt(0); the other
+// counters of the immediate left at their maxima, i.e. not waited for).
+__device__ __forceinline__ void wait_vmem_all() { __builtin_amdgcn_s_waitcnt(0x0f70); }
+
 // ----------------------------------------------------------------------------------
 // launch geometry of the exact scan kernels (shared by host dispatch and kernels)
 // ----------------------------------------------------------------------------------

@@ -12,6 +12,7 @@
 //               with Tm, Bq and K'' = Tm^T K prepared ahead by the matrix waves.
 //   key side    one workgroup per (row, half of the key channels): columns of S and of G in fp32 accumulators,
 //               both plain running sums (it reads d_value from the first launch); writes d_query and d_key.
+#include <type_traits>
 #include "common.hpp"
 #include "dfw_chunk.hpp"
 #include "dfw_scan.hpp"
@@ -89,53 +90,57 @@ template <bool SP> __device__ __forceinline__ void vs_slab_wave(const DfwBwdArgs
             for (int e = 0; e < 4; ++e)
                 x[bb][e] = go[(size_t)min(reverse_tok0(nblocks, DNB, stage, bb) + 4 * g + e, T - 1) * CH_N + d];
     };
-    auto tick_body = [&](int tick, floatx4 (&gcur)[DNB], floatx4 (&gnxt)[DNB]) {
-        const int stage = tick - 2;
-        load_g(gnxt, min(max(stage + 1, 0), nstages - 1));
-        if (stage >= 0) {
+    // One stage.  FULL: every token of the stage is below T and the body has no branch.  (The waits that the
+    // compiler places count outstanding memory operations along every path: a path that skips stores, or loads
+    // still pending where the loop is entered, would make each stage wait for the stores of the stage before.)
+    auto stage_body = [&](auto full, int stage, floatx4 (&gcur)[DNB], floatx4 (&gnxt)[DNB]) {
+        constexpr bool FULL = decltype(full)::value;
+        load_g(gnxt, min(stage + 1, nstages - 1));
 #pragma unroll
-            for (int bb = 0; bb < DNB; ++bb) {
-                const int tok0 = reverse_tok0(nblocks, DNB, stage, bb);
+        for (int bb = 0; bb < DNB; ++bb) {
+            const int tok0 = reverse_tok0(nblocks, DNB, stage, bb);
+            if constexpr (!FULL) {
 #pragma unroll
                 for (int e = 0; e < 4; ++e) gcur[bb][e] = tok0 + 4 * g + e < T ? gcur[bb][e] : 0.f;
-                const unsigned char *raw = VsRing::raw(smem, stage, bb);
-                const unsigned char *st = VsRing::st(smem, stage, bb);
-                const TmTile<SP> KPP(st + VS_KPP);
-                const CmTile<SP> KC(raw + VS_KC), QC(raw + VS_QC);
-                // dU[tok 4g+e][d] = Tm^T (Bq^T g) + K'' G_end^T: only the second term waits for the adjoint
-                const Sp2<SP> gs = split4<SP>(gcur[bb]);
-                const floatx4 bg = mma16(st_load<SP>(st + VS_BQ, lane), gs, zero);
-                const floatx4 tbg = mma16(st_load<SP>(st + VS_TM, lane), split4<SP>(bg), zero);
-                const Sp4<SP> gb0 = cat(split4<SP>(G[0]), split4<SP>(G[1])), gb1 = cat(split4<SP>(G[2]), split4<SP>(G[3]));
-                const floatx4 kg = mma32(KPP.acc_order(r, g, 1), gb1, mma32(KPP.acc_order(r, g, 0), gb0, zero));
-                const floatx4 du = tbg + kg;
-                float *const vb = d_v + (size_t)tok0 * CH_N;        // wave-uniform
-                if (tok0 + DL <= T) {
+            }
+            const unsigned char *raw = VsRing::raw(smem, stage, bb);
+            const unsigned char *st = VsRing::st(smem, stage, bb);
+            const TmTile<SP> KPP(st + VS_KPP);
+            const CmTile<SP> KC(raw + VS_KC), QC(raw + VS_QC);
+            // dU[tok 4g+e][d] = Tm^T (Bq^T g) + K'' G_end^T: only the second term waits for the adjoint
+            const Sp2<SP> gs = split4<SP>(gcur[bb]);
+            const floatx4 bg = mma16(st_load<SP>(st + VS_BQ, lane), gs, zero);
+            const floatx4 tbg = mma16(st_load<SP>(st + VS_TM, lane), split4<SP>(bg), zero);
+            const Sp4<SP> gb0 = cat(split4<SP>(G[0]), split4<SP>(G[1])), gb1 = cat(split4<SP>(G[2]), split4<SP>(G[3]));
+            const floatx4 kg = mma32(KPP.acc_order(r, g, 1), gb1, mma32(KPP.acc_order(r, g, 0), gb0, zero));
+            const floatx4 du = tbg + kg;
+            float *const vb = d_v + (size_t)tok0 * CH_N;        // wave-uniform
 #pragma unroll
-                    for (int e = 0; e < 4; ++e) vb[lane_off + e * CH_N] = du[e];
-                } else {
+            for (int e = 0; e < 4; ++e)
+                if (FULL || tok0 + 4 * g + e < T) vb[lane_off + e * CH_N] = du[e];
+            // G += g^T Q - dU^T K
+            const Sp2<SP> ndu = split4<SP>(-du);
 #pragma unroll
-                    for (int e = 0; e < 4; ++e)
-                        if (tok0 + 4 * g + e < T) vb[lane_off + e * CH_N] = du[e];
-                }
-                // G += g^T Q - dU^T K
-                const Sp2<SP> ndu = split4<SP>(-du);
-#pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    G[j] = mma16(QC.tokens(16 * j + r, g), gs, G[j]);
-                    G[j] = mma16(KC.tokens(16 * j + r, g), ndu, G[j]);
-                }
+            for (int j = 0; j < 4; ++j) {
+                G[j] = mma16(QC.tokens(16 * j + r, g), gs, G[j]);
+                G[j] = mma16(KC.tokens(16 * j + r, g), ndu, G[j]);
             }
         }
         __syncthreads();
     };
     floatx4 g_a[DNB], g_b[DNB];
     load_g(g_a, 0);
-    const int nticks = nstages + 2;
-    for (int tick = 0; tick < nticks; tick += 2) {
-        tick_body(tick, g_a, g_b);
-        if (tick + 1 < nticks) tick_body(tick + 1, g_b, g_a);
+    __syncthreads();        // ticks 0 and 1: the prep and matrix waves fill the pipeline
+    __syncthreads();
+    // the blocks are visited last to first: only stage 0 can hold tokens at or past T
+    stage_body(std::false_type{}, 0, g_a, g_b);
+    wait_vmem_all();
+    int stage = 1;
+    for (; stage + 2 <= nstages; stage += 2) {
+        stage_body(std::true_type{}, stage, g_b, g_a);
+        stage_body(std::true_type{}, stage + 1, g_a, g_b);
     }
+    if (stage < nstages) stage_body(std::true_type{}, stage, g_b, g_a);
     float *ds0 = reinterpret_cast<float *>(p.d_s0) + (b * CH_N + d) * CH_N + 4 * g;
 #pragma unroll
     for (int j = 0; j < 4; ++j) *reinterpret_cast<float4 *>(ds0 + 16 * j) = make_float4(G[j][0], G[j][1], G[j][2], G[j][3]);
@@ -227,53 +232,50 @@ template <bool SP> __device__ __forceinline__ void ks_slab_wave(const DfwBwdArgs
                 G[j][e] = gs[(16 * j + 4 * g + e) * CH_N];
             }
     }
-    for (int tick = 0; tick < nstages + 2; ++tick) {
-        const int stage = tick - 2;
-        if (stage >= 0) {
-            const int tok0 = reverse_tok0(nblocks, 1, stage, 0);
-            const unsigned char *raw = KsRing::raw(smem, stage, 0);
-            const unsigned char *st = KsRing::st(smem, stage, 0);
-            const TmTile<SP> DT(raw + KS_DT), GT(raw + KS_GT), NUT(raw + KS_NUT);
-            const CmTile<SP> NDC(raw + KS_NDC), GC(raw + KS_GC), NUC(raw + KS_NUC), KC(raw + KS_KC), QC(raw + KS_QC);
-            const Sp2<SP> kb = KC.tokens(m, g), qb = QC.tokens(m, g);          // K[t = 4g+e][m], Q[t][m]
-            // the adjoint after the block, before it takes the block in
-            const Sp4<SP> gb0 = cat(split4<SP>(G[0]), split4<SP>(G[1])), gb1 = cat(split4<SP>(G[2]), split4<SP>(G[3]));
-            // S0 = S_end - Delta^T K
+    // one stage (= one block); FULL as on the value side
+    auto stage_body = [&](auto full, int stage) {
+        constexpr bool FULL = decltype(full)::value;
+        const int tok0 = reverse_tok0(nblocks, 1, stage, 0);
+        const unsigned char *raw = KsRing::raw(smem, stage, 0);
+        const unsigned char *st = KsRing::st(smem, stage, 0);
+        const TmTile<SP> DT(raw + KS_DT), GT(raw + KS_GT), NUT(raw + KS_NUT);
+        const CmTile<SP> NDC(raw + KS_NDC), GC(raw + KS_GC), NUC(raw + KS_NUC), KC(raw + KS_KC), QC(raw + KS_QC);
+        const Sp2<SP> kb = KC.tokens(m, g), qb = QC.tokens(m, g);          // K[t = 4g+e][m], Q[t][m]
+        // the adjoint after the block, before it takes the block in
+        const Sp4<SP> gb0 = cat(split4<SP>(G[0]), split4<SP>(G[1])), gb1 = cat(split4<SP>(G[2]), split4<SP>(G[3]));
+        // S0 = S_end - Delta^T K
 #pragma unroll
-            for (int j = 0; j < 4; ++j) S[j] = mma16(NDC.tokens(16 * j + r, g), kb, S[j]);
-            const Sp4<SP> sb0 = cat(split4<SP>(S[0]), split4<SP>(S[1])), sb1 = cat(split4<SP>(S[2]), split4<SP>(S[3]));
-            // d_query[t][m] = g S0 + X1 K
-            const floatx4 dq = mma32(GT.acc_order(r, g, 1), sb1, mma32(GT.acc_order(r, g, 0), sb0, zero)) +
-                               mma16(st_load<SP>(st + KS_X1T, lane), kb, zero);
-            // d_key[s][m] = Delta G_end - dU S0 + X1^T Q + (X2 + X2^T) K
-            const floatx4 dk = mma32(NUT.acc_order(r, g, 1), sb1,
-                                     mma32(NUT.acc_order(r, g, 0), sb0,
-                                           mma32(DT.acc_order(r, g, 1), gb1, mma32(DT.acc_order(r, g, 0), gb0, zero)))) +
-                               mma16(st_load<SP>(st + KS_X2S, lane), kb, mma16(st_load<SP>(st + KS_X1, lane), qb, zero));
-            float *const qo = d_q + (size_t)tok0 * CH_N, *const ko = d_k + (size_t)tok0 * CH_N;      // wave-uniform
-            if (tok0 + DL <= T) {
+        for (int j = 0; j < 4; ++j) S[j] = mma16(NDC.tokens(16 * j + r, g), kb, S[j]);
+        const Sp4<SP> sb0 = cat(split4<SP>(S[0]), split4<SP>(S[1])), sb1 = cat(split4<SP>(S[2]), split4<SP>(S[3]));
+        // d_query[t][m] = g S0 + X1 K
+        const floatx4 dq = mma32(GT.acc_order(r, g, 1), sb1, mma32(GT.acc_order(r, g, 0), sb0, zero)) +
+                           mma16(st_load<SP>(st + KS_X1T, lane), kb, zero);
+        // d_key[s][m] = Delta G_end - dU S0 + X1^T Q + (X2 + X2^T) K
+        const floatx4 dk = mma32(NUT.acc_order(r, g, 1), sb1,
+                                 mma32(NUT.acc_order(r, g, 0), sb0,
+                                       mma32(DT.acc_order(r, g, 1), gb1, mma32(DT.acc_order(r, g, 0), gb0, zero)))) +
+                           mma16(st_load<SP>(st + KS_X2S, lane), kb, mma16(st_load<SP>(st + KS_X1, lane), qb, zero));
+        float *const qo = d_q + (size_t)tok0 * CH_N, *const ko = d_k + (size_t)tok0 * CH_N;      // wave-uniform
 #pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    qo[lane_off + e * CH_N] = dq[e];
-                    ko[lane_off + e * CH_N] = dk[e];
-                }
-            } else {
-#pragma unroll
-                for (int e = 0; e < 4; ++e)
-                    if (tok0 + 4 * g + e < T) {
-                        qo[lane_off + e * CH_N] = dq[e];
-                        ko[lane_off + e * CH_N] = dk[e];
-                    }
+        for (int e = 0; e < 4; ++e)
+            if (FULL || tok0 + 4 * g + e < T) {
+                qo[lane_off + e * CH_N] = dq[e];
+                ko[lane_off + e * CH_N] = dk[e];
             }
-            // G_start = G_end + g^T Q - dU^T K
+        // G_start = G_end + g^T Q - dU^T K
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                G[j] = mma16(GC.tokens(16 * j + r, g), qb, G[j]);
-                G[j] = mma16(NUC.tokens(16 * j + r, g), kb, G[j]);
-            }
+        for (int j = 0; j < 4; ++j) {
+            G[j] = mma16(GC.tokens(16 * j + r, g), qb, G[j]);
+            G[j] = mma16(NUC.tokens(16 * j + r, g), kb, G[j]);
         }
         __syncthreads();
-    }
+    };
+    __syncthreads();        // ticks 0 and 1: the prep and matrix waves fill the pipeline
+    __syncthreads();
+    // the blocks are visited last to first: only stage 0 can hold tokens at or past T
+    stage_body(std::false_type{}, 0);
+    wait_vmem_all();
+    for (int stage = 1; stage < nstages; ++stage) stage_body(std::true_type{}, stage);
 }
 
 // Waves 0, 1: slab waves (16 key channels each), alone on SIMDs 0 and 1; wave 2: matrix wave; waves 3, 6, 7: prep

@@ -12,6 +12,7 @@
 //
 // Replaces lfw_cuda_fwd_kernel of the reference's delta rule (t2fw/csrc/dfw_kernel.cu:105-196), semantics
 // t2fw/torch.py:44-53; `delta` is the tensor that kernel emits for its backward (dfw_kernel.cu:176-183).
+#include <type_traits>
 #include "common.hpp"
 #include "dfw_chunk.hpp"
 #include "dfw_scan.hpp"
@@ -138,56 +139,64 @@ template <bool SP> __device__ __forceinline__ void slab_wave(const DfwFwdArgs &p
 #pragma unroll
             for (int e = 0; e < 4; ++e) x[bb][e] = v[(size_t)min((stage * DNB + bb) * DL + 4 * g + e, T - 1) * CH_N + d];
     };
-    auto tick_body = [&](int tick, floatx4 (&vcur)[DNB], floatx4 (&vnxt)[DNB]) {
-        const int stage = tick - 2;
-        load_v(vnxt, min(max(stage + 1, 0), nstages - 1));
-        if (stage >= 0) {
+    // One stage.  FULL: every token of the stage is below T, and the body is free of branches: the waits that
+    // the compiler places count outstanding memory operations along every path, so a path that skips stores
+    // would make the loads of the next stage wait for the stores of this one.
+    auto stage_body = [&](auto full, int stage, floatx4 (&vcur)[DNB], floatx4 (&vnxt)[DNB]) {
+        constexpr bool FULL = decltype(full)::value;
+        load_v(vnxt, min(stage + 1, nstages - 1));
 #pragma unroll
-            for (int bb = 0; bb < DNB; ++bb) {
-                const int tok0 = (stage * DNB + bb) * DL;
+        for (int bb = 0; bb < DNB; ++bb) {
+            const int tok0 = (stage * DNB + bb) * DL;
+            if constexpr (!FULL) {
 #pragma unroll
                 for (int e = 0; e < 4; ++e) vcur[bb][e] = tok0 + 4 * g + e < T ? vcur[bb][e] : 0.f;
-                const unsigned char *raw = raw_block(smem, stage, bb);
-                const unsigned char *st = st_block(smem, stage, bb);
-                const TmTile<SP> QT(raw + FW_QT), KP(st + FW_KP);
-                const CmTile<SP> KC(raw + FW_KC);
-                // Delta[tok 4g+e][d] = Tm V - K' S0^T: only the second term waits for the state
-                const floatx4 tv = mma16(st_load<SP>(st + FW_TT, lane), split4<SP>(vcur[bb]), zero);
-                const Sp4<SP> sb0 = cat(split4<SP>(S[0]), split4<SP>(S[1])), sb1 = cat(split4<SP>(S[2]), split4<SP>(S[3]));
-                const floatx4 ks = mma32(KP.acc_order(r, g, 1), sb1, mma32(KP.acc_order(r, g, 0), sb0, zero));
-                const floatx4 dl = tv - ks;
-                const Sp2<SP> dls = split4<SP>(dl);
-                // O = Q S0^T + Bq Delta
-                const floatx4 qs = mma32(QT.acc_order(r, g, 1), sb1, mma32(QT.acc_order(r, g, 0), sb0, zero));
-                const floatx4 o = qs + mma16(st_load<SP>(st + FW_BQT, lane), dls, zero);
-                float *const ob = out + (size_t)tok0 * CH_N, *const db = delta + (size_t)tok0 * CH_N;      // wave-uniform
-                if (tok0 + DL <= T) {
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) {
-                        ob[lane_off + e * CH_N] = o[e];
-                        db[lane_off + e * CH_N] = dl[e];
-                    }
-                } else {
-#pragma unroll
-                    for (int e = 0; e < 4; ++e)
-                        if (tok0 + 4 * g + e < T) {
-                            ob[lane_off + e * CH_N] = o[e];
-                            db[lane_off + e * CH_N] = dl[e];
-                        }
-                }
-                // S += Delta^T K
-#pragma unroll
-                for (int j = 0; j < 4; ++j) S[j] = mma16(KC.tokens(16 * j + r, g), dls, S[j]);
             }
+            const unsigned char *raw = raw_block(smem, stage, bb);
+            const unsigned char *st = st_block(smem, stage, bb);
+            const TmTile<SP> QT(raw + FW_QT), KP(st + FW_KP);
+            const CmTile<SP> KC(raw + FW_KC);
+            // Delta[tok 4g+e][d] = Tm V - K' S0^T: only the second term waits for the state
+            const floatx4 tv = mma16(st_load<SP>(st + FW_TT, lane), split4<SP>(vcur[bb]), zero);
+            const Sp4<SP> sb0 = cat(split4<SP>(S[0]), split4<SP>(S[1])), sb1 = cat(split4<SP>(S[2]), split4<SP>(S[3]));
+            const floatx4 ks = mma32(KP.acc_order(r, g, 1), sb1, mma32(KP.acc_order(r, g, 0), sb0, zero));
+            const floatx4 dl = tv - ks;
+            const Sp2<SP> dls = split4<SP>(dl);
+            // O = Q S0^T + Bq Delta
+            const floatx4 qs = mma32(QT.acc_order(r, g, 1), sb1, mma32(QT.acc_order(r, g, 0), sb0, zero));
+            const floatx4 o = qs + mma16(st_load<SP>(st + FW_BQT, lane), dls, zero);
+            float *const ob = out + (size_t)tok0 * CH_N, *const db = delta + (size_t)tok0 * CH_N;      // wave-uniform
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+                if (FULL || tok0 + 4 * g + e < T) {
+                    ob[lane_off + e * CH_N] = o[e];
+                    db[lane_off + e * CH_N] = dl[e];
+                }
+            // S += Delta^T K
+#pragma unroll
+            for (int j = 0; j < 4; ++j) S[j] = mma16(KC.tokens(16 * j + r, g), dls, S[j]);
         }
         __syncthreads();
     };
     floatx4 v_a[DNB], v_b[DNB];
     load_v(v_a, 0);
-    const int nticks = nstages + 2;
-    for (int tick = 0; tick < nticks; tick += 2) {      // stage 0 runs in tick 2: the even ticks use set a
-        tick_body(tick, v_a, v_b);
-        if (tick + 1 < nticks) tick_body(tick + 1, v_b, v_a);
+    __syncthreads();        // ticks 0 and 1: the prep and matrix waves fill the pipeline
+    __syncthreads();
+    // Nothing of this wave's is in flight when the loop is entered: the compiler merges what may be outstanding at
+    // the loop head over both ways in, and loads still pending on entry would turn every iteration's waits into
+    // waits for the stores of the iteration before.
+    wait_vmem_all();
+    const int nfull = T / (DL * DNB);       // stages without a token at or past T; at most one more follows
+    int stage = 0;
+    for (; stage + 2 <= nfull; stage += 2) {
+        stage_body(std::true_type{}, stage, v_a, v_b);
+        stage_body(std::true_type{}, stage + 1, v_b, v_a);
+    }
+    if (stage < nfull) {
+        stage_body(std::true_type{}, stage, v_a, v_b);
+        if (stage + 1 < nstages) stage_body(std::false_type{}, stage + 1, v_b, v_a);
+    } else if (stage < nstages) {
+        stage_body(std::false_type{}, stage, v_a, v_b);
     }
     float *fin = reinterpret_cast<float *>(p.final_state) + (b * CH_N + d) * CH_N + 4 * g;
 #pragma unroll
