@@ -216,7 +216,6 @@ static_assert(2 * GR_SMEM <= 160 * 1024, "two workgroups of the gradient kernel 
 
 template <int NT> struct SideState {
     LaneChunk<NT> lc;
-    float inv[NT][4];
 };
 
 template <typename IOE, int NT, bool HEADS, bool FULL> struct GradsItem {
@@ -262,9 +261,12 @@ template <typename IOE, int NT, bool HEADS, bool FULL> struct GradsItem {
         st.lc.scale_by(__builtin_amdgcn_rcpf(st.lc.ref));      // the products up to the middle of the chunk divide out
         to_floats<IOE, NT, FULL>(fv, r.v, n_left);
         to_floats<IOE, NT, FULL>(fa, r.a, n_left);
-        inverse_products<NT>(st.inv, st.lc, gt);
+        // 1 / pre lives only here: the sweeps take the reciprocals again where they use them, which costs four
+        // instructions per token tile and frees sixteen registers for the whole kernel
+        float inv[NT][4];
+        inverse_products<NT>(inv, st.lc, gt);
         uint2 valT[NT], adjS[NT];
-        scale_pack<NT>(valT, fv, st.inv);
+        scale_pack<NT>(valT, fv, inv);
         scale_pack<NT>(adjS, fa, st.lc.pre);
         store_cm<NT>(tile_val<SIDE>(), c, kg, valT);
         store_cm<NT>(tile_adj<SIDE>(), c, kg, adjS);
@@ -357,6 +359,7 @@ template <typename IOE, int NT, bool HEADS, bool FULL> struct GradsItem {
         u16 *d_val, *d_gate, *d_adj;
         float du[NT][4];
         float anchor_acc;                        // sum_t adjS_t * (S0' adj-op_t)
+        float anchor, carry;                     // gate gradient: see begin_gate_gradient
 
         __device__ __forceinline__ Sweep(const GradsItem &g_, const SideState<NT> &st_) : g(g_), st(st_) {
             own_adj = g.template tile_adj<SIDE>(); own_val = g.template tile_val<SIDE>();
@@ -408,7 +411,13 @@ template <typename IOE, int NT, bool HEADS, bool FULL> struct GradsItem {
 #pragma unroll
             for (int j = 0; j < 4; ++j) du[m][j] = af[j] * acc[j];
         }
-        // backward-like sweep, token tile n: x' (value side) / k' (key side)
+        // gate gradient = (anchor - sum over the earlier tokens of du) / gate; diag = rowsum / colsum of Gh' * S0'
+        __device__ __forceinline__ void begin_gate_gradient(float diag_part) {
+            anchor = diag_part + row_scan_add(anchor_acc, g.kg).all;
+            carry = 0.f;
+        }
+        // backward-like sweep, token tile n: x' (value side) / k' (key side); then the tile's gate gradient (du of
+        // this tile and of the earlier ones is final by now)
         __device__ __forceinline__ void backward_tile(int n, const uint4 &gha, const uint4 &ghb) {
             const floatx4 zero = {0.f, 0.f, 0.f, 0.f};
             const uint2 none = make_uint2(0u, 0u);
@@ -420,37 +429,30 @@ template <typename IOE, int NT, bool HEADS, bool FULL> struct GradsItem {
                                    cat(b_adj(m0), m0 + 1 < NT ? b_adj(m0 + 1) : none), acc);
             const float4 dgv = *reinterpret_cast<const float4 *>(pd + 16 * n + 4 * g.kg);
             const float dg[4] = {dgv.x, dgv.y, dgv.z, dgv.w};
-            float af[4], vf[4], dv[4];
+            float af[4], vf[4], dv[4], inv[4];
             unpack4<Bf16>(b_adj(n), af);
             unpack4<Bf16>(b_val(n), vf);
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
-                dv[j] = st.inv[n][j] * (acc[j] + af[j] * dg[j]);
+                inv[j] = __builtin_amdgcn_rcpf(st.lc.pre[n][j]);
+                dv[j] = inv[j] * (acc[j] + af[j] * dg[j]);
                 du[n][j] -= vf[j] * acc[j];
             }
             store4(d_val, n, dv);
-        }
-        // gate gradient = (anchor - sum over the earlier tokens of du) / gate; diag = rowsum / colsum of Gh' * S0'
-        __device__ __forceinline__ void gate_gradient(float diag_part) {
-            const float anchor = diag_part + row_scan_add(anchor_acc, g.kg).all;
-            float carry = 0.f;
+            float e[4];
+            e[0] = 0.f;
 #pragma unroll
-            for (int m = 0; m < NT; ++m) {
-                float e[4];
-                e[0] = 0.f;
+            for (int j = 1; j < 4; ++j) e[j] = e[j - 1] + du[n][j - 1];
+            const RowScan sc = row_scan_add(e[3] + du[n][3], g.kg);
+            const float base = anchor - (carry + sc.lower);
+            carry += sc.all;
+            float dgt[4];
 #pragma unroll
-                for (int j = 1; j < 4; ++j) e[j] = e[j - 1] + du[m][j - 1];
-                const RowScan sc = row_scan_add(e[3] + du[m][3], g.kg);
-                const float base = anchor - (carry + sc.lower);
-                carry += sc.all;
-                float dgt[4];
-#pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    const float rgate = (j == 0 ? st.lc.off[m] : st.lc.pre[m][j > 0 ? j - 1 : 0]) * st.inv[m][j];      // 1 / gate
-                    dgt[j] = (base - e[j]) * rgate;
-                }
-                store4(d_gate, m, dgt);
+            for (int j = 0; j < 4; ++j) {
+                const float rgate = (j == 0 ? st.lc.off[n] : st.lc.pre[n][j > 0 ? j - 1 : 0]) * inv[j];      // 1 / gate
+                dgt[j] = (base - e[j]) * rgate;
             }
+            store4(d_gate, n, dgt);
         }
         // rowsum / colsum of Gh' * S0' = diagonal of Gh' S0'^T
         __device__ __forceinline__ float state_diagonal(const uint4 &s0a, const uint4 &s0b, const uint4 &gha, const uint4 &ghb) const {
@@ -477,13 +479,13 @@ template <typename IOE, int NT, bool HEADS, bool FULL> struct GradsItem {
         {
             lds_fence();
             const uint4 gha = w.state_op(GR_GH, 0), ghb = w.state_op(GR_GH, 1);
+            w.begin_gate_gradient(diag_part);
 #pragma unroll
             for (int n = 0; n < NT; ++n) {
                 lds_fence();
                 w.backward_tile(n, gha, ghb);
             }
         }
-        w.gate_gradient(diag_part);
     }
 
     template <int SIDE> __device__ __forceinline__ void run_side() const {
