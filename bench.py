@@ -353,6 +353,8 @@ def main():
             torch.cuda.empty_cache()
             others["dfw"] = brief(bench_dfw(args, 20, 5))
             others["dfw_bf16_operands"] = brief(bench_dfw(args, 20, 5, bf16_operands=True))
+            torch.cuda.empty_cache()
+            others["cfg3_float32"] = bench_float32(args, 20, 3)
             line["other_configs"] = others
     print(json.dumps(line))
 
@@ -511,6 +513,50 @@ def bench_dfw(args, steps, warmup, bf16_operands=False):
         "cpu_baseline": None,
     }
     return line
+
+
+def bench_float32(args, steps, warmup):
+    """cfg3's shape with float32 tensors through the autograd API: LFWFunction.apply (exact kernels: the
+    matrix-core kernels take 16-bit tensors) against lfw_apply_16bit (casts to float16 around the matrix-core
+    kernels, the caller's explicit choice), and the second one's error against the first's results."""
+    import torch
+    from t2fw_amd import LFWFunction, lfw_apply_16bit
+    from t2fw_amd.synthetic import make_config_inputs
+    w = WORKLOADS["cfg3"]
+    B, T, D, K = w["B"], w["T"], w["D"], w["K"]
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    os.environ["T2FW_CKPT_INTERVAL"] = str(args.ckpt_interval)
+    os.environ["T2FW_FLAGS"] = "0"
+    x, f, q, k, fk, s0, go, gs = make_config_inputs(B, T, D, K, torch.float32, seed=0, gate_mean=w["gate_mean"])
+    leaves = [t.to(dev).requires_grad_(True) for t in (x, f, q, k, fk, s0)]
+    go, gs = go.to(dev), gs.to(dev)
+
+    def run(fn, n):
+        res = None
+        for _ in range(n):
+            for t in leaves:
+                t.grad = None
+            o, nx = fn(*leaves)
+            torch.autograd.backward([o, nx], [go, gs])
+            res = [o.detach(), nx.detach()] + [t.grad for t in leaves]
+        return res
+    out = {}
+    results = {}
+    for name, fn, n in (("exact_float32", LFWFunction.apply, max(2, steps // 4)), ("cast_to_float16", lfw_apply_16bit, steps)):
+        run(fn, warmup)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        results[name] = run(fn, n)
+        torch.cuda.synchronize()
+        ms = (time.perf_counter() - t0) / n * 1e3
+        out[name] = {"value": round(B * T / ms / 1e3, 1), "unit": "Mtokens/s", "ms_per_step": round(ms, 5), "steps": n}
+    names = ["outputs", "next_state", "d_x", "d_f", "d_q", "d_k", "d_f_key", "d_state"]
+    worst = max(((a - b).abs().max() / b.abs().max()).item() for a, b in zip(results["cast_to_float16"], results["exact_float32"]))
+    out["cast_to_float16"]["max_abs_over_max_ref_vs_exact_float32"] = round(worst, 6)
+    out["cast_to_float16"]["tensors"] = names
+    out["workload"] = "cfg3 shape, float32 tensors, LFWFunction.apply + autograd backward (host and allocations included)"
+    return out
 
 
 def bench_generation(args, steps, warmup):

@@ -237,6 +237,15 @@ int t2fw_dfw_backward(const void *g_out, const void *g_state,
                       int32_t dtype, int32_t flags, void *stream);
 
 /*
+ * Conversion of `count` (<= 8) arrays of n[i] elements each between float32 and float16 / bfloat16 in one
+ * launch (src_dtype -> dst_dtype, one of them T2FW_F32); arrays 16-byte aligned, `src`, `dst`, `n` host arrays.
+ * No counterpart in the reference (one kernel serves every dtype there, lfw_kernel.cu:157-168): it is what a
+ * caller with float32 tensors uses to run the 16-bit matrix-core kernels (lfw_apply_16bit of the Python side).
+ */
+int t2fw_cast(const void *const *src, void *const *dst, const int64_t *n, int32_t count,
+              int32_t src_dtype, int32_t dst_dtype, void *stream);
+
+/*
  * Sigmoid gating of both forget gates in one launch: f = sigmoid(f_logit) [n_f elements],
  * f_key = sigmoid(fk_logit) [n_fk elements]; outputs may alias the inputs.  The reference leaves
  * the non-linearity to the caller (functional_lfw.py:25-30); dtype f32 / f16 / bf16.

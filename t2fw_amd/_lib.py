@@ -42,6 +42,7 @@ SIGNATURES = {
     "t2fw_lfw_forward_heads": (ctypes.c_int, [_vp] * 9 + [_i64] * 5 + [_i32] * 3 + [_vp, _sz, _vp]),
     "t2fw_lfw_backward_heads": (ctypes.c_int, [_vp] * 15 + [_i64] * 5 + [_i32] * 3 + [_vp, _sz, _vp]),
     "t2fw_lfw_step": (ctypes.c_int, [_vp] * 8 + [_i64] * 3 + [_i32, _vp]),
+    "t2fw_cast": (ctypes.c_int, [ctypes.POINTER(ctypes.c_void_p)] * 2 + [ctypes.POINTER(ctypes.c_int64), _i32, _i32, _i32, _vp]),
     "t2fw_gate_forward": (ctypes.c_int, [_vp] * 4 + [_i64] * 2 + [_i32, _vp]),
     "t2fw_gate_backward": (ctypes.c_int, [_vp] * 6 + [_i64] * 2 + [_i32, _vp]),
     "t2fw_dfw_forward": (ctypes.c_int, [_vp] * 7 + [_i64] * 4 + [_i32, _i32, _vp]),
@@ -85,3 +86,18 @@ def ptr(t):
 
 def current_stream_handle(device):
     return ctypes.c_void_p(torch.cuda.current_stream(device).cuda_stream)
+
+
+def cast_tensors(srcs, dsts, stream):
+    """One launch of t2fw_cast: srcs[i] -> dsts[i] elementwise (float32 <-> float16 / bfloat16; every source of
+    one dtype, every destination of one dtype; contiguous tensors of equal element counts, at most eight)."""
+    lib = load()
+    n = len(srcs)
+    assert n == len(dsts) and 0 < n <= 8
+    for a, b in zip(srcs, dsts):
+        assert a.numel() == b.numel() and a.is_contiguous() and b.is_contiguous()
+        assert a.dtype == srcs[0].dtype and b.dtype == dsts[0].dtype
+    sp = (ctypes.c_void_p * n)(*[ptr(t) for t in srcs])
+    dp = (ctypes.c_void_p * n)(*[ptr(t) for t in dsts])
+    cnt = (ctypes.c_int64 * n)(*[t.numel() for t in srcs])
+    check(lib.t2fw_cast(sp, dp, cnt, n, DTYPE_CODE[srcs[0].dtype], DTYPE_CODE[dsts[0].dtype], stream))

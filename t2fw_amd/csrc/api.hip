@@ -5,6 +5,7 @@
 #include "lfw_chunk.hpp"
 #include "lfw_par.hpp"
 #include "dfw_scan.hpp"
+#include "cast.hpp"
 #include "gate.hpp"
 #include "lfw_step.hpp"
 
@@ -566,6 +567,21 @@ int t2fw_dfw_backward(const void *g_out, const void *g_state, const void *q, con
         aligned16({g_out, g_state, q, k, delta, final_state, d_q, d_k, d_v, d_s0}))
         return dfw_chunk_backward(a, (flags & T2FW_FLAG_BF16_OPERANDS) == 0, st);
     return dfw_backward(a, dtype, st);
+}
+
+int t2fw_cast(const void *const *src, void *const *dst, const int64_t *n, int32_t count, int32_t src_dtype,
+              int32_t dst_dtype, void *stream) {
+    if (count < 0 || count > CAST_MAX_TENSORS) return fail(T2FW_ERR_BAD_SHAPE, "t2fw_cast takes 0 to %d arrays, got %d", CAST_MAX_TENSORS, count);
+    if (count > 0 && (src == nullptr || dst == nullptr || n == nullptr)) return fail(T2FW_ERR_NULL_POINTER, "null pointer list");
+    CastArgs a{};
+    a.count = count;
+    for (int i = 0; i < count; ++i) {
+        if (n[i] < 0) return fail(T2FW_ERR_BAD_SHAPE, "element counts must be non-negative");
+        if (n[i] > 0 && (src[i] == nullptr || dst[i] == nullptr)) return fail(T2FW_ERR_NULL_POINTER, "null array pointer");
+        if (!aligned16({src[i], dst[i]})) return fail(T2FW_ERR_MISALIGNED, "arrays must be 16-byte aligned");
+        a.src[i] = src[i]; a.dst[i] = dst[i]; a.n[i] = n[i];
+    }
+    return cast_tensors(a, src_dtype, dst_dtype, static_cast<hipStream_t>(stream));
 }
 
 int t2fw_gate_forward(const void *f_logit, const void *fk_logit, void *f, void *f_key, int64_t n_f, int64_t n_fk,

@@ -288,6 +288,68 @@ class LFWHeadsFunction(torch.autograd.Function):
         return d_x, d_f, d_q, d_k, d_fk, d_s, None
 
 
+def _narrow_copies(tensors, dtype, stream):
+    """``dtype`` copies of float32 tensors: one allocation, one launch."""
+    dev = tensors[0].device
+    offs, total = [], 0
+    for t in tensors:
+        offs.append(total)
+        total += (t.numel() + 127) // 128 * 128          # every copy starts 256 bytes aligned
+    buf = torch.empty(total, dtype=dtype, device=dev)
+    outs = [buf[o:o + t.numel()].view(t.shape) for o, t in zip(offs, tensors)]
+    _lib.cast_tensors(list(tensors), outs, stream)
+    return outs
+
+
+class LFW16Function(torch.autograd.Function):
+    """The recurrence on float32 tensors through the 16-bit matrix-core kernels (see lfw_apply_16bit).  The
+    16-bit copies of the inputs, not the float32 tensors, are what is kept for the backward."""
+
+    @staticmethod
+    def forward(ctx, value, forget, query, key, f_key, state, dtype):
+        ins = (value, forget, query, key, f_key, state)
+        for t, n in zip(ins, ("x", "f", "query", "key", "f_key", "state")):
+            _check_input(t, n)
+            if t.dtype != torch.float32:
+                raise RuntimeError("t2fw: lfw_apply_16bit takes float32 tensors, %s is %s" % (n, t.dtype))
+        need_grad = any(ctx.needs_input_grad)
+        dev = value.device
+        with _on_device(dev):
+            stream = _lib.current_stream_handle(dev)
+            narrow = _narrow_copies(ins, dtype, stream)
+            out16, nxt16, ckpt, C, flags, hints = _lfw_forward(*narrow, need_grad)
+            outputs, next_state = torch.empty_like(value), torch.empty_like(state)
+            _lib.cast_tensors([out16, nxt16], [outputs, next_state], stream)
+        if need_grad:
+            ctx.save_for_backward(*narrow, ckpt)
+            ctx.ckpt_interval, ctx.flags, ctx.hints, ctx.narrow = C, flags, hints, dtype
+        return outputs, next_state
+
+    @staticmethod
+    def backward(ctx, grad_output, grad_state):
+        *narrow, ckpt = ctx.saved_tensors
+        dev = grad_output.device
+        with _on_device(dev):
+            stream = _lib.current_stream_handle(dev)
+            go16, gs16 = _narrow_copies((grad_output.contiguous().float(), grad_state.contiguous().float()), ctx.narrow, stream)
+            grads16 = _lfw_backward(go16, gs16, *narrow, ckpt, ctx.ckpt_interval, ctx.flags, hints=ctx.hints)
+            grads = [torch.empty(g.shape, dtype=torch.float32, device=dev) for g in grads16]
+            _lib.cast_tensors(list(grads16), grads, stream)
+        return (*grads, None)
+
+
+def lfw_apply_16bit(value, forget, query, key, f_key, state, dtype=torch.float16):
+    """``LFWFunction.apply`` for float32 tensors at the speed of the 16-bit matrix-core kernels: the six
+    inputs are converted to ``dtype`` (float16 or bfloat16) in one launch, the recurrence and its backward
+    run in that type, outputs and gradients come back as float32.  An explicit choice of the caller: the
+    results carry the 16-bit kernels' accuracy (within 1e-2 of max|ref| per tensor; gates are rounded to
+    ``dtype`` before they are multiplied up, 2^-11 relative per step in float16, so bfloat16 is for short
+    memories only), where ``LFWFunction.apply`` on float32 tensors runs the exact kernels.  The reference
+    has one kernel for every dtype (t2fw/csrc/lfw_kernel.cu:157-168) and no counterpart of this."""
+    assert dtype in (torch.float16, torch.bfloat16)
+    return LFW16Function.apply(value, forget, query, key, f_key, state, dtype)
+
+
 def lfw_step(x, f, query, key, f_key, state, out=None, inplace=True):
     """One generation step (T = 1) without autograd: x,f [B,D]; query,key,f_key [B,K];
     state [B,D,K] updated in place when ``inplace``.  Returns (out [B,D], state).

@@ -29,7 +29,7 @@ def declared_functions():
 def test_header_declares_the_expected_entry_points():
     names = declared_functions()
     for n in ("t2fw_lfw_forward", "t2fw_lfw_backward", "t2fw_lfw_step", "t2fw_dfw_forward",
-              "t2fw_dfw_backward", "t2fw_last_error", "t2fw_abi_version", "t2fw_lfw_num_ckpt",
+              "t2fw_dfw_backward", "t2fw_cast", "t2fw_last_error", "t2fw_abi_version", "t2fw_lfw_num_ckpt",
               "t2fw_lfw_workspace_bytes"):
         assert n in names
 

@@ -351,3 +351,26 @@ def test_sparse_checkpoints_with_rows_that_fall_back():
     for n, g, r in zip(NAMES, grads, r_grads):
         assert_close(g, r, torch.float16, n, tol=TOL_CHUNK_GATE if n in ("d_f", "d_f_key") else TOL_CHUNK)
         assert_close(g[1:2], r[1:2], torch.float16, n + "[row on the exact scan]")
+
+
+def test_float32_tensors_through_the_16_bit_kernels_by_explicit_cast():
+    """lfw_apply_16bit: float32 in and out, the float16 matrix-core kernels in between; against the float64
+    oracle on the float32 inputs, every tensor within 1e-2 of max|ref| (the gates' rounding to float16
+    included), and the plain float32 call on the same inputs within the exact kernels' tolerance"""
+    from oracle.lfw_ref import lfw_reference_grads
+    from t2fw_amd import LFWFunction, lfw_apply_16bit
+    x, f, q, k, fk, s, go, gs = make_config_inputs(4, 200, 64, 64, torch.float32, seed=77, state_std=0.2)
+    r_out, r_nxt, r_grads = lfw_reference_grads(x, f, q, k, fk, s, go, gs)
+    refs = [r_out, r_nxt] + list(r_grads)
+    names = ["outputs", "next_state", "d_x", "d_f", "d_q", "d_k", "d_f_key", "d_state"]
+    for fn, bound in ((lfw_apply_16bit, 1e-2), (LFWFunction.apply, 1e-4)):
+        ins = [t.cuda().requires_grad_(True) for t in (x, f, q, k, fk, s)]
+        o, n = fn(*ins)
+        assert o.dtype == torch.float32 and n.dtype == torch.float32
+        torch.autograd.backward([o, n], [go.cuda(), gs.cuda()])
+        got = [o, n] + [t.grad for t in ins]
+        for name, g, r in zip(names, got, refs):
+            assert g.dtype == torch.float32
+            err = (g.detach().double().cpu() - r.double()).abs().max().item()
+            scale = r.double().abs().max().item()
+            assert err <= bound * scale, "%s (bound %g of max|ref|): max error %.3e against max|ref| %.3e" % (name, bound, err, scale)
