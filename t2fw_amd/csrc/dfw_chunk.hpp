@@ -81,6 +81,7 @@ template <bool SP> __device__ __forceinline__ floatx4 mma32(const Sp4<SP> &a, co
 // ---- tiles in LDS: a head tile followed by a remainder tile of the same shape ----------------------
 // token-major [16][DTS]: channel c of a token sits at tm_pos(c), so that the sixteen channels a matrix lane
 // (r, g) pairs with its accumulators (16 j + 4 g + e) are contiguous at 16 g
+typedef __attribute__((address_space(3))) short4_t *lds_tr_ptr;
 template <bool SP> struct TmTile {
     const u16 *hi, *lo;
     __device__ __forceinline__ TmTile(const unsigned char *base) : hi(reinterpret_cast<const u16 *>(base)), lo(reinterpret_cast<const u16 *>(base + TM_TILE)) {}
@@ -97,6 +98,16 @@ template <bool SP> struct TmTile {
         o.hi = ld4(hi + row * DTS + 8 * g + 32 * h);
         o.lo = SP ? ld4(lo + row * DTS + 8 * g + 32 * h) : make_uint4(0u, 0u, 0u, 0u);
         return o;
+    }
+    // A operand "channel 16 j + r, tokens 4 g .. 4 g + 3" for lane (r, g): a column of the tile, through the
+    // transposing LDS read (lane r of a 16-lane group fetches the 8 bytes of token 4 g + r / 4 that hold channels
+    // 16 j + 4 (r % 4) .. + 3; the hardware hands lane r the four tokens of channel 16 j + r)
+    __device__ __forceinline__ Sp2<SP> column(int j, int r, int g) const {
+        const int o = (4 * g + (r >> 2)) * DTS + 16 * (r & 3) + 4 * j;
+        Sp2<SP> v;
+        v.hi = __builtin_bit_cast(uint2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_tr_ptr)(hi + o)));
+        v.lo = SP ? __builtin_bit_cast(uint2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_tr_ptr)(lo + o))) : make_uint2(0u, 0u);
+        return v;
     }
 };
 // channel-major [64][DCS]: A operand "channel `ch`, tokens 4 g .. 4 g + 3"
@@ -231,51 +242,79 @@ template <int RAW_BLOCK, int ST_BLOCK, int NBLK> struct Ring {
     }
 };
 
-// One wave stages NJOBS arrays (all token-major or all channel-major) for every stage, two stages ahead of the
-// slab waves.  Loads of a stage are issued, unconditionally, one stage before its tiles are built, into the
-// register set the stage before last has left.  tok0_of(stage, bb): first token of a block (at or past T: a
-// block of zeros).
+// One wave stages NJOBS arrays for every stage, two stages ahead of the slab waves.  An array is loaded once,
+// token-major (four 16-byte loads per lane and block), and written as a token-major tile; where a channel-major
+// tile of the same array is wanted too, the wave reads its own token-major tile back with the transposing LDS
+// read and writes that (the loads of a second layout were what the wave waited for: a wave can have 63 memory
+// instructions outstanding, and a channel-major tile loaded directly is sixteen 4-byte loads per lane).
+// Loads are unconditional and issued SETS - 1 stages before their tiles are built, into the register set that the
+// stage before has left (SETS sets in turn; the stage loop is unrolled SETS times so that no register copy waits
+// for a load).  tok0_of(stage, bb): first token of a block (at or past T: a block of zeros).
 struct PrepJob {
     const float *src;       // token 0 of the batch row
-    int off;                // byte offset of the tile inside a block's raw tiles
-    float sign;             // the tile holds sign * src
+    int tm_off;             // byte offset of the token-major tile inside a block's raw tiles; < 0: the wave's scratch tile
+    int cm_off;             // byte offset of the channel-major tile; < 0: none
+    float sign;             // the token-major tile holds sign * src
+    bool cm_negated;        // the channel-major tile holds the negative of the token-major one
 };
-template <typename RING, int NBLK, bool CHANNEL_MAJOR, int NJOBS, bool SP, typename TOK0>
+template <typename RING, int NBLK, int NJOBS, bool SP, int SETS, typename TOK0>
 __device__ __forceinline__ void prep_wave_jobs(unsigned char *smem, const PrepJob (&jobs)[NJOBS], int T, int nstages, int lane,
-                                               TOK0 tok0_of) {
-    Raw16 set_a[NJOBS][NBLK], set_b[NJOBS][NBLK];
-    auto load = [&](Raw16 (&r)[NJOBS][NBLK], int stage) {
+                                               TOK0 tok0_of, unsigned char *scratch_tile) {
+    static_assert(SETS == 2 || SETS == 3, "two or three register sets");
+    const int r = lane & 15, g = lane >> 4;
+    Raw16 set_a[NJOBS][NBLK], set_b[NJOBS][NBLK], set_c[SETS == 3 ? NJOBS : 1][SETS == 3 ? NBLK : 1];
+    auto load = [&](auto &regs, int stage) {
+#pragma unroll
+        for (int a = 0; a < NJOBS; ++a)
+#pragma unroll
+            for (int bb = 0; bb < NBLK; ++bb) regs[a][bb] = load_tm(jobs[a].src, tok0_of(stage, bb), T, lane);
+    };
+    // stage `stage` out of `cur`; the loads of stage + SETS - 1 into `far` (the set that stage - 1 has left)
+    auto stage_body = [&](int stage, auto &cur, auto &far) {
+        load(far, min(stage + SETS - 1, nstages - 1));
 #pragma unroll
         for (int a = 0; a < NJOBS; ++a)
 #pragma unroll
             for (int bb = 0; bb < NBLK; ++bb) {
-                const int tok0 = tok0_of(stage, bb);
-                r[a][bb] = CHANNEL_MAJOR ? load_cm(jobs[a].src, tok0, T, lane) : load_tm(jobs[a].src, tok0, T, lane);
-            }
-    };
-    auto tick_body = [&](int tick, Raw16 (&cur)[NJOBS][NBLK], Raw16 (&nxt)[NJOBS][NBLK]) {
-        load(nxt, min(tick + 1, nstages - 1));
-        if (tick < nstages) {
+                unsigned char *const raw = RING::raw(smem, stage, bb);
+                unsigned char *const tm = jobs[a].tm_off >= 0 ? raw + jobs[a].tm_off : scratch_tile;
+                store_tm<SP>(tm, lane, cur[a][bb], tok0_of(stage, bb), T, jobs[a].sign);
+                if (jobs[a].cm_off >= 0) {
+                    // DS operations of one wave execute in order: the reads below see the tile just written
+                    const TmTile<SP> own(tm);
+                    u16 *const hi = reinterpret_cast<u16 *>(raw + jobs[a].cm_off), *const lo = reinterpret_cast<u16 *>(raw + jobs[a].cm_off + CM_TILE);
+                    const u32 flip = jobs[a].cm_negated ? 0x80008000u : 0u;
 #pragma unroll
-            for (int a = 0; a < NJOBS; ++a)
-#pragma unroll
-                for (int bb = 0; bb < NBLK; ++bb) {
-                    unsigned char *tile = RING::raw(smem, tick, bb) + jobs[a].off;
-                    const int tok0 = tok0_of(tick, bb);
-                    if (CHANNEL_MAJOR)
-                        store_cm<SP>(tile, lane, cur[a][bb], tok0, T, jobs[a].sign);
-                    else
-                        store_tm<SP>(tile, lane, cur[a][bb], tok0, T, jobs[a].sign);
+                    for (int j = 0; j < 4; ++j) {
+                        const Sp2<SP> col = own.column(j, r, g);          // channel 16 j + r, tokens 4 g .. 4 g + 3
+                        const int o = (16 * j + r) * DCS + 4 * g;
+                        *reinterpret_cast<uint2 *>(hi + o) = make_uint2(col.hi.x ^ flip, col.hi.y ^ flip);
+                        if constexpr (SP) *reinterpret_cast<uint2 *>(lo + o) = make_uint2(col.lo.x ^ flip, col.lo.y ^ flip);
+                    }
                 }
-        }
+            }
         __syncthreads();
     };
     load(set_a, 0);
-    const int nticks = nstages + 2;
-    for (int tick = 0; tick < nticks; tick += 2) {
-        tick_body(tick, set_a, set_b);
-        if (tick + 1 < nticks) tick_body(tick + 1, set_b, set_a);
+    int stage = 0;
+    if constexpr (SETS == 3) {
+        load(set_b, min(1, nstages - 1));
+        for (; stage + 3 <= nstages; stage += 3) {
+            stage_body(stage, set_a, set_c);
+            stage_body(stage + 1, set_b, set_a);
+            stage_body(stage + 2, set_c, set_b);
+        }
+        if (stage < nstages) stage_body(stage, set_a, set_c);
+        if (stage + 1 < nstages) stage_body(stage + 1, set_b, set_a);
+    } else {
+        for (; stage + 2 <= nstages; stage += 2) {
+            stage_body(stage, set_a, set_b);
+            stage_body(stage + 1, set_b, set_a);
+        }
+        if (stage < nstages) stage_body(stage, set_a, set_b);
     }
+    __syncthreads();        // the two ticks in which the other waves finish
+    __syncthreads();
 }
 
 }  // namespace dfwc

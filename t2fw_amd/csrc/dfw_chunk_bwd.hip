@@ -164,11 +164,11 @@ template <bool SP> __global__ __launch_bounds__(BW_THREADS) void dfw_chunk_bwd_v
     } else if (wave < 4) {
         vs_structure_wave<SP>(smem, nstages, wave - 2, lane);
     } else if (wave == 6) {
-        const PrepJob jobs[2] = {{k, VS_KT, 1.f}, {q, VS_QT, 1.f}};
-        prep_wave_jobs<VsRing, DNB, false, 2, SP>(smem, jobs, T, nstages, lane, tok0_of);
+        const PrepJob jobs[1] = {{k, VS_KT, VS_KC, 1.f, false}};
+        prep_wave_jobs<VsRing, DNB, 1, SP, 3>(smem, jobs, T, nstages, lane, tok0_of, nullptr);
     } else if (wave == 7) {
-        const PrepJob jobs[2] = {{k, VS_KC, 1.f}, {q, VS_QC, 1.f}};
-        prep_wave_jobs<VsRing, DNB, true, 2, SP>(smem, jobs, T, nstages, lane, tok0_of);
+        const PrepJob jobs[1] = {{q, VS_QT, VS_QC, 1.f, false}};
+        prep_wave_jobs<VsRing, DNB, 1, SP, 3>(smem, jobs, T, nstages, lane, tok0_of, nullptr);
     }
 }
 
@@ -179,7 +179,15 @@ constexpr int KS_DT = 0, KS_GT = KS_DT + 2 * TM_TILE, KS_NUT = KS_GT + 2 * TM_TI
               KS_QC = KS_KC + 2 * CM_TILE, KS_RAW_BLOCK = KS_QC + 2 * CM_TILE;
 constexpr int KS_X1 = 0, KS_X1T = KS_X1 + 2 * ST_TILE, KS_X2S = KS_X1T + 2 * ST_TILE, KS_ST_BLOCK = KS_X2S + 2 * ST_TILE;
 using KsRing = Ring<KS_RAW_BLOCK, KS_ST_BLOCK, 1>;
-static_assert(KsRing::SMEM <= 160 * 1024, "key-side tiles exceed the LDS of one CU");
+// The adjoint waves hand G_end of a block to the state waves as a ready B operand: per (stage parity, wave,
+// half of the value channels, head / remainder) 16 bytes per lane.
+constexpr int KS_XG = KsRing::SMEM, KS_XG_PIECE = 64 * 16, KS_SCRATCH = KS_XG + 2 * 2 * 2 * 2 * KS_XG_PIECE;
+// ... and two prep waves keep a token-major tile of their own (K, Q: wanted channel-major only)
+constexpr int KS_SMEM = KS_SCRATCH + 2 * 2 * TM_TILE;
+static_assert(KS_SMEM <= 160 * 1024, "key-side tiles exceed the LDS of one CU");
+__device__ __forceinline__ uint4 *xg_piece(unsigned char *smem, int stage, int wave, int which, int part, int lane) {
+    return reinterpret_cast<uint4 *>(smem + KS_XG + ((((stage & 1) * 2 + wave) * 2 + which) * 2 + part) * KS_XG_PIECE) + lane;
+}
 
 template <bool SP> __device__ __forceinline__ void ks_structure_wave(unsigned char *smem, int nstages, int lane) {
     const int r = lane & 15, g = lane >> 4;
@@ -213,36 +221,75 @@ template <bool SP> __device__ __forceinline__ void ks_structure_wave(unsigned ch
     }
 }
 
-template <bool SP> __device__ __forceinline__ void ks_slab_wave(const DfwBwdArgs &p, unsigned char *smem, int64_t b, int m0, int nstages, int lane) {
+// The adjoint chain of 16 key channels: G_start = G_end + g^T Q - dU^T K, one stage ahead of the state waves, to
+// which it hands G_end of every block as a split B operand.  It shares a SIMD with the state wave of the same
+// channels: two independent chains whose instruction streams interleave.
+template <bool SP> __device__ __forceinline__ void ks_adjoint_wave(const DfwBwdArgs &p, unsigned char *smem, int64_t b, int m0, int w, int nstages, int lane) {
+    const int r = lane & 15, g = lane >> 4, m = m0 + r;
+    // G[j][e] = G[d = 16 j + 4 g + e][m]: columns of the state's adjoint
+    floatx4 G[4];
+    {
+        const float *gs = reinterpret_cast<const float *>(p.g_state) + b * CH_N * CH_N + m;
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) G[j][e] = gs[(16 * j + 4 * g + e) * CH_N];
+    }
+    for (int tick = 0; tick < nstages + 2; ++tick) {
+        const int stage = tick - 1;
+        if (stage >= 0 && stage < nstages) {
+            const unsigned char *raw = KsRing::raw(smem, stage, 0);
+            const CmTile<SP> GC(raw + KS_GC), NUC(raw + KS_NUC), KC(raw + KS_KC), QC(raw + KS_QC);
+            const Sp2<SP> kb = KC.tokens(m, g), qb = QC.tokens(m, g);          // K[t = 4g+e][m], Q[t][m]
+            const Sp4<SP> gb0 = cat(split4<SP>(G[0]), split4<SP>(G[1])), gb1 = cat(split4<SP>(G[2]), split4<SP>(G[3]));
+            *xg_piece(smem, stage, w, 0, 0, lane) = gb0.hi;
+            *xg_piece(smem, stage, w, 1, 0, lane) = gb1.hi;
+            if constexpr (SP) {
+                *xg_piece(smem, stage, w, 0, 1, lane) = gb0.lo;
+                *xg_piece(smem, stage, w, 1, 1, lane) = gb1.lo;
+            }
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                G[j] = mma16(GC.tokens(16 * j + r, g), qb, G[j]);
+                G[j] = mma16(NUC.tokens(16 * j + r, g), kb, G[j]);
+            }
+        }
+        __syncthreads();
+    }
+}
+
+// The state chain of 16 key channels, walked backwards (S0 = S_end - Delta^T K), and the block's d_query, d_key.
+template <bool SP> __device__ __forceinline__ void ks_slab_wave(const DfwBwdArgs &p, unsigned char *smem, int64_t b, int m0, int w, int nstages, int lane) {
     const int r = lane & 15, g = lane >> 4, m = m0 + r, T = (int)p.T, nblocks = nstages;
     const floatx4 zero = {0.f, 0.f, 0.f, 0.f};
     float *const d_q = reinterpret_cast<float *>(p.d_q) + b * p.T * CH_N;
     float *const d_k = reinterpret_cast<float *>(p.d_k) + b * p.T * CH_N;
     const u32 lane_off = (u32)(4 * g * CH_N + m);
-    // S[j][e] = S[d = 16 j + 4 g + e][m], G likewise: columns of the state and of its adjoint
-    floatx4 S[4], G[4];
+    // S[j][e] = S[d = 16 j + 4 g + e][m]: columns of the state
+    floatx4 S[4];
     {
         const float *fs = reinterpret_cast<const float *>(p.final_state) + b * CH_N * CH_N + m;
-        const float *gs = reinterpret_cast<const float *>(p.g_state) + b * CH_N * CH_N + m;
 #pragma unroll
         for (int j = 0; j < 4; ++j)
 #pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                S[j][e] = fs[(16 * j + 4 * g + e) * CH_N];
-                G[j][e] = gs[(16 * j + 4 * g + e) * CH_N];
-            }
+            for (int e = 0; e < 4; ++e) S[j][e] = fs[(16 * j + 4 * g + e) * CH_N];
     }
-    // one stage (= one block); FULL as on the value side
+    // one stage (= one block).  FULL: every token of the stage is below T and the body has no branch (see the
+    // value side)
     auto stage_body = [&](auto full, int stage) {
         constexpr bool FULL = decltype(full)::value;
         const int tok0 = reverse_tok0(nblocks, 1, stage, 0);
         const unsigned char *raw = KsRing::raw(smem, stage, 0);
         const unsigned char *st = KsRing::st(smem, stage, 0);
         const TmTile<SP> DT(raw + KS_DT), GT(raw + KS_GT), NUT(raw + KS_NUT);
-        const CmTile<SP> NDC(raw + KS_NDC), GC(raw + KS_GC), NUC(raw + KS_NUC), KC(raw + KS_KC), QC(raw + KS_QC);
+        const CmTile<SP> NDC(raw + KS_NDC), KC(raw + KS_KC), QC(raw + KS_QC);
         const Sp2<SP> kb = KC.tokens(m, g), qb = QC.tokens(m, g);          // K[t = 4g+e][m], Q[t][m]
-        // the adjoint after the block, before it takes the block in
-        const Sp4<SP> gb0 = cat(split4<SP>(G[0]), split4<SP>(G[1])), gb1 = cat(split4<SP>(G[2]), split4<SP>(G[3]));
+        // the adjoint after the block, as the adjoint wave left it one stage ago
+        Sp4<SP> gb0, gb1;
+        gb0.hi = *xg_piece(smem, stage, w, 0, 0, lane);
+        gb1.hi = *xg_piece(smem, stage, w, 1, 0, lane);
+        gb0.lo = SP ? *xg_piece(smem, stage, w, 0, 1, lane) : make_uint4(0u, 0u, 0u, 0u);
+        gb1.lo = SP ? *xg_piece(smem, stage, w, 1, 1, lane) : make_uint4(0u, 0u, 0u, 0u);
         // S0 = S_end - Delta^T K
 #pragma unroll
         for (int j = 0; j < 4; ++j) S[j] = mma16(NDC.tokens(16 * j + r, g), kb, S[j]);
@@ -262,15 +309,9 @@ template <bool SP> __device__ __forceinline__ void ks_slab_wave(const DfwBwdArgs
                 qo[lane_off + e * CH_N] = dq[e];
                 ko[lane_off + e * CH_N] = dk[e];
             }
-        // G_start = G_end + g^T Q - dU^T K
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            G[j] = mma16(GC.tokens(16 * j + r, g), qb, G[j]);
-            G[j] = mma16(NUC.tokens(16 * j + r, g), kb, G[j]);
-        }
         __syncthreads();
     };
-    __syncthreads();        // ticks 0 and 1: the prep and matrix waves fill the pipeline
+    __syncthreads();        // ticks 0 and 1: the prep, matrix and adjoint waves fill the pipeline
     __syncthreads();
     // the blocks are visited last to first: only stage 0 can hold tokens at or past T
     stage_body(std::false_type{}, 0);
@@ -278,8 +319,8 @@ template <bool SP> __device__ __forceinline__ void ks_slab_wave(const DfwBwdArgs
     for (int stage = 1; stage < nstages; ++stage) stage_body(std::true_type{}, stage);
 }
 
-// Waves 0, 1: slab waves (16 key channels each), alone on SIMDs 0 and 1; wave 2: matrix wave; waves 3, 6, 7: prep
-// waves; waves 4, 5 leave at once.
+// Waves 0, 1: state waves (16 key channels each) and waves 4, 5: the adjoint waves of the same channels, on SIMDs 0
+// and 1; wave 2: matrix wave; waves 3, 6, 7: prep waves.
 template <bool SP> __global__ __launch_bounds__(BW_THREADS) void dfw_chunk_bwd_key_kernel(DfwBwdArgs p, int rows_padded) {
     extern __shared__ __align__(16) unsigned char smem[];
     const int half = (int)blockIdx.x >= rows_padded ? 1 : 0;
@@ -295,18 +336,20 @@ template <bool SP> __global__ __launch_bounds__(BW_THREADS) void dfw_chunk_bwd_k
     const float *const dv = reinterpret_cast<const float *>(p.d_v) + row;
     auto tok0_of = [=](int stage, int bb) { return reverse_tok0(nstages, 1, stage, bb); };
     if (wave < 2) {
-        ks_slab_wave<SP>(p, smem, b, 32 * half + 16 * wave, nstages, lane);
+        ks_slab_wave<SP>(p, smem, b, 32 * half + 16 * wave, wave, nstages, lane);
+    } else if (wave == 4 || wave == 5) {
+        ks_adjoint_wave<SP>(p, smem, b, 32 * half + 16 * (wave - 4), wave - 4, nstages, lane);
     } else if (wave == 2) {
         ks_structure_wave<SP>(smem, nstages, lane);
     } else if (wave == 3) {
-        const PrepJob jobs[3] = {{dl, KS_DT, 1.f}, {go, KS_GT, 1.f}, {dv, KS_NUT, -1.f}};
-        prep_wave_jobs<KsRing, 1, false, 3, SP>(smem, jobs, T, nstages, lane, tok0_of);
+        const PrepJob jobs[2] = {{dl, KS_DT, KS_NDC, 1.f, true}, {go, KS_GT, KS_GC, 1.f, false}};
+        prep_wave_jobs<KsRing, 1, 2, SP, 3>(smem, jobs, T, nstages, lane, tok0_of, nullptr);
     } else if (wave == 6) {
-        const PrepJob jobs[3] = {{dl, KS_NDC, -1.f}, {go, KS_GC, 1.f}, {dv, KS_NUC, -1.f}};
-        prep_wave_jobs<KsRing, 1, true, 3, SP>(smem, jobs, T, nstages, lane, tok0_of);
+        const PrepJob jobs[2] = {{dv, KS_NUT, KS_NUC, -1.f, false}, {k, -1, KS_KC, 1.f, false}};
+        prep_wave_jobs<KsRing, 1, 2, SP, 3>(smem, jobs, T, nstages, lane, tok0_of, smem + KS_SCRATCH);
     } else if (wave == 7) {
-        const PrepJob jobs[2] = {{k, KS_KC, 1.f}, {q, KS_QC, 1.f}};
-        prep_wave_jobs<KsRing, 1, true, 2, SP>(smem, jobs, T, nstages, lane, tok0_of);
+        const PrepJob jobs[1] = {{q, -1, KS_QC, 1.f, false}};
+        prep_wave_jobs<KsRing, 1, 1, SP, 3>(smem, jobs, T, nstages, lane, tok0_of, smem + KS_SCRATCH + 2 * TM_TILE);
     }
 }
 
@@ -317,11 +360,11 @@ template <bool SP> static int launch_backward(const DfwBwdArgs &a, hipStream_t s
     auto key_side = dfw_chunk_bwd_key_kernel<SP>;
     int rc = enable_lds(reinterpret_cast<const void *>(value_side), VsRing::SMEM, "hipFuncSetAttribute(delta-rule backward kernel, value side)");
     if (rc) return rc;
-    if ((rc = enable_lds(reinterpret_cast<const void *>(key_side), KsRing::SMEM, "hipFuncSetAttribute(delta-rule backward kernel, key side)"))) return rc;
+    if ((rc = enable_lds(reinterpret_cast<const void *>(key_side), KS_SMEM, "hipFuncSetAttribute(delta-rule backward kernel, key side)"))) return rc;
     const int rows_padded = (int)((a.B + 7) / 8 * 8);
     hipLaunchKernelGGL(value_side, dim3(2u * (unsigned)rows_padded), dim3(BW_THREADS), VsRing::SMEM, stream, a, rows_padded);
     if ((rc = check_hip(hipGetLastError(), "dfw_chunk_bwd_value_kernel launch"))) return rc;
-    hipLaunchKernelGGL(key_side, dim3(2u * (unsigned)rows_padded), dim3(BW_THREADS), KsRing::SMEM, stream, a, rows_padded);
+    hipLaunchKernelGGL(key_side, dim3(2u * (unsigned)rows_padded), dim3(BW_THREADS), KS_SMEM, stream, a, rows_padded);
     return check_hip(hipGetLastError(), "dfw_chunk_bwd_key_kernel launch");
 }
 

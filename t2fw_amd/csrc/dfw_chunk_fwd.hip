@@ -1,13 +1,14 @@
 // Forward pass of the delta rule on the matrix cores, D = M = 64, fp32 tensors (algebra and precision:
 // dfw_chunk.hpp).  Two workgroups per batch row, one per half of the value channels: the rows S[d, :] of the
-// state, and with them the columns of V, Delta and O, never interact.  A workgroup has seven waves:
+// state, and with them the columns of V, Delta and O, never interact.  A workgroup has six waves (eight are launched; two leave at once):
 //   two slab waves    each keeps 16 rows of the state in fp32 accumulators for the whole sequence; per block:
 //                     Delta = Tm V - K' S0^T, O = Q S0^T + Bq Delta, S += Delta^T K; they load V and store O
 //                     and Delta themselves (64 contiguous bytes per token)
 //   two matrix waves  everything that does not depend on the state, one stage ahead of the slab waves, one
 //                     block of the stage each: K K^T and K Q^T, the triangular masks, Tm = (I + A)^-1 by
 //                     squarings, K' = Tm K; they leave Tm^T and Bq^T as ready operands and K' as a tile in LDS
-//   three prep waves  K and Q token-major and K channel-major as bf16 head / remainder tiles, two stages ahead
+//   two prep waves    K (token-major, and channel-major derived from that tile) and Q (token-major) as bf16
+//                     head / remainder tiles, two stages ahead
 // One workgroup barrier per stage of two blocks.
 //
 // Replaces lfw_cuda_fwd_kernel of the reference's delta rule (t2fw/csrc/dfw_kernel.cu:105-196), semantics
@@ -31,53 +32,14 @@ constexpr int FW_RAW = 0;                                        // three stages
 constexpr int FW_ST = FW_RAW + 3 * DNB * FW_RAW_BLOCK;           // two stages of the matrix waves' results
 constexpr int FW_SMEM = FW_ST + 2 * DNB * FW_ST_BLOCK;
 static_assert(FW_SMEM <= 160 * 1024, "forward tiles exceed the LDS of one CU");
+using FwRing = Ring<FW_RAW_BLOCK, FW_ST_BLOCK, DNB>;         // the same layout, for the shared prep-wave routine
+static_assert(FwRing::SMEM == FW_SMEM && FwRing::ST == FW_ST, "ring layout");
 
 __device__ __forceinline__ unsigned char *raw_block(unsigned char *smem, int stage, int bb) {
     return smem + FW_RAW + ((stage % 3) * DNB + bb) * FW_RAW_BLOCK;
 }
 __device__ __forceinline__ unsigned char *st_block(unsigned char *smem, int stage, int bb) {
     return smem + FW_ST + ((stage & 1) * DNB + bb) * FW_ST_BLOCK;
-}
-
-// One array into one kind of tile, for every stage of the sequence, two stages ahead of the slab waves.  The
-// loads of a stage are issued one stage before its tiles are built, into the register set that the stage
-// before last has left: two sets in turn, so that nothing waits for a load in the stage that issued it.
-template <bool CHANNEL_MAJOR, int NARR, bool SP>
-__device__ __forceinline__ void prep_wave(unsigned char *smem, const float *row0, const float *row1, int off0, int off1, int T,
-                                          int nstages, int lane) {
-    Raw16 set_a[NARR][DNB], set_b[NARR][DNB];
-    auto load = [&](Raw16 (&r)[NARR][DNB], int stage) {
-#pragma unroll
-        for (int a = 0; a < NARR; ++a)
-#pragma unroll
-            for (int bb = 0; bb < DNB; ++bb) {
-                const int tok0 = (stage * DNB + bb) * DL;
-                r[a][bb] = CHANNEL_MAJOR ? load_cm(a ? row1 : row0, tok0, T, lane) : load_tm(a ? row1 : row0, tok0, T, lane);
-            }
-    };
-    auto tick_body = [&](int tick, Raw16 (&cur)[NARR][DNB], Raw16 (&nxt)[NARR][DNB]) {
-        load(nxt, min(tick + 1, nstages - 1));          // unconditional: the same loads in flight on every path
-        if (tick < nstages) {
-#pragma unroll
-            for (int a = 0; a < NARR; ++a)
-#pragma unroll
-                for (int bb = 0; bb < DNB; ++bb) {
-                    unsigned char *tile = raw_block(smem, tick, bb) + (a ? off1 : off0);
-                    const int tok0 = (tick * DNB + bb) * DL;
-                    if (CHANNEL_MAJOR)
-                        store_cm<SP>(tile, lane, cur[a][bb], tok0, T);
-                    else
-                        store_tm<SP>(tile, lane, cur[a][bb], tok0, T);
-                }
-        }
-        __syncthreads();
-    };
-    load(set_a, 0);
-    const int nticks = nstages + 2;
-    for (int tick = 0; tick < nticks; tick += 2) {
-        tick_body(tick, set_a, set_b);
-        if (tick + 1 < nticks) tick_body(tick + 1, set_b, set_a);
-    }
 }
 
 // The state-independent part of block `bb` of every stage, one stage ahead of the slab waves.
@@ -219,14 +181,18 @@ template <bool SP> __global__ __launch_bounds__(FW_THREADS) void dfw_chunk_fwd_k
     // leave at once; a workgroup barrier waits only for the waves that are left), the matrix waves and the
     // prep waves share SIMDs 2 and 3.
     static_assert(DNB == 2, "one matrix wave per block of a stage");
+    auto tok0_of = [](int stage, int bb) { return (stage * DNB + bb) * DL; };
     if (wave < 2)
         slab_wave<SP>(p, smem, b, 32 * half + 16 * wave, nstages, lane);
     else if (wave < 4)
         structure_wave<SP>(smem, nstages, wave - 2, lane);
-    else if (wave == 6)
-        prep_wave<false, 2, SP>(smem, k, q, FW_KT, FW_QT, T, nstages, lane);
-    else if (wave == 7)
-        prep_wave<true, 1, SP>(smem, k, k, FW_KC, FW_KC, T, nstages, lane);
+    else if (wave == 6) {          // K: token-major, and channel-major derived from it
+        const PrepJob jobs[1] = {{k, FW_KT, FW_KC, 1.f, false}};
+        prep_wave_jobs<FwRing, DNB, 1, SP, 3>(smem, jobs, T, nstages, lane, tok0_of, nullptr);
+    } else if (wave == 7) {        // Q: token-major
+        const PrepJob jobs[1] = {{q, FW_QT, -1, 1.f, false}};
+        prep_wave_jobs<FwRing, DNB, 1, SP, 3>(smem, jobs, T, nstages, lane, tok0_of, nullptr);
+    }
 }
 
 }  // namespace
