@@ -173,10 +173,9 @@ template <bool SP> __global__ __launch_bounds__(BW_THREADS) void dfw_chunk_bwd_v
 }
 
 // ---- key side -------------------------------------------------------------------------------------------
-// one block per stage: eight raw tiles per block leave no room for more
+// one block per stage; raw tiles per block: Delta, g, -dU token-major, -Delta, K, Q channel-major
 constexpr int KS_DT = 0, KS_GT = KS_DT + 2 * TM_TILE, KS_NUT = KS_GT + 2 * TM_TILE, KS_NDC = KS_NUT + 2 * TM_TILE,
-              KS_GC = KS_NDC + 2 * CM_TILE, KS_NUC = KS_GC + 2 * CM_TILE, KS_KC = KS_NUC + 2 * CM_TILE,
-              KS_QC = KS_KC + 2 * CM_TILE, KS_RAW_BLOCK = KS_QC + 2 * CM_TILE;
+              KS_KC = KS_NDC + 2 * CM_TILE, KS_QC = KS_KC + 2 * CM_TILE, KS_RAW_BLOCK = KS_QC + 2 * CM_TILE;
 constexpr int KS_X1 = 0, KS_X1T = KS_X1 + 2 * ST_TILE, KS_X2S = KS_X1T + 2 * ST_TILE, KS_ST_BLOCK = KS_X2S + 2 * ST_TILE;
 using KsRing = Ring<KS_RAW_BLOCK, KS_ST_BLOCK, 1>;
 // The adjoint waves hand G_end of a block to the state waves as a ready B operand: per (stage parity, wave,
@@ -239,7 +238,10 @@ template <bool SP> __device__ __forceinline__ void ks_adjoint_wave(const DfwBwdA
         const int stage = tick - 1;
         if (stage >= 0 && stage < nstages) {
             const unsigned char *raw = KsRing::raw(smem, stage, 0);
-            const CmTile<SP> GC(raw + KS_GC), NUC(raw + KS_NUC), KC(raw + KS_KC), QC(raw + KS_QC);
+            // g and -dU along the tokens of a value channel come out of the token-major tiles through the transposing
+            // read: this wave has the time for it, the prep waves do not have it for two more derived tiles
+            const TmTile<SP> GT(raw + KS_GT), NUT(raw + KS_NUT);
+            const CmTile<SP> KC(raw + KS_KC), QC(raw + KS_QC);
             const Sp2<SP> kb = KC.tokens(m, g), qb = QC.tokens(m, g);          // K[t = 4g+e][m], Q[t][m]
             const Sp4<SP> gb0 = cat(split4<SP>(G[0]), split4<SP>(G[1])), gb1 = cat(split4<SP>(G[2]), split4<SP>(G[3]));
             *xg_piece(smem, stage, w, 0, 0, lane) = gb0.hi;
@@ -250,8 +252,8 @@ template <bool SP> __device__ __forceinline__ void ks_adjoint_wave(const DfwBwdA
             }
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
-                G[j] = mma16(GC.tokens(16 * j + r, g), qb, G[j]);
-                G[j] = mma16(NUC.tokens(16 * j + r, g), kb, G[j]);
+                G[j] = mma16(GT.column(j, r, g), qb, G[j]);
+                G[j] = mma16(NUT.column(j, r, g), kb, G[j]);
             }
         }
         __syncthreads();
@@ -342,14 +344,14 @@ template <bool SP> __global__ __launch_bounds__(BW_THREADS) void dfw_chunk_bwd_k
     } else if (wave == 2) {
         ks_structure_wave<SP>(smem, nstages, lane);
     } else if (wave == 3) {
-        const PrepJob jobs[2] = {{dl, KS_DT, KS_NDC, 1.f, true}, {go, KS_GT, KS_GC, 1.f, false}};
-        prep_wave_jobs<KsRing, 1, 2, SP, 3>(smem, jobs, T, nstages, lane, tok0_of, nullptr);
+        const PrepJob jobs[1] = {{dl, KS_DT, KS_NDC, 1.f, true}};
+        prep_wave_jobs<KsRing, 1, 1, SP, 3>(smem, jobs, T, nstages, lane, tok0_of, nullptr);
     } else if (wave == 6) {
-        const PrepJob jobs[2] = {{dv, KS_NUT, KS_NUC, -1.f, false}, {k, -1, KS_KC, 1.f, false}};
+        const PrepJob jobs[2] = {{go, KS_GT, -1, 1.f, false}, {k, -1, KS_KC, 1.f, false}};
         prep_wave_jobs<KsRing, 1, 2, SP, 3>(smem, jobs, T, nstages, lane, tok0_of, smem + KS_SCRATCH);
     } else if (wave == 7) {
-        const PrepJob jobs[1] = {{q, -1, KS_QC, 1.f, false}};
-        prep_wave_jobs<KsRing, 1, 1, SP, 3>(smem, jobs, T, nstages, lane, tok0_of, smem + KS_SCRATCH + 2 * TM_TILE);
+        const PrepJob jobs[2] = {{dv, KS_NUT, -1, -1.f, false}, {q, -1, KS_QC, 1.f, false}};
+        prep_wave_jobs<KsRing, 1, 2, SP, 3>(smem, jobs, T, nstages, lane, tok0_of, smem + KS_SCRATCH + 2 * TM_TILE);
     }
 }
 
