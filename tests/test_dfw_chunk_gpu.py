@@ -68,6 +68,23 @@ def test_unnormalised_keys(scale):
     check(2, 200, seed=300, key_scale=scale)
 
 
+def test_long_sequence():
+    """T = 2050: 65 stages of the forward, 129 of the key side, a partial last block"""
+    check(2, 2050, seed=77)
+
+
+def test_large_values_and_states():
+    """values of size 100 and a state of size 50: the relative accuracy of the split operands does not depend on scale"""
+    q, k, v, s, go, gs = make_inputs(3, 130, 64, 64, torch.float32, seed=31)
+    v, s = v * 100.0, s * 50.0
+    r_out, r_fin, r_grads = dfw_reference_grads(q, k, v, s, go, gs)
+    out, fin, delta, grads = run_abi(q, k, v, s, go, gs)
+    assert_close(out, r_out, torch.float32, "outputs", tol=TOL)
+    assert_close(fin, r_fin, torch.float32, "final_state", tol=TOL)
+    for n, g, r in zip(NAMES, grads, r_grads):
+        assert_close(g, r, torch.float32, n, tol=TOL)
+
+
 def test_headline_shape_rows_against_the_oracle():
     """B = 96, T = 1024 as the benchmark runs it; the oracle on three rows"""
     q, k, v, s, go, gs = make_inputs(96, 1024, 64, 64, torch.float32, seed=5)
