@@ -551,6 +551,29 @@ def bench_float32(args, steps, warmup):
         torch.cuda.synchronize()
         ms = (time.perf_counter() - t0) / n * 1e3
         out[name] = {"value": round(B * T / ms / 1e3, 1), "unit": "Mtokens/s", "ms_per_step": round(ms, 5), "steps": n}
+    # the cast path recorded once into a HIP graph and replayed: its GPU time without the host's share
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        run(lfw_apply_16bit, 1)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    for t in leaves:
+        t.grad = None
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        o, nx = lfw_apply_16bit(*leaves)
+        torch.autograd.backward([o, nx], [go, gs])
+    for _ in range(3):
+        graph.replay()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        graph.replay()
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) / steps * 1e3
+    out["cast_to_float16"]["graph_replay_ms_per_step"] = round(ms, 5)
+    out["cast_to_float16"]["graph_replay_value"] = round(B * T / ms / 1e3, 1)
     names = ["outputs", "next_state", "d_x", "d_f", "d_q", "d_k", "d_f_key", "d_state"]
     worst = max(((a - b).abs().max() / b.abs().max()).item() for a, b in zip(results["cast_to_float16"], results["exact_float32"]))
     out["cast_to_float16"]["max_abs_over_max_ref_vs_exact_float32"] = round(worst, 6)
