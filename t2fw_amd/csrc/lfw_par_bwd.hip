@@ -491,12 +491,18 @@ template <typename IOE, int NT, bool HEADS, bool FULL> struct GradsItem {
     template <int SIDE> __device__ __forceinline__ void run_side() const {
         SideState<NT> st;
         {
+            // The row's verdict (second launch) is fetched with the inputs and looked at once they are in (a branch
+            // before that would have the compiler move the input loads behind it).  A row that the form cannot take
+            // is left alone from there on: the launch that follows redoes it whole, and under T2FW_FLAG_NO_FIXUP
+            // its results are declared invalid anyway.  The branch is uniform over the workgroup.
+            const int declined = p.row_flags[item / NC];
             Raw r;
             MatRegs mr;
             issue_raw<SIDE>(r);
             issue_mats(mr);
             prep<SIDE>(st, r);
             stage_mats(mr);
+            if (__builtin_amdgcn_readfirstlane(declined)) return;
         }
         __syncthreads();                         // tiles, S0', Gh' complete
         products<SIDE>();
