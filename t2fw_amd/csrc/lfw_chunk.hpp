@@ -94,6 +94,11 @@ struct Bf16 {
     static constexpr u16 ONE_BITS = 0x3F80;
     static constexpr u16 FLOOR_BITS = 0x3380;        // 2^-24: gates enter the forward's products no smaller
     static constexpr u16 BWD_FLOOR_BITS = 0x3980;    // 2^-12: ... and the chunk-parallel backward's
+    // As the tensors' type: results of size 2^28 and more are representable, which is where an intermediate of the
+    // matrix-core forms (the result times up to 1 / product) can leave fp32: the kernels then look at what they
+    // store and hand rows with an inf or NaN to the exact recurrence.  With fp16 tensors such a result is beyond
+    // the type anyway, and no operand can overflow (values up to 2^16, 1 / product up to 2^100).
+    static constexpr bool CHECK_RESULTS = true;
     // smallest 16-step gate product accepted with operands of this type: the inverse
     // 1/product scales the intra-block operands and must stay far from overflow
     static constexpr float MIN_PRODUCT = 7.8886090522101181e-31f;   // 2^-100
@@ -120,6 +125,7 @@ struct Fp16 {
     static constexpr u16 ONE_BITS = 0x3C00;
     static constexpr u16 FLOOR_BITS = 0x0001;        // 2^-24, the smallest positive fp16
     static constexpr u16 BWD_FLOOR_BITS = 0x0C00;    // 2^-12
+    static constexpr bool CHECK_RESULTS = false;     // see Bf16
     static constexpr float MIN_PRODUCT = 0.00390625f;               // 2^-8
     static __device__ __forceinline__ float to_f32(u16 v) { return (float)__builtin_bit_cast(_Float16, v); }
     // products of raw 16-bit values (a fused form with fp16 operands converted on the fly exists,

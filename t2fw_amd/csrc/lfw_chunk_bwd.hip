@@ -537,6 +537,7 @@ __device__ __forceinline__ void bwd_matrix_waves(const ChunkBwdArgs &p, unsigned
     take_state(pf, G);
     load_state(ckpt + (NC - 1) * (CH_N * CH_N), pf);
     float carry = 0.f;
+    float chk = 0.f;         // 0 until a stored result is inf or NaN, then NaN
     int s = 0;
     if (tid == 0) {      // both flag slots of the row (the backward kernels report in the first)
         p.row_flags[b] = 0;
@@ -649,9 +650,15 @@ __device__ __forceinline__ void bwd_matrix_waves(const ChunkBwdArgs &p, unsigned
                     // one address per array; the four tokens are immediate offsets from it (folded rows)
                     u16 *const pv = d_val + go, *const pg = d_gate + go, *const pa = d_adj + go;
                     auto store = [&](int ii) {
-                        pv[ii * ts] = cvt1<IOE>(ipv[ii] * (va[ii] + asv[ii] * pd[ii]));
-                        pg[ii * ts] = cvt1<IOE>(du[ii] * rgv[ii]);
-                        if (side == 1) pa[ii * ts] = cvt1<IOE>(ppv[ii] * (oa[ii] + vtv[ii] * pd[ii]));
+                        const float rv = ipv[ii] * (va[ii] + asv[ii] * pd[ii]), rg = du[ii] * rgv[ii];
+                        if constexpr (IOE::CHECK_RESULTS) chk = __builtin_fmaf(rv, 0.0f, __builtin_fmaf(rg, 0.0f, chk));
+                        pv[ii * ts] = cvt1<IOE>(rv);
+                        pg[ii * ts] = cvt1<IOE>(rg);
+                        if (side == 1) {
+                            const float ra = ppv[ii] * (oa[ii] + vtv[ii] * pd[ii]);
+                            if constexpr (IOE::CHECK_RESULTS) chk = __builtin_fmaf(ra, 0.0f, chk);
+                            pa[ii * ts] = cvt1<IOE>(ra);
+                        }
                     };
                     if ((int)chunk * C + (i + 1) * CH_L <= T) {
 #pragma unroll
@@ -751,6 +758,18 @@ __device__ __forceinline__ void bwd_matrix_waves(const ChunkBwdArgs &p, unsigned
         u16 *ds = reinterpret_cast<u16 *>(p.d_s0) + b * (CH_N * CH_N);
 #pragma unroll
         for (int j = 0; j < 4; ++j) *reinterpret_cast<uint2 *>(ds + ch * CH_N + 16 * j + 4 * g) = pack4v<IOE>(G[j]);
+    }
+    // A result that is not finite (a scaled operand or a product of scaled operands left the range of its type)
+    // hands this side of the row to the exact recurrence, like a gate outside the range does.
+    if constexpr (IOE::CHECK_RESULTS) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) chk = __builtin_fmaf(G[j][i], 0.0f, chk);
+    }
+    if (!(chk == 0.0f)) {
+        p.row_flags[b] = 1;
+        *reinterpret_cast<volatile int *>(smem + OFF_VERDICT) = 1;
     }
 }
 

@@ -386,6 +386,7 @@ __device__ __forceinline__ void fwd_matrix_waves(const ChunkFwdArgs &p, unsigned
     }
     int until_ckpt = 0;
     int64_t chunk = 0;
+    float omax = 0.f;
     if (tid == 0) {
         p.row_flags[flag_slot] = 0;
         if (clear_other_slot) p.row_flags[chunk_rows_padded(p.B) + b] = 0;
@@ -446,13 +447,19 @@ __device__ __forceinline__ void fwd_matrix_waves(const ChunkFwdArgs &p, unsigned
             // 16 lanes write 32 contiguous bytes of a token row; the four waves complete the row
             const int tg = n * CH_STEP + tok0 + 4 * g;
             u16 *const po = out + ((u32)tg * ts + (u32)d);      // the four tokens: immediate offsets (folded rows)
+            float res[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                res[i] = (o[i] + oi[i]) * asv[i];
+                if constexpr (IOE::CHECK_RESULTS) omax = __builtin_fmaf(res[i], 0.0f, omax);        // 0 until a result is inf or NaN, then NaN
+            }
             if constexpr (FULL) {
 #pragma unroll
-                for (int i = 0; i < 4; ++i) po[i * ts] = cvt1<IOE>((o[i] + oi[i]) * asv[i]);
+                for (int i = 0; i < 4; ++i) po[i * ts] = cvt1<IOE>(res[i]);
             } else {
 #pragma unroll
                 for (int i = 0; i < 4; ++i)
-                    if (tg + i < T) po[i * ts] = cvt1<IOE>((o[i] + oi[i]) * asv[i]);
+                    if (tg + i < T) po[i * ts] = cvt1<IOE>(res[i]);
             }
             // S_L = (a_L (x) b_L) * S0 + sum_s xh_s (x) kh_s
             const float aL = AL[hh * CH_N + d];
@@ -482,6 +489,19 @@ __device__ __forceinline__ void fwd_matrix_waves(const ChunkFwdArgs &p, unsigned
             step(nfull, std::false_type{}, std::true_type{});
     }
     store_state<IOE>(S, reinterpret_cast<u16 *>(p.next_state) + b * (CH_N * CH_N), d, g);
+    // A result that is not finite (an operand scaled by 1 / product left the range of its type, or a product of
+    // scaled operands that of fp32) hands the row to the exact recurrence like a gate outside the range does.
+    if constexpr (IOE::CHECK_RESULTS) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) omax = __builtin_fmaf(S[j][i], 0.0f, omax);
+    }
+    if (!(omax == 0.0f)) {
+        p.row_flags[flag_slot] = 1;
+        *reinterpret_cast<volatile int *>(smem + OFF_VERDICT) = 1;
+        if (p.par_hint != nullptr) p.par_hint[flag_slot] = 1;
+    }
 }
 
 // End of a workgroup's work on its (part of a) batch row.  A barrier publishes the prep waves'

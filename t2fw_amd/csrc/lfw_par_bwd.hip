@@ -360,6 +360,7 @@ template <typename IOE, int NT, bool HEADS, bool FULL> struct GradsItem {
         float du[NT][4];
         float anchor_acc;                        // sum_t adjS_t * (S0' adj-op_t)
         float anchor, carry;                     // gate gradient: see begin_gate_gradient
+        float chk;                               // 0 until a stored result is inf or NaN, then NaN
 
         __device__ __forceinline__ Sweep(const GradsItem &g_, const SideState<NT> &st_) : g(g_), st(st_) {
             own_adj = g.template tile_adj<SIDE>(); own_val = g.template tile_val<SIDE>();
@@ -371,6 +372,7 @@ template <typename IOE, int NT, bool HEADS, bool FULL> struct GradsItem {
             d_gate = reinterpret_cast<u16 *>(SIDE ? g.p.d_f_key : g.p.d_f) + g.chunk_off;
             d_adj = reinterpret_cast<u16 *>(g.p.d_q) + g.chunk_off;          // key side only
             anchor_acc = 0.f;
+            chk = 0.f;
         }
         // operands of the own side (this lane's channel, tokens 16 m + 4 kg + j), re-read from the own tiles
         __device__ __forceinline__ uint2 b_val(int m) const { return ld2(own_val + g.c * CMS + 16 * m + 4 * g.kg); }
@@ -380,10 +382,12 @@ template <typename IOE, int NT, bool HEADS, bool FULL> struct GradsItem {
             const u16 *mt = reinterpret_cast<const u16 *>(g.smem + region);
             return SIDE ? mat_cols_op(mt, 16 * g.cb, h, g.i, g.kg) : mat_rows_op(mt, 16 * g.cb, h, g.i, g.kg);
         }
-        __device__ __forceinline__ void store4(u16 *dst, int mm, const float (&v)[4]) const {
+        __device__ __forceinline__ void store4(u16 *dst, int mm, const float (&v)[4]) {
 #pragma unroll
-            for (int j = 0; j < 4; ++j)
+            for (int j = 0; j < 4; ++j) {
+                if constexpr (IOE::CHECK_RESULTS) chk = __builtin_fmaf(v[j], 0.0f, chk);
                 if (FULL || 16 * mm + j < g.n_left) (dst + (size_t)(16 * mm + j) * g.ts)[g.lane_off] = cvt1<IOE>(v[j]);
+            }
         }
         // forward-like sweep, token tile m: o' (value side) / q' (key side)
         __device__ __forceinline__ void forward_tile(int m, const uint4 &s0a, const uint4 &s0b) {
@@ -486,6 +490,9 @@ template <typename IOE, int NT, bool HEADS, bool FULL> struct GradsItem {
                 w.backward_tile(n, gha, ghb);
             }
         }
+        // A result that is not finite (a scaled operand or a product of scaled operands left the range of its
+        // type) declines the row after the fact: the launch that follows redoes it.
+        if (!(w.chk == 0.0f)) p.row_flags[item / NC] = 1;
     }
 
     template <int SIDE> __device__ __forceinline__ void run_side() const {
