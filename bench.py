@@ -5,27 +5,32 @@ A "step" is one forward + backward pass of the decay-rule recurrence over one ba
 synthetic input already resident in HBM, at the headline configuration
 (B*H=96, T=1024, D=K=64, fp16 I/O, checkpoint interval 64).  Prints ONE JSON line.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg3|cfg3_heads|cfg2|cfg4|cfg5|dfw|copy256|copy64]
-                    [--no-cpu-baseline]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg3|cfg3_heads|cfg3_refgates|cfg2|cfg4|cfg5|dfw|copy256|copy64]
+                    [--no-cpu-baseline] [--no-other-configs] [--force-scan] [--dfw-bf16-operands]
 
 value      = B*T*steps / wall time of the timed region, in Mtokens/s (token = one
              (batch row, time step) pair), driving the C ABI directly with preallocated
              outputs; `autograd_api` repeats it through LFWFunction.apply + backward.
-roofline   = algorithmic bytes of the dominant call (the backward: three launches, named in
-             `launches`) / its mean duration measured with events on the launch stream (the call is
-             repeated with the flag that skips the launch for flagged rows that follows them, so
-             that the events bracket those kernels; `call_with_fixup_launch_ms` is the call as
-             shipped), against 8 TB/s.  `traffic` = measured HBM bytes of the same launches, from
-             profiles/traffic_<workload>.json (rocprofv3 counters).
+roofline   = algorithmic bytes of the dominant call (the backward: four launches, named in
+             `launches`) / its mean duration as shipped (flags 0), measured with events on the launch
+             stream; `launch_ms` gives the median and the 20th / 80th percentile of the same calls;
+             `backward_no_fixup_ms` / `frac_no_fixup` are the call a caller makes that holds the
+             forward's all-zero hints (it leaves the fourth launch out).  `traffic` = HBM bytes of the
+             same launches from profiles/traffic_<workload>.json (rocprofv3 counters, not measured in
+             this run: `traffic_source` says so).  Against 8 TB/s.
+other_configs = after the headline's timed region (cfg3 only): cfg2, cfg4, cfg3 with the gates of the
+             reference's tests, cfg5, the delta rule (default and single-operand mode) and cfg3's shape
+             with float32 tensors, each briefly.
 dfw        = the delta-rule kernels (forward + backward) at cfg3's shape in fp32, the dtype the
-             reference tests them in.
+             reference tests them in (--dfw-bf16-operands: their opt-in single-operand mode).
 copy256    = calibration workload for those counters: a 256 MiB device-to-device copy.
 copy64     = the same copy at 64 MiB: source and destination together stay inside the 256 MB of last-level cache.
 cpu_baseline = the TorchScript restatement of the reference loop (oracle/), fp32,
              forward + autograd backward, timed on this host's cores on a bounded sample.
 parity     = computed in the same CPU leg: per tensor, the GPU results of the first three rows of
              input set 0 against the float64 oracle on the same quantised inputs (max-abs error,
-             max-abs error / max|reference|, mean relative error).
+             max-abs error / max|reference|, mean relative error), and beside each the error of the
+             reference's own arithmetic (its recurrence evaluated in the tensors' dtype on the CPU).
 """
 import argparse
 import json
