@@ -562,7 +562,12 @@ __device__ __forceinline__ void bwd_matrix_waves(const ChunkBwdArgs &p, unsigned
                     d[0] = cat(a0, a1);
                     d[1] = cat(a2, a3);
                 }
-                const float lo = LO[ch];
+                // (the index is made opaque so that the byte offset is formed here, from the channel, instead of
+                // living in a register of its own across the stages: at this kernel's register limit that register
+                // is spilled, and its reload after the gradient stores makes the wave wait for those stores)
+                int ch_here = ch;
+                asm volatile("" : "+v"(ch_here));
+                const float lo = LO[ch_here];
                 const uint2 vhc = ld2(VHc + ch * CC + 4 * g);
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
@@ -606,7 +611,12 @@ __device__ __forceinline__ void bwd_matrix_waves(const ChunkBwdArgs &p, unsigned
                 }
                 const uint2 pa_o = pack4v<OPE>(pt1), pa_v = pack4v<OPE>(pt2);
                 const uint2 vtc = ld2(VTc + ch * CC + 4 * g), asc = ld2(ASc + ch * CC + 4 * g);
-                const float lo = LO[ch];
+                // (the index is made opaque so that the byte offset is formed here, from the channel, instead of
+                // living in a register of its own across the stages: at this kernel's register limit that register
+                // is spilled, and its reload after the gradient stores makes the wave wait for those stores)
+                int ch_here = ch;
+                asm volatile("" : "+v"(ch_here));
+                const float lo = LO[ch_here];
                 const int po = r * TS + 16 * g;
                 // o' uses the block-start state
                 floatx4 oa = OPE::mfma32(ld4(AOS + po + 8), sb1, OPE::mfma32(ld4(AOS + po), sb0, zero));
