@@ -14,7 +14,11 @@
 // both halves of every chunk to stay above PAR_MIN_PRODUCT (operands are bf16, which has the exponent
 // range of fp32) and gates in (0, 1].  Rows that violate this are flagged and redone with the exact
 // scan.  The state and the adjoint enter the products scaled to the same reference:
-// S0' = (a_mid (x) b_mid) * S0 and Gh' = (a_CL/a_mid (x) b_CL/b_mid) * Ge, all factors <= 1.
+// S0' = (a_mid (x) b_mid) * S0 and Gh' = (a_CL/a_mid (x) b_CL/b_mid) * Ge, all factors <= 1.  These two
+// carry the half-chunk products of BOTH sides, down to PAR_MIN_PRODUCT^2 = 2^-160, which no 32-bit
+// exponent holds, while what they are multiplied with carries the inverse of one side's product: they
+// are stored times PAR_STATE_SHIFT, and the contractions with them are multiplied by PAR_STATE_UNSHIFT
+// before anything else is added.
 //
 // Lane layout ("C layout"): a workgroup has 8 waves = (side, channel block cb); side 0 owns the value
 // side (x, f, g_out), side 1 the key side (k, f_key, q).  Lane (i = lane & 15, kg = lane >> 4) of
@@ -64,6 +68,13 @@ constexpr int CM_BYTES = CH_N * CMS * 2;
 // smallest chunk gate product this form accepts: 1 / product scales operands that are then
 // multiplied by values and summed in fp32, which has to stay far below 2^128
 constexpr float PAR_MIN_PRODUCT = 8.271806125530277e-25f;     // 2^-80
+// S0' and Gh' are stored times 2^44: an element of magnitude 2^-10 under two half-chunk products of 2^-80
+// is still a normal bf16 number (2^-126), and the one contraction of S0' with Gh' (both shifted, 64
+// terms) stays finite up to |S0| |Ge| = 2^34, beyond what two fp16 tensors can hold.  The factor goes
+// onto one side's product before the other side's is multiplied in, so that no intermediate leaves
+// the range either.
+constexpr float PAR_STATE_SHIFT = 17592186044416.0f;          // 2^44
+constexpr float PAR_STATE_UNSHIFT = 5.684341886080802e-14f;   // 2^-44
 
 typedef __attribute__((address_space(3))) short4_t *lds_short4_ptr;
 
@@ -131,21 +142,12 @@ __device__ __forceinline__ RowScan row_scan_add(float v, int kg) {
 // ---- one lane's share of a chunk of one side ------------------------------------------------------
 // NT = CL / 16 token tiles; element [m][j] is token 16 m + 4 kg + j of the chunk.
 template <int NT> struct LaneChunk {
-    float pre[NT][4];     // gate products from the chunk start up to and including the token
+    float pre[NT][4];     // gate products from the origin up to and including the token
     float off[NT];        // gate product up to the token before [m][0]
     float tot;            // the whole chunk's gate product (the same in every lane of the channel)
     float ref;            // the product of the first half of the chunk (tokens 0 .. CL / 2 - 1)
     float sfx;            // the product of the second half
     u32 bad;              // a gate outside (0, 1] or a half-chunk product below PAR_MIN_PRODUCT
-    // rescale pre and off
-    __device__ __forceinline__ void scale_by(float r) {
-#pragma unroll
-        for (int m = 0; m < NT; ++m) {
-            off[m] *= r;
-#pragma unroll
-            for (int j = 0; j < 4; ++j) pre[m][j] *= r;
-        }
-    }
 };
 
 // Raw 16-bit loads of one array: this lane's NT * 4 tokens of channel c, two tokens per register
@@ -192,6 +194,12 @@ __device__ __forceinline__ void load_tokens(RawTokens<NT> &r, const u16 *ubase, 
 // Gates -> prefix products (and the range verdict).  FULL = false: tokens at or past n_left act as
 // identity (gate 1).
 //
+// Origin of pre and off: the chunk start (MID = false), or the middle of the chunk (MID = true), that
+// is pre = a_t / a_mid, from 1 / ref down to 1 over the first half and from 1 down to sfx over the
+// second.  The second half's products are then built from 1 at the middle, not from the chunk start and
+// divided: the product of both halves may lie far below the smallest fp32 number while each half is in
+// range.
+//
 // Gates below 2^-12 (an exactly zero gate above all, which an fp16 sigmoid returns below a logit of
 // about -17) enter as 2^-12.  The forward's state after such a step holds at most 2^-24 of what was there
 // before it; here 2^-12 of it leaks through, 2.4e-4 of a term that the operands' bf16 rounding already
@@ -200,7 +208,7 @@ __device__ __forceinline__ void load_tokens(RawTokens<NT> &r, const u16 *ubase, 
 // terms that cancel in it, and d_gate = that / gate with the floored gate is then good to 2^-12 of those
 // terms.  (d_gate at a step does not depend on the step's own gate, so the floored gate gives the right
 // value.)
-template <typename IOE, int NT, bool FULL>
+template <typename IOE, int NT, bool FULL, bool MID>
 __device__ __forceinline__ void gate_scan(LaneChunk<NT> &lc, float (&gate)[NT][4], const RawTokens<NT> &raw, int kg,
                                           int n_left) {
     us2 mx = {0, 0};
@@ -229,13 +237,25 @@ __device__ __forceinline__ void gate_scan(LaneChunk<NT> &lc, float (&gate)[NT][4
         const RowScan s = row_scan_mul(l[3], kg);
         lc.off[m] = carry * s.lower;
         carry *= s.all;
-        if (m == NT / 2 - 1) lc.ref = carry;
+        if (m == NT / 2 - 1) {
+            lc.ref = carry;
+            if (MID) carry = 1.0f;
+        }
         if (m >= NT / 2) second *= s.all;
 #pragma unroll
         for (int j = 0; j < 4; ++j) lc.pre[m][j] = lc.off[m] * l[j];
     }
-    lc.tot = carry;
+    lc.tot = MID ? lc.ref * second : carry;
     lc.sfx = second;
+    if (MID) {
+        const float r = __builtin_amdgcn_rcpf(lc.ref);
+#pragma unroll
+        for (int m = 0; m < NT / 2; ++m) {
+            lc.off[m] *= r;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) lc.pre[m][j] *= r;
+        }
+    }
     const u16 hi = mx.x > mx.y ? mx.x : mx.y;
     lc.bad = (hi > IOE::ONE_BITS || !(lc.ref >= PAR_MIN_PRODUCT) || !(second >= PAR_MIN_PRODUCT)) ? 1u : 0u;
 }

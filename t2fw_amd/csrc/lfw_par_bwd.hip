@@ -68,12 +68,12 @@ __global__ __launch_bounds__(PAR_THREADS) void lfw_par_incr_kernel(ParBwdArgs p)
         if (chunk * CL + CL <= T) {
             load_tokens<NT, true>(rg, gate, lane_off, ts, n_left);
             load_tokens<NT, true>(ra, adj, lane_off, ts, n_left);
-            gate_scan<IOE, NT, true>(lc, gt, rg, kg, n_left);
+            gate_scan<IOE, NT, true, false>(lc, gt, rg, kg, n_left);
             to_floats<IOE, NT, true>(av, ra, n_left);
         } else {
             load_tokens<NT, false>(rg, gate, lane_off, ts, n_left);
             load_tokens<NT, false>(ra, adj, lane_off, ts, n_left);
-            gate_scan<IOE, NT, false>(lc, gt, rg, kg, n_left);
+            gate_scan<IOE, NT, false, false>(lc, gt, rg, kg, n_left);
             to_floats<IOE, NT, false>(av, ra, n_left);
         }
         bad = lc.bad;
@@ -165,7 +165,7 @@ template <typename IOE> __global__ __launch_bounds__(SCAN_TPB) void lfw_par_scan
 #pragma unroll
         for (int u = 0; u < SCAN_BATCH; ++u) {
             const float *v = vl + u * SCAN_VEC;
-            const float ta = v[dl], sa = v[8 + dl];
+            const float ta = v[dl], sa = v[8 + dl] * PAR_STATE_SHIFT;      // Gh' is stored shifted
             const float2 tb = *reinterpret_cast<const float2 *>(v + 16 + k), sb = *reinterpret_cast<const float2 *>(v + 16 + CH_N + k);
             tau0[u] = ta * tb.x; tau1[u] = ta * tb.y;
             sig0[u] = sa * sb.x; sig1[u] = sa * sb.y;
@@ -257,8 +257,7 @@ template <typename IOE, int NT, bool HEADS, bool FULL> struct GradsItem {
     // phase A of one side: gate products relative to the middle of the chunk, scaled operands -> tiles
     template <int SIDE> __device__ __forceinline__ void prep(SideState<NT> &st, const Raw &r) const {
         float gt[NT][4], fv[NT][4], fa[NT][4];
-        gate_scan<IOE, NT, FULL>(st.lc, gt, r.g, kg, n_left);
-        st.lc.scale_by(__builtin_amdgcn_rcpf(st.lc.ref));      // the products up to the middle of the chunk divide out
+        gate_scan<IOE, NT, FULL, true>(st.lc, gt, r.g, kg, n_left);      // products relative to the middle of the chunk
         to_floats<IOE, NT, FULL>(fv, r.v, n_left);
         to_floats<IOE, NT, FULL>(fa, r.a, n_left);
         // 1 / pre lives only here: the sweeps take the reciprocals again where they use them, which costs four
@@ -289,11 +288,12 @@ template <typename IOE, int NT, bool HEADS, bool FULL> struct GradsItem {
     __device__ __forceinline__ void stage_mats(const MatRegs &r) const {
         const float rbv[8] = {r.rb[0].x, r.rb[0].y, r.rb[0].z, r.rb[0].w, r.rb[1].x, r.rb[1].y, r.rb[1].z, r.rb[1].w};
         const u32 sw[4] = {r.s0.x, r.s0.y, r.s0.z, r.s0.w};
+        const float ras = r.ra * PAR_STATE_SHIFT;                 // S0' is stored shifted
         float v[8];
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
-            v[2 * e] = IOE::to_f32((u16)(sw[e] & 0xffffu)) * (r.ra * rbv[2 * e]);
-            v[2 * e + 1] = IOE::to_f32((u16)(sw[e] >> 16)) * (r.ra * rbv[2 * e + 1]);
+            v[2 * e] = IOE::to_f32((u16)(sw[e] & 0xffffu)) * (ras * rbv[2 * e]);
+            v[2 * e + 1] = IOE::to_f32((u16)(sw[e] >> 16)) * (ras * rbv[2 * e + 1]);
         }
         const int o = (tid >> 3) * CMS + (tid & 7) * 8;
         *reinterpret_cast<uint4 *>(reinterpret_cast<u16 *>(smem + GR_S0) + o) =
@@ -395,6 +395,8 @@ template <typename IOE, int NT, bool HEADS, bool FULL> struct GradsItem {
             const uint2 none = make_uint2(0u, 0u);
             const uint4 a0 = tok_rows_op(oth_adj, 16 * m, 0, g.i, g.kg), a1 = tok_rows_op(oth_adj, 16 * m, 1, g.i, g.kg);
             floatx4 acc = Bf16::mfma32(a1, s0b, Bf16::mfma32(a0, s0a, zero));
+#pragma unroll
+            for (int j = 0; j < 4; ++j) acc[j] *= PAR_STATE_UNSHIFT;
             float af[4];
             unpack4<Bf16>(b_adj(m), af);
 #pragma unroll
@@ -427,6 +429,8 @@ template <typename IOE, int NT, bool HEADS, bool FULL> struct GradsItem {
             const uint2 none = make_uint2(0u, 0u);
             const uint4 v0 = tok_rows_op(oth_val, 16 * n, 0, g.i, g.kg), v1 = tok_rows_op(oth_val, 16 * n, 1, g.i, g.kg);
             floatx4 acc = Bf16::mfma32(v1, ghb, Bf16::mfma32(v0, gha, zero));
+#pragma unroll
+            for (int j = 0; j < 4; ++j) acc[j] *= PAR_STATE_UNSHIFT;
 #pragma unroll
             for (int m0 = n; m0 < NT; m0 += 2)
                 acc = Bf16::mfma32(cat(g.template bw_read<SIDE>(m0, n), m0 + 1 < NT ? g.template bw_read<SIDE>(m0 + 1, n) : none),
@@ -464,7 +468,7 @@ template <typename IOE, int NT, bool HEADS, bool FULL> struct GradsItem {
             const floatx4 d = Bf16::mfma32(ghb, s0b, Bf16::mfma32(gha, s0a, zero));
             const int jj = g.i & 3;
             const float sel = jj == 0 ? d[0] : (jj == 1 ? d[1] : (jj == 2 ? d[2] : d[3]));      // element (i, i), held by row i / 4
-            return __shfl(sel, 16 * (g.i >> 2) + g.i, 64);
+            return __shfl(sel, 16 * (g.i >> 2) + g.i, 64) * (PAR_STATE_UNSHIFT * PAR_STATE_UNSHIFT);
         }
     };
 

@@ -116,6 +116,45 @@ def test_small_gates_across_a_half_chunk_boundary_are_accepted():
     check_against_oracle((x, f, q, k, fk, s), go, gs, C, torch.float16, expect_flagged=0, gate_tol=(2e-1, 4e-2))
 
 
+@pytest.mark.parametrize("C", [32, 64])
+@pytest.mark.parametrize("where", ["first_half", "second_half", "both_halves"])
+def test_small_gate_products_on_both_sides_at_once(where, C):
+    """Every channel of BOTH gates decays by 2^-76 over half a chunk: inside the accepted range on
+    either side, while the state entering the chunk and the adjoint entering it from the future are
+    scaled by the product of the two sides, 2^-152, which no 32-bit exponent holds unshifted.  The
+    half's first token keeps gates of one, so that d_q, d_f and d_f_key there see the whole entering
+    state; the chunk's last token always sees the whole adjoint from beyond the chunk (d_x, d_k)."""
+    B, T, h = 3, 3 * C, C // 2
+    x, f, q, k, fk, s, go, gs = make_config_inputs(B, T, 64, 64, torch.float16, seed=53 + C, gate_mean=3.0,
+                                                    state_std=0.5)
+    f, fk = f.clone(), fk.clone()
+    small_first = 2.0 ** (-76.0 / (h - 1))       # h - 1 steps after a first step of one
+    small_second = 2.0 ** (-76.0 / h)
+    for b, c0 in ((0, 0), (1, C), (2, 2 * C)):       # row b: chunk b
+        if where != "second_half":
+            for g in (f, fk):
+                g[b, c0] = 1.0
+                g[b, c0 + 1:c0 + h] = small_first
+        if where != "first_half":
+            for g in (f, fk):
+                g[b, c0 + h:c0 + C] = small_second
+    check_against_oracle((x, f, q, k, fk, s), go, gs, C, torch.float16, expect_flagged=0, gate_tol=(2e-1, 4e-2),
+                         reference_bounds=False)
+    # the tokens named above, on their own scale
+    out, nxt, ckpt, grads, flagged = run_abi((x, f, q, k, fk, s), go, gs, C)
+    r_grads = c_oracle.lfw_backward(go, gs, x, f, q, k, fk, s)
+    for b, c0 in ((0, 0), (1, C), (2, 2 * C)):
+        checks = []
+        if where != "second_half":
+            checks += [("d_q", c0)]
+        if where != "first_half":
+            checks += [("d_x", c0 + C - 1), ("d_k", c0 + C - 1)]
+        for n, t in checks:
+            got = grads[NAMES.index(n)][b, t].double().cpu()
+            ref = torch.as_tensor(r_grads[NAMES.index(n)])[b, t].double()
+            assert (got - ref).abs().max() <= 2e-2 * ref.abs().max(), (n, b, t)
+
+
 @pytest.mark.parametrize("chunk", [0, 15, 16, 17, 36])
 @pytest.mark.parametrize("bad", [-0.0, -0.25, 1.0625])
 def test_a_gate_outside_the_range_in_any_chunk_flags_the_row(chunk, bad):
