@@ -131,6 +131,39 @@ def test_gated_function_matches_oracle(dtype, B, T, D, K):
             assert_close(t.grad, r, dtype, n, tol=tol)
 
 
+@pytest.mark.parametrize("logit_mean,bound", [(-2.0, 8e-2), (-1.0, 4e-2), (0.0, 2e-2)])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_logit_gradients_at_fast_decay(dtype, logit_mean, bound):
+    """Gates from sigmoid(N(m, 1)) for m down to -2 (gates down to 1e-3; the chunk-parallel backward
+    declines most rows at m = -2 and the block-wise kernel takes them).  d_gate at a step with a small
+    gate is (gate * d_gate) / gate, with an absolute error set by the bf16 rounding of the terms that
+    cancel in gate * d_gate; the logit gradient multiplies the gate back in.  Bounds: the worst of a
+    randomized sweep was 4.9e-2 / 1.8e-2 / 1.1e-2 of max|ref| for m = -2 / -1 / 0."""
+    from t2fw_amd import LFWGatedFunction, sigmoid_gates
+    B, T = 6, 200
+    g = torch.Generator().manual_seed(11)
+    x, q, k = [(torch.randn(B, T, 64, generator=g) * 0.125).to(dtype) for _ in range(3)]
+    zf, zk = [(torch.randn(B, T, 64, generator=g) + logit_mean).to(dtype) for _ in range(2)]
+    s = (torch.randn(B, 64, 64, generator=g) * 0.3).to(dtype)
+    go = torch.randn(B, T, 64, generator=g).to(dtype)
+    gs = (torch.randn(B, 64, 64, generator=g) * 0.1).to(dtype)
+    ins = [t.cuda().requires_grad_(True) for t in (x, zf, q, k, zk, s)]
+    out, nxt = LFWGatedFunction.apply(*ins)
+    torch.autograd.backward([out, nxt], [go.cuda(), gs.cuda()])
+    torch.cuda.synchronize()
+    f, fk = [t.cpu() for t in sigmoid_gates(ins[1].detach(), ins[4].detach())]
+    inputs = (x, f, q, k, fk, s)
+    r_out, _ = c_oracle.lfw_forward(*inputs)
+    r_grads = [torch.as_tensor(t).double() for t in c_oracle.lfw_backward(go, gs, *inputs)]
+    assert_close(out, r_out, dtype, "outputs", tol=TOL_CHUNK)
+    for i, n in ((0, "d_x"), (2, "d_q"), (3, "d_k"), (5, "d_state")):
+        assert_close(ins[i].grad, r_grads[i], dtype, n, tol=TOL_CHUNK)
+    for i, gate, n in ((1, f, "d_f_logit"), (4, fk, "d_fk_logit")):
+        ref = r_grads[i] * gate.double() * (1 - gate.double())
+        err = (ins[i].grad.double().cpu() - ref).abs().max() / ref.abs().max()
+        assert err <= bound, (n, float(err))
+
+
 def test_gated_function_equals_ungated_on_its_own_gates():
     """same kernels underneath: outputs and non-gate gradients are bit-identical to LFWFunction on
     sigmoid_gates' output, and the logit gradients are the gate gradients times f(1-f)"""
