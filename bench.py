@@ -7,6 +7,7 @@ synthetic input already resident in HBM, at the headline configuration
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg3|cfg3_heads|cfg3_refgates|cfg2|cfg4|cfg5|dfw|copy256|copy64]
                     [--no-cpu-baseline] [--no-other-configs] [--force-scan] [--dfw-bf16-operands]
+                    [--dfw-dtype float32|float16|bfloat16]
 
 value      = B*T*steps / wall time of the timed region, in Mtokens/s (token = one
              (batch row, time step) pair), driving the C ABI directly with preallocated
@@ -22,7 +23,8 @@ other_configs = after the headline's timed region (cfg3 only): cfg2, cfg4, cfg3 
              reference's tests, cfg5, the delta rule (default and single-operand mode) and cfg3's shape
              with float32 tensors, each briefly.
 dfw        = the delta-rule kernels (forward + backward) at cfg3's shape in fp32, the dtype the
-             reference tests them in (--dfw-bf16-operands: their opt-in single-operand mode).
+             reference tests them in (--dfw-bf16-operands: their opt-in single-operand mode;
+             --dfw-dtype: 16-bit tensors through the same kernels).
 copy256    = calibration workload for those counters: a 256 MiB device-to-device copy.
 copy64     = the same copy at 64 MiB: source and destination together stay inside the 256 MB of last-level cache.
 cpu_baseline = the TorchScript restatement of the reference loop (oracle/), fp32,
@@ -325,6 +327,8 @@ def main():
     ap.add_argument("--force-scan", action="store_true", help="exact scan kernels only")
     ap.add_argument("--dfw-bf16-operands", action="store_true",
                     help="--workload dfw: the opt-in single-bf16 operand mode (flag 16)")
+    ap.add_argument("--dfw-dtype", default="float32", choices=["float32", "float16", "bfloat16"],
+                    help="--workload dfw: tensor dtype")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU only (the path shards over the batch with no "
@@ -341,7 +345,7 @@ def main():
     elif args.workload in ("copy256", "copy64"):
         line = bench_copy(args)
     elif args.workload == "dfw":
-        line = bench_dfw(args, args.steps, args.warmup, args.dfw_bf16_operands)
+        line = bench_dfw(args, args.steps, args.warmup, args.dfw_bf16_operands, args.dfw_dtype)
     elif args.workload == "cfg3_refgates":
         line = bench_lfw(args, "cfg3", args.steps, args.warmup, extras=False, gates="reference_test")
     else:
@@ -358,6 +362,8 @@ def main():
             torch.cuda.empty_cache()
             others["dfw"] = brief(bench_dfw(args, 20, 5))
             others["dfw_bf16_operands"] = brief(bench_dfw(args, 20, 5, bf16_operands=True))
+            others["dfw_float16"] = brief(bench_dfw(args, 20, 5, dtype_name="float16"))
+            others["dfw_bfloat16_bf16_operands"] = brief(bench_dfw(args, 20, 5, bf16_operands=True, dtype_name="bfloat16"))
             torch.cuda.empty_cache()
             others["cfg3_float32"] = bench_float32(args, 20, 3)
             line["other_configs"] = others
@@ -438,9 +444,10 @@ def bench_copy(args):
             "config": {"workload": "%s: torch copy_ of %d bytes, device to device" % (args.workload, n)}}
 
 
-def bench_dfw(args, steps, warmup, bf16_operands=False):
+def bench_dfw(args, steps, warmup, bf16_operands=False, dtype_name="float32"):
     """Delta rule (t2fw/functional_dfw.py:29-65) forward + backward through the C ABI: B=96, T=1024,
-    D=M=64, fp32, keys built as the reference's test builds them (tests/test_dfw.py:45-46).  A step
+    D=M=64, fp32 (dtype_name: or float16 / bfloat16 tensors), keys built as the reference's test builds them
+    (tests/test_dfw.py:45-46).  A step
     is one forward and one backward call; the backward call is two launches (value side, then
     query/key side).  bf16_operands: the opt-in single-bf16 mode of the matrix-core kernels (flag 16)
     instead of their default split operands.  Bytes: forward reads q,k,v,s0 and writes out,delta,final_state; backward
@@ -449,7 +456,8 @@ def bench_dfw(args, steps, warmup, bf16_operands=False):
     from t2fw_amd import _lib
     lib = _lib.load()
     B, T, D, M = 96, 1024, 64, 64
-    dtype, es = torch.float32, 4
+    dtype = getattr(torch, dtype_name)
+    es = torch.empty(0, dtype=dtype).element_size()
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     code = _lib.DTYPE_CODE[dtype]
@@ -467,7 +475,7 @@ def bench_dfw(args, steps, warmup, bf16_operands=False):
         s0 = torch.randn(B, D, M, generator=g)
         go = torch.randn(B, T, D, generator=g)
         gs = torch.randn(B, D, M, generator=g)
-        d = {n: t.to(dev) for n, t in (("q", q), ("k", k), ("v", v), ("s0", s0), ("go", go), ("gs", gs))}
+        d = {n: t.to(dtype).to(dev) for n, t in (("q", q), ("k", k), ("v", v), ("s0", s0), ("go", go), ("gs", gs))}
         for n, like in (("out", "v"), ("delta", "v"), ("fin", "s0"), ("d_q", "q"), ("d_k", "k"), ("d_v", "v"), ("d_s0", "s0")):
             d[n] = torch.empty_like(d[like])
         sets.append(d)
@@ -503,11 +511,12 @@ def bench_dfw(args, steps, warmup, bf16_operands=False):
     ms_per_step = wall / steps * 1e3
     achieved = bwd_bytes / (bwd_ms * 1e-3) / 1e9
     line = {
-        "metric": "delta rule fwd+bwd Mtokens/s, B=96 T=1024 D=M=64 fp32", "value": round(tok * steps / wall / 1e6, 1),
+        "metric": "delta rule fwd+bwd Mtokens/s, B=96 T=1024 D=M=64 %s" % {"float32": "fp32", "float16": "fp16", "bfloat16": "bf16"}[dtype_name],
+        "value": round(tok * steps / wall / 1e6, 1),
         "unit": "Mtokens/s", "n_gpus": 1, "steps": steps, "warmup": warmup,
         "ms_per_step": round(ms_per_step, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "f32", "data": "synthetic",
-        "config": {"workload": "dfw: B=%d T=%d D=%d M=%d float32 fwd+bwd" % (B, T, D, M), "input_sets_rotated": nsets,
+        "dtype": {"float32": "f32", "float16": "f16 I/O, fp32 accumulate", "bfloat16": "bf16 I/O, fp32 accumulate"}[dtype_name], "data": "synthetic",
+        "config": {"workload": "dfw: B=%d T=%d D=%d M=%d %s fwd+bwd" % (B, T, D, M, dtype_name), "input_sets_rotated": nsets,
                    "operands": "exact per-step kernels" if args.force_scan else
                                ("single bf16 (flag 16)" if bf16_operands else "bf16 head + remainder (default)")},
         "forward_avg_ms": round(fwd_ms, 5), "backward_avg_ms": round(bwd_ms, 5),

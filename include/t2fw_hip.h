@@ -93,9 +93,11 @@ extern "C" {
 
 #define T2FW_FLAG_BF16_OPERANDS 16 /* delta rule, matrix-core path: single bf16 operands (2^-9 per operand;
                                      results within 1e-2 of max|ref| like the LFW kernels') instead of
-                                     operands split into bf16 head + remainder (fp32-level results, three
-                                     matrix-core products per product): for callers that train in reduced
-                                     precision anyway.  Off by default.                               */
+                                     operands split into bf16 head + remainder (fp32-level results before
+                                     they are rounded to the tensors' type, three matrix-core products per
+                                     product): for callers that train in reduced precision anyway.  With
+                                     bf16 tensors it costs next to nothing in accuracy (what is stored is
+                                     rounded to bf16 either way).  Off unless passed.                 */
 
 int t2fw_abi_version(void);
 const char *t2fw_last_error(void);
@@ -223,6 +225,9 @@ int t2fw_lfw_step(const void *x, const void *f, const void *q, const void *k,
  * Delta rule.  out_t = S_{t-1} q_t ; delta_t = v_t - S_{t-1} k_t ;
  * S_t = S_{t-1} + delta_t (x) k_t.   q,k,d_q,d_k [B,T,M]; v,out,delta,g_out,d_v [B,T,D];
  * s0,final_state,g_state,d_s0 [B,D,M].  Replaces dfw.cpp:27-39 / :41-64.
+ * D = M = 64 with fp32, fp16 or bf16 tensors and 16-byte aligned pointers runs on the matrix cores in blocks of
+ * 16 steps (flags: T2FW_FLAG_BF16_OPERANDS above); everything else, or T2FW_FLAG_FORCE_SCAN, the exact
+ * per-step kernels.
  */
 int t2fw_dfw_forward(const void *q, const void *k, const void *v, const void *s0,
                      void *out, void *final_state, void *delta,

@@ -503,9 +503,10 @@ int t2fw_lfw_step(const void *x, const void *f, const void *q, const void *k, co
                             T2FW_FLAG_FORCE_SCAN, nullptr, 0, stream);
 }
 
-// The block-wise matrix-core kernels of the delta rule cover D = M = 64 with fp32 tensors.
+// The block-wise matrix-core kernels of the delta rule cover D = M = 64 with fp32, fp16 and bf16 tensors.
 static bool dfw_chunk_ok(int64_t D, int64_t M, int32_t dtype, int32_t flags) {
-    return (flags & T2FW_FLAG_FORCE_SCAN) == 0 && D == 64 && M == 64 && dtype == T2FW_F32;
+    return (flags & T2FW_FLAG_FORCE_SCAN) == 0 && D == 64 && M == 64 &&
+           (dtype == T2FW_F32 || dtype == T2FW_F16 || dtype == T2FW_BF16);
 }
 
 int t2fw_dfw_forward(const void *q, const void *k, const void *v, const void *s0, void *out, void *final_state,
@@ -533,7 +534,7 @@ int t2fw_dfw_forward(const void *q, const void *k, const void *v, const void *s0
     a.q = q; a.k = k; a.v = v; a.s0 = s0; a.out = out; a.final_state = final_state; a.delta = delta;
     a.B = B; a.T = T; a.D = D; a.M = M;
     if (dfw_chunk_ok(D, M, dtype, flags) && T * CH_N < 0x7fffffffLL && aligned16({q, k, v, s0, out, final_state, delta}))
-        return dfw_chunk_forward(a, (flags & T2FW_FLAG_BF16_OPERANDS) == 0, st);
+        return dfw_chunk_forward(a, dtype, (flags & T2FW_FLAG_BF16_OPERANDS) == 0, st);
     return dfw_forward(a, dtype, st);
 }
 
@@ -565,7 +566,7 @@ int t2fw_dfw_backward(const void *g_out, const void *g_state, const void *q, con
     a.B = B; a.T = T; a.D = D; a.M = M;
     if (dfw_chunk_ok(D, M, dtype, flags) && T * CH_N < 0x7fffffffLL &&
         aligned16({g_out, g_state, q, k, delta, final_state, d_q, d_k, d_v, d_s0}))
-        return dfw_chunk_backward(a, (flags & T2FW_FLAG_BF16_OPERANDS) == 0, st);
+        return dfw_chunk_backward(a, dtype, (flags & T2FW_FLAG_BF16_OPERANDS) == 0, st);
     return dfw_backward(a, dtype, st);
 }
 

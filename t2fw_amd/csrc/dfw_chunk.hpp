@@ -1,4 +1,4 @@
-// Block-wise matrix-core form of the delta rule for D = M = 64, fp32 tensors (dfw_chunk_fwd.hip,
+// Block-wise matrix-core form of the delta rule for D = M = 64, fp32 / fp16 / bf16 tensors (dfw_chunk_fwd.hip,
 // dfw_chunk_bwd.hip): shared layout constants and device helpers.
 //
 // Inside a block of L = 16 steps that starts from the state S0 (all matrices with one row per step):
@@ -10,11 +10,15 @@
 // K' = Tm K do not depend on the state, so they are prepared ahead of the sequential pass, whose chain per
 // block is then only  S0 -> Delta = Tm V - K' S0^T -> S_L.  The backward pass uses Tm transposed the same way.
 //
-// Precision: the tensors are fp32 and the matrix cores take bf16, so every operand is split into a bf16
-// head and a bf16 remainder (x = hi + lo up to 2^-17 of x) and a product runs as three MFMAs
+// Precision: the matrix cores take bf16, so every operand (an fp32 or fp16 input, an fp32 intermediate) is
+// split into a bf16 head and a bf16 remainder (x = hi + lo up to 2^-17 of x) and a product runs as three MFMAs
 // (hi*hi + hi*lo + lo*hi) with fp32 accumulation: results carry fp32-level rounding (measured against the
-// fp64 oracle: 3e-5 of max|ref|), not the 2^-9 of a single bf16 operand.  A caller that prefers speed asks for
-// the heads alone (T2FW_FLAG_BF16_OPERANDS; template parameter SP = false below).
+// fp64 oracle: 3e-5 of max|ref|), not the 2^-9 of a single bf16 operand, before they are rounded to the tensors'
+// type.  A caller that prefers speed asks for the heads alone (T2FW_FLAG_BF16_OPERANDS; template parameter
+// SP = false below).
+//
+// Tensor element types: the kernels are templates over an element policy E (ElF32, El16<Fp16>, El16<Bf16>) that
+// says how a lane moves elements between global memory and registers; all arithmetic is the same.
 #pragma once
 
 #include "lfw_chunk.hpp"
@@ -34,6 +38,67 @@ constexpr int DCS = 20;                       // row stride of channel-major til
 constexpr int TM_TILE = DL * DTS * 2;         // bytes of one token-major tile (one of hi / lo)
 constexpr int CM_TILE = CH_N * DCS * 2;       // bytes of one channel-major tile
 constexpr int ST_TILE = 64 * 8;               // a 16 x 16 matrix as a packed MFMA operand: 8 bytes per lane
+
+// ---- element types of the tensors ----------------------------------------------------------------------
+// elem: the type in memory.  A value that is loaded ahead of its use stays in the form it was loaded in (elem,
+// Raw16) and is converted where it is used: a conversion next to the load would wait for the load there.
+struct ElF32 {
+    typedef float elem;
+    struct Raw16 {          // sixteen consecutive channels of one token
+        float4 v[4];
+    };
+    static __device__ __forceinline__ float f(elem x) { return x; }
+    static __device__ __forceinline__ elem e(float x) { return x; }
+    static __device__ __forceinline__ Raw16 load16(const elem *p) {
+        Raw16 r;
+#pragma unroll
+        for (int a = 0; a < 4; ++a) r.v[a] = reinterpret_cast<const float4 *>(p)[a];
+        return r;
+    }
+    static __device__ __forceinline__ void floats(const Raw16 &r, float (&o)[16]) {
+#pragma unroll
+        for (int a = 0; a < 4; ++a) {
+            o[4 * a] = r.v[a].x; o[4 * a + 1] = r.v[a].y; o[4 * a + 2] = r.v[a].z; o[4 * a + 3] = r.v[a].w;
+        }
+    }
+    // four consecutive elements, 16-byte aligned
+    static __device__ __forceinline__ floatx4 load4(const elem *p) {
+        const float4 t = *reinterpret_cast<const float4 *>(p);
+        return floatx4{t.x, t.y, t.z, t.w};
+    }
+    static __device__ __forceinline__ void store4(elem *p, const floatx4 &v) {
+        *reinterpret_cast<float4 *>(p) = make_float4(v[0], v[1], v[2], v[3]);
+    }
+};
+template <typename IOE> struct El16 {          // IOE = Fp16 or Bf16 (lfw_chunk.hpp)
+    typedef u16 elem;
+    struct Raw16 {
+        uint4 v[2];
+    };
+    static __device__ __forceinline__ float f(elem x) { return IOE::to_f32(x); }
+    static __device__ __forceinline__ elem e(float x) { return cvt1<IOE>(x); }
+    static __device__ __forceinline__ Raw16 load16(const elem *p) {
+        Raw16 r;
+        r.v[0] = reinterpret_cast<const uint4 *>(p)[0];
+        r.v[1] = reinterpret_cast<const uint4 *>(p)[1];
+        return r;
+    }
+    static __device__ __forceinline__ void floats(const Raw16 &r, float (&o)[16]) {
+        const u32 w[8] = {r.v[0].x, r.v[0].y, r.v[0].z, r.v[0].w, r.v[1].x, r.v[1].y, r.v[1].z, r.v[1].w};
+#pragma unroll
+        for (int a = 0; a < 8; ++a) {
+            o[2 * a] = IOE::to_f32((u16)(w[a] & 0xffffu));
+            o[2 * a + 1] = IOE::to_f32((u16)(w[a] >> 16));
+        }
+    }
+    // four consecutive elements, 8-byte aligned
+    static __device__ __forceinline__ floatx4 load4(const elem *p) {
+        float o[4];
+        unpack4<IOE>(*reinterpret_cast<const uint2 *>(p), o);
+        return floatx4{o[0], o[1], o[2], o[3]};
+    }
+    static __device__ __forceinline__ void store4(elem *p, const floatx4 &v) { *reinterpret_cast<uint2 *>(p) = packq<IOE>(v[0], v[1], v[2], v[3]); }
+};
 
 // An operand of a 16-deep (Sp2) or 32-deep (Sp4) contraction as bf16 head and remainder.  SP = false (the
 // caller asked for T2FW_FLAG_BF16_OPERANDS): the head alone, one MFMA per product, 2^-9 per operand.
@@ -180,51 +245,25 @@ template <bool SP> struct BlockInverse {
     __device__ __forceinline__ floatx4 acc_tm() const { return mma16(p2t, p1, floatx4{0.f, 0.f, 0.f, 0.f}); }
 };
 
-// ---- staging of an fp32 [T, 64] array into tiles (one wave per array and layout) -------------------
-// sixteen floats of one lane: token-major staging takes token lane >> 2, channels 16 (lane & 3) .. + 15;
-// channel-major staging takes channel `lane`, tokens 0 .. 15 of the block.  Rows at or past T read as zero.
-struct Raw16 {
-    float4 v[4];
-};
+// ---- staging of a [T, 64] array into tiles (one wave per array) ---------------------------------------
+// sixteen elements of one lane: token lane >> 2, channels 16 (lane & 3) .. + 15.  Rows at or past T read as zero.
 // Loads are issued unconditionally (rows at or past T are read from row T - 1 and zeroed when the tile is
 // built): a load inside a branch would make every later wait for a load a wait for all of them.
-__device__ __forceinline__ Raw16 load_tm(const float *row0, int tok0, int T, int lane) {
-    Raw16 r;
+template <typename E> __device__ __forceinline__ typename E::Raw16 load_tm(const typename E::elem *row0, int tok0, int T, int lane) {
     const int t = min(tok0 + (lane >> 2), T - 1);
-    const float4 *p = reinterpret_cast<const float4 *>(row0 + (size_t)t * CH_N + 16 * (lane & 3));
-#pragma unroll
-    for (int a = 0; a < 4; ++a) r.v[a] = p[a];
-    return r;
+    return E::load16(row0 + (size_t)t * CH_N + 16 * (lane & 3));
 }
-template <bool SP> __device__ __forceinline__ void store_tm(unsigned char *tile, int lane, const Raw16 &r, int tok0, int T, float sign = 1.f) {
+template <bool SP, typename E> __device__ __forceinline__ void store_tm(unsigned char *tile, int lane, const typename E::Raw16 &r, int tok0, int T, float sign = 1.f) {
     u16 *hi = reinterpret_cast<u16 *>(tile), *lo = reinterpret_cast<u16 *>(tile + TM_TILE);
     const int o = (lane >> 2) * DTS + 4 * (lane & 3);
     const float keep = tok0 + (lane >> 2) < T ? sign : 0.f;
+    float v[16];
+    E::floats(r, v);
 #pragma unroll
     for (int a = 0; a < 4; ++a) {          // channels 16 q + 4 a + e sit at 16 a + 4 q + e
-        const Sp2<SP> s = split4<SP>(r.v[a].x * keep, r.v[a].y * keep, r.v[a].z * keep, r.v[a].w * keep);
+        const Sp2<SP> s = split4<SP>(v[4 * a] * keep, v[4 * a + 1] * keep, v[4 * a + 2] * keep, v[4 * a + 3] * keep);
         *reinterpret_cast<uint2 *>(hi + o + 16 * a) = s.hi;
         if constexpr (SP) *reinterpret_cast<uint2 *>(lo + o + 16 * a) = s.lo;
-    }
-}
-__device__ __forceinline__ Raw16 load_cm(const float *row0, int tok0, int T, int lane) {
-    Raw16 r;
-    float f[16];
-#pragma unroll
-    for (int t = 0; t < 16; ++t) f[t] = row0[(size_t)min(tok0 + t, T - 1) * CH_N + lane];
-#pragma unroll
-    for (int a = 0; a < 4; ++a) r.v[a] = make_float4(f[4 * a], f[4 * a + 1], f[4 * a + 2], f[4 * a + 3]);
-    return r;
-}
-template <bool SP> __device__ __forceinline__ void store_cm(unsigned char *tile, int lane, const Raw16 &r, int tok0, int T, float sign = 1.f) {
-    u16 *hi = reinterpret_cast<u16 *>(tile), *lo = reinterpret_cast<u16 *>(tile + CM_TILE);
-#pragma unroll
-    for (int a = 0; a < 4; ++a) {
-        const int t = tok0 + 4 * a;
-        const Sp2<SP> s = split4<SP>(t < T ? r.v[a].x * sign : 0.f, t + 1 < T ? r.v[a].y * sign : 0.f, t + 2 < T ? r.v[a].z * sign : 0.f,
-                                     t + 3 < T ? r.v[a].w * sign : 0.f);
-        *reinterpret_cast<uint2 *>(hi + lane * DCS + 4 * a) = s.hi;
-        if constexpr (SP) *reinterpret_cast<uint2 *>(lo + lane * DCS + 4 * a) = s.lo;
     }
 }
 
@@ -243,31 +282,32 @@ template <int RAW_BLOCK, int ST_BLOCK, int NBLK> struct Ring {
 };
 
 // One wave stages NJOBS arrays for every stage, two stages ahead of the slab waves.  An array is loaded once,
-// token-major (four 16-byte loads per lane and block), and written as a token-major tile; where a channel-major
+// token-major (four 16-byte loads per lane and block for fp32 tensors, two for 16-bit ones), and written as a token-major tile; where a channel-major
 // tile of the same array is wanted too, the wave reads its own token-major tile back with the transposing LDS
 // read and writes that (the loads of a second layout were what the wave waited for: a wave can have 63 memory
 // instructions outstanding, and a channel-major tile loaded directly is sixteen 4-byte loads per lane).
 // Loads are unconditional and issued SETS - 1 stages before their tiles are built, into the register set that the
 // stage before has left (SETS sets in turn; the stage loop is unrolled SETS times so that no register copy waits
 // for a load).  tok0_of(stage, bb): first token of a block (at or past T: a block of zeros).
-struct PrepJob {
-    const float *src;       // token 0 of the batch row
+template <typename E> struct PrepJob {
+    const typename E::elem *src;       // token 0 of the batch row
     int tm_off;             // byte offset of the token-major tile inside a block's raw tiles; < 0: the wave's scratch tile
     int cm_off;             // byte offset of the channel-major tile; < 0: none
     float sign;             // the token-major tile holds sign * src
     bool cm_negated;        // the channel-major tile holds the negative of the token-major one
 };
-template <typename RING, int NBLK, int NJOBS, bool SP, int SETS, typename TOK0>
-__device__ __forceinline__ void prep_wave_jobs(unsigned char *smem, const PrepJob (&jobs)[NJOBS], int T, int nstages, int lane,
+template <typename RING, int NBLK, int NJOBS, bool SP, int SETS, typename E, typename TOK0>
+__device__ __forceinline__ void prep_wave_jobs(unsigned char *smem, const PrepJob<E> (&jobs)[NJOBS], int T, int nstages, int lane,
                                                TOK0 tok0_of, unsigned char *scratch_tile) {
     static_assert(SETS == 2 || SETS == 3, "two or three register sets");
     const int r = lane & 15, g = lane >> 4;
+    typedef typename E::Raw16 Raw16;
     Raw16 set_a[NJOBS][NBLK], set_b[NJOBS][NBLK], set_c[SETS == 3 ? NJOBS : 1][SETS == 3 ? NBLK : 1];
     auto load = [&](auto &regs, int stage) {
 #pragma unroll
         for (int a = 0; a < NJOBS; ++a)
 #pragma unroll
-            for (int bb = 0; bb < NBLK; ++bb) regs[a][bb] = load_tm(jobs[a].src, tok0_of(stage, bb), T, lane);
+            for (int bb = 0; bb < NBLK; ++bb) regs[a][bb] = load_tm<E>(jobs[a].src, tok0_of(stage, bb), T, lane);
     };
     // stage `stage` out of `cur`; the loads of stage + SETS - 1 into `far` (the set that stage - 1 has left)
     auto stage_body = [&](int stage, auto &cur, auto &far) {
@@ -278,7 +318,7 @@ __device__ __forceinline__ void prep_wave_jobs(unsigned char *smem, const PrepJo
             for (int bb = 0; bb < NBLK; ++bb) {
                 unsigned char *const raw = RING::raw(smem, stage, bb);
                 unsigned char *const tm = jobs[a].tm_off >= 0 ? raw + jobs[a].tm_off : scratch_tile;
-                store_tm<SP>(tm, lane, cur[a][bb], tok0_of(stage, bb), T, jobs[a].sign);
+                store_tm<SP, E>(tm, lane, cur[a][bb], tok0_of(stage, bb), T, jobs[a].sign);
                 if (jobs[a].cm_off >= 0) {
                     // DS operations of one wave execute in order: the reads below see the tile just written
                     const TmTile<SP> own(tm);

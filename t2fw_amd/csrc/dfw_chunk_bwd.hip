@@ -1,5 +1,5 @@
-// Backward pass of the delta rule on the matrix cores, D = M = 64, fp32 tensors (block algebra, precision
-// and staging: dfw_chunk.hpp).  Blocks of 16 steps are visited last to first.  With g = dL/dO of the block,
+// Backward pass of the delta rule on the matrix cores, D = M = 64, fp32 / fp16 / bf16 tensors (block algebra,
+// precision, element types and staging: dfw_chunk.hpp).  Blocks of 16 steps are visited last to first.  With g = dL/dO of the block,
 // G_end the adjoint of the state after it, Delta the block's saved deltas and Tm = (I + A)^-1:
 //   dDelta = Bq^T g + K G_end^T            dU = Tm^T dDelta  (= d_value)
 //   G_start = G_end + g^T Q - dU^T K       (d_state = G before the first block)
@@ -67,57 +67,58 @@ template <bool SP> __device__ __forceinline__ void vs_structure_wave(unsigned ch
     }
 }
 
-template <bool SP> __device__ __forceinline__ void vs_slab_wave(const DfwBwdArgs &p, unsigned char *smem, int64_t b, int d0, int nstages, int lane) {
+template <bool SP, typename E> __device__ __forceinline__ void vs_slab_wave(const DfwBwdArgs &p, unsigned char *smem, int64_t b, int d0, int nstages, int lane) {
+    typedef typename E::elem elem;
     const int r = lane & 15, g = lane >> 4, d = d0 + r, T = (int)p.T, nblocks = nstages * DNB;
     const floatx4 zero = {0.f, 0.f, 0.f, 0.f};
-    const float *const go = reinterpret_cast<const float *>(p.g_out) + b * p.T * CH_N;
-    float *const d_v = reinterpret_cast<float *>(p.d_v) + b * p.T * CH_N;
+    const elem *const go = reinterpret_cast<const elem *>(p.g_out) + b * p.T * CH_N;
+    elem *const d_v = reinterpret_cast<elem *>(p.d_v) + b * p.T * CH_N;
     const u32 lane_off = (u32)(4 * g * CH_N + d);
     // G[j][e] = G[d][16 j + 4 g + e]
     floatx4 G[4];
     {
-        const float *gs = reinterpret_cast<const float *>(p.g_state) + (b * CH_N + d) * CH_N + 4 * g;
+        const elem *gs = reinterpret_cast<const elem *>(p.g_state) + (b * CH_N + d) * CH_N + 4 * g;
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            const float4 t = *reinterpret_cast<const float4 *>(gs + 16 * j);
-            G[j] = floatx4{t.x, t.y, t.z, t.w};
-        }
+        for (int j = 0; j < 4; ++j) G[j] = E::load4(gs + 16 * j);
     }
-    auto load_g = [&](floatx4 (&x)[DNB], int stage) {
+    // g of a stage as loaded, one stage ahead (converted where the stage uses it)
+    struct GRaw {
+        elem x[DNB][4];
+    };
+    auto load_g = [&](GRaw &x, int stage) {
 #pragma unroll
         for (int bb = 0; bb < DNB; ++bb)
 #pragma unroll
             for (int e = 0; e < 4; ++e)
-                x[bb][e] = go[(size_t)min(reverse_tok0(nblocks, DNB, stage, bb) + 4 * g + e, T - 1) * CH_N + d];
+                x.x[bb][e] = go[(size_t)min(reverse_tok0(nblocks, DNB, stage, bb) + 4 * g + e, T - 1) * CH_N + d];
     };
     // One stage.  FULL: every token of the stage is below T and the body has no branch.  (The waits that the
     // compiler places count outstanding memory operations along every path: a path that skips stores, or loads
     // still pending where the loop is entered, would make each stage wait for the stores of the stage before.)
-    auto stage_body = [&](auto full, int stage, floatx4 (&gcur)[DNB], floatx4 (&gnxt)[DNB]) {
+    auto stage_body = [&](auto full, int stage, GRaw &graw, GRaw &gnxt) {
         constexpr bool FULL = decltype(full)::value;
         load_g(gnxt, min(stage + 1, nstages - 1));
 #pragma unroll
         for (int bb = 0; bb < DNB; ++bb) {
             const int tok0 = reverse_tok0(nblocks, DNB, stage, bb);
-            if constexpr (!FULL) {
+            floatx4 gcur;
 #pragma unroll
-                for (int e = 0; e < 4; ++e) gcur[bb][e] = tok0 + 4 * g + e < T ? gcur[bb][e] : 0.f;
-            }
+            for (int e = 0; e < 4; ++e) gcur[e] = (FULL || tok0 + 4 * g + e < T) ? E::f(graw.x[bb][e]) : 0.f;
             const unsigned char *raw = VsRing::raw(smem, stage, bb);
             const unsigned char *st = VsRing::st(smem, stage, bb);
             const TmTile<SP> KPP(st + VS_KPP);
             const CmTile<SP> KC(raw + VS_KC), QC(raw + VS_QC);
             // dU[tok 4g+e][d] = Tm^T (Bq^T g) + K'' G_end^T: only the second term waits for the adjoint
-            const Sp2<SP> gs = split4<SP>(gcur[bb]);
+            const Sp2<SP> gs = split4<SP>(gcur);
             const floatx4 bg = mma16(st_load<SP>(st + VS_BQ, lane), gs, zero);
             const floatx4 tbg = mma16(st_load<SP>(st + VS_TM, lane), split4<SP>(bg), zero);
             const Sp4<SP> gb0 = cat(split4<SP>(G[0]), split4<SP>(G[1])), gb1 = cat(split4<SP>(G[2]), split4<SP>(G[3]));
             const floatx4 kg = mma32(KPP.acc_order(r, g, 1), gb1, mma32(KPP.acc_order(r, g, 0), gb0, zero));
             const floatx4 du = tbg + kg;
-            float *const vb = d_v + (size_t)tok0 * CH_N;        // wave-uniform
+            elem *const vb = d_v + (size_t)tok0 * CH_N;        // wave-uniform
 #pragma unroll
             for (int e = 0; e < 4; ++e)
-                if (FULL || tok0 + 4 * g + e < T) vb[lane_off + e * CH_N] = du[e];
+                if (FULL || tok0 + 4 * g + e < T) vb[lane_off + e * CH_N] = E::e(du[e]);
             // G += g^T Q - dU^T K
             const Sp2<SP> ndu = split4<SP>(-du);
 #pragma unroll
@@ -128,7 +129,7 @@ template <bool SP> __device__ __forceinline__ void vs_slab_wave(const DfwBwdArgs
         }
         __syncthreads();
     };
-    floatx4 g_a[DNB], g_b[DNB];
+    GRaw g_a, g_b;
     load_g(g_a, 0);
     __syncthreads();        // ticks 0 and 1: the prep and matrix waves fill the pipeline
     __syncthreads();
@@ -141,34 +142,35 @@ template <bool SP> __device__ __forceinline__ void vs_slab_wave(const DfwBwdArgs
         stage_body(std::true_type{}, stage + 1, g_a, g_b);
     }
     if (stage < nstages) stage_body(std::true_type{}, stage, g_b, g_a);
-    float *ds0 = reinterpret_cast<float *>(p.d_s0) + (b * CH_N + d) * CH_N + 4 * g;
+    elem *ds0 = reinterpret_cast<elem *>(p.d_s0) + (b * CH_N + d) * CH_N + 4 * g;
 #pragma unroll
-    for (int j = 0; j < 4; ++j) *reinterpret_cast<float4 *>(ds0 + 16 * j) = make_float4(G[j][0], G[j][1], G[j][2], G[j][3]);
+    for (int j = 0; j < 4; ++j) E::store4(ds0 + 16 * j, G[j]);
 }
 
 // blockIdx = half * rows_padded + row (rows_padded a multiple of 8: both halves of a row on one XCD).  Waves 0, 1:
 // slab waves, alone on SIMDs 0 and 1; waves 2, 3: matrix waves; waves 6, 7: prep waves; waves 4, 5 leave at once.
-template <bool SP> __global__ __launch_bounds__(BW_THREADS) void dfw_chunk_bwd_value_kernel(DfwBwdArgs p, int rows_padded) {
+template <bool SP, typename E> __global__ __launch_bounds__(BW_THREADS) void dfw_chunk_bwd_value_kernel(DfwBwdArgs p, int rows_padded) {
+    typedef typename E::elem elem;
     extern __shared__ __align__(16) unsigned char smem[];
     const int half = (int)blockIdx.x >= rows_padded ? 1 : 0;
     const int64_t b = (int)blockIdx.x - half * rows_padded;
     if (b >= p.B) return;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
     const int T = (int)p.T, nstages = (T + DL * DNB - 1) / (DL * DNB), nblocks = nstages * DNB;
-    const float *const k = reinterpret_cast<const float *>(p.k) + b * p.T * CH_N;
-    const float *const q = reinterpret_cast<const float *>(p.q) + b * p.T * CH_N;
+    const elem *const k = reinterpret_cast<const elem *>(p.k) + b * p.T * CH_N;
+    const elem *const q = reinterpret_cast<const elem *>(p.q) + b * p.T * CH_N;
     auto tok0_of = [=](int stage, int bb) { return reverse_tok0(nblocks, DNB, stage, bb); };
     static_assert(DNB == 2, "one matrix wave per block of a stage");
     if (wave < 2) {
-        vs_slab_wave<SP>(p, smem, b, 32 * half + 16 * wave, nstages, lane);
+        vs_slab_wave<SP, E>(p, smem, b, 32 * half + 16 * wave, nstages, lane);
     } else if (wave < 4) {
         vs_structure_wave<SP>(smem, nstages, wave - 2, lane);
     } else if (wave == 6) {
-        const PrepJob jobs[1] = {{k, VS_KT, VS_KC, 1.f, false}};
-        prep_wave_jobs<VsRing, DNB, 1, SP, 3>(smem, jobs, T, nstages, lane, tok0_of, nullptr);
+        const PrepJob<E> jobs[1] = {{k, VS_KT, VS_KC, 1.f, false}};
+        prep_wave_jobs<VsRing, DNB, 1, SP, 3, E>(smem, jobs, T, nstages, lane, tok0_of, nullptr);
     } else if (wave == 7) {
-        const PrepJob jobs[1] = {{q, VS_QT, VS_QC, 1.f, false}};
-        prep_wave_jobs<VsRing, DNB, 1, SP, 3>(smem, jobs, T, nstages, lane, tok0_of, nullptr);
+        const PrepJob<E> jobs[1] = {{q, VS_QT, VS_QC, 1.f, false}};
+        prep_wave_jobs<VsRing, DNB, 1, SP, 3, E>(smem, jobs, T, nstages, lane, tok0_of, nullptr);
     }
 }
 
@@ -223,16 +225,17 @@ template <bool SP> __device__ __forceinline__ void ks_structure_wave(unsigned ch
 // The adjoint chain of 16 key channels: G_start = G_end + g^T Q - dU^T K, one stage ahead of the state waves, to
 // which it hands G_end of every block as a split B operand.  It shares a SIMD with the state wave of the same
 // channels: two independent chains whose instruction streams interleave.
-template <bool SP> __device__ __forceinline__ void ks_adjoint_wave(const DfwBwdArgs &p, unsigned char *smem, int64_t b, int m0, int w, int nstages, int lane) {
+template <bool SP, typename E> __device__ __forceinline__ void ks_adjoint_wave(const DfwBwdArgs &p, unsigned char *smem, int64_t b, int m0, int w, int nstages, int lane) {
+    typedef typename E::elem elem;
     const int r = lane & 15, g = lane >> 4, m = m0 + r;
     // G[j][e] = G[d = 16 j + 4 g + e][m]: columns of the state's adjoint
     floatx4 G[4];
     {
-        const float *gs = reinterpret_cast<const float *>(p.g_state) + b * CH_N * CH_N + m;
+        const elem *gs = reinterpret_cast<const elem *>(p.g_state) + b * CH_N * CH_N + m;
 #pragma unroll
         for (int j = 0; j < 4; ++j)
 #pragma unroll
-            for (int e = 0; e < 4; ++e) G[j][e] = gs[(16 * j + 4 * g + e) * CH_N];
+            for (int e = 0; e < 4; ++e) G[j][e] = E::f(gs[(16 * j + 4 * g + e) * CH_N]);
     }
     for (int tick = 0; tick < nstages + 2; ++tick) {
         const int stage = tick - 1;
@@ -261,20 +264,21 @@ template <bool SP> __device__ __forceinline__ void ks_adjoint_wave(const DfwBwdA
 }
 
 // The state chain of 16 key channels, walked backwards (S0 = S_end - Delta^T K), and the block's d_query, d_key.
-template <bool SP> __device__ __forceinline__ void ks_slab_wave(const DfwBwdArgs &p, unsigned char *smem, int64_t b, int m0, int w, int nstages, int lane) {
+template <bool SP, typename E> __device__ __forceinline__ void ks_slab_wave(const DfwBwdArgs &p, unsigned char *smem, int64_t b, int m0, int w, int nstages, int lane) {
+    typedef typename E::elem elem;
     const int r = lane & 15, g = lane >> 4, m = m0 + r, T = (int)p.T, nblocks = nstages;
     const floatx4 zero = {0.f, 0.f, 0.f, 0.f};
-    float *const d_q = reinterpret_cast<float *>(p.d_q) + b * p.T * CH_N;
-    float *const d_k = reinterpret_cast<float *>(p.d_k) + b * p.T * CH_N;
+    elem *const d_q = reinterpret_cast<elem *>(p.d_q) + b * p.T * CH_N;
+    elem *const d_k = reinterpret_cast<elem *>(p.d_k) + b * p.T * CH_N;
     const u32 lane_off = (u32)(4 * g * CH_N + m);
     // S[j][e] = S[d = 16 j + 4 g + e][m]: columns of the state
     floatx4 S[4];
     {
-        const float *fs = reinterpret_cast<const float *>(p.final_state) + b * CH_N * CH_N + m;
+        const elem *fs = reinterpret_cast<const elem *>(p.final_state) + b * CH_N * CH_N + m;
 #pragma unroll
         for (int j = 0; j < 4; ++j)
 #pragma unroll
-            for (int e = 0; e < 4; ++e) S[j][e] = fs[(16 * j + 4 * g + e) * CH_N];
+            for (int e = 0; e < 4; ++e) S[j][e] = E::f(fs[(16 * j + 4 * g + e) * CH_N]);
     }
     // one stage (= one block).  FULL: every token of the stage is below T and the body has no branch (see the
     // value side)
@@ -304,12 +308,12 @@ template <bool SP> __device__ __forceinline__ void ks_slab_wave(const DfwBwdArgs
                                  mma32(NUT.acc_order(r, g, 0), sb0,
                                        mma32(DT.acc_order(r, g, 1), gb1, mma32(DT.acc_order(r, g, 0), gb0, zero)))) +
                            mma16(st_load<SP>(st + KS_X2S, lane), kb, mma16(st_load<SP>(st + KS_X1, lane), qb, zero));
-        float *const qo = d_q + (size_t)tok0 * CH_N, *const ko = d_k + (size_t)tok0 * CH_N;      // wave-uniform
+        elem *const qo = d_q + (size_t)tok0 * CH_N, *const ko = d_k + (size_t)tok0 * CH_N;      // wave-uniform
 #pragma unroll
         for (int e = 0; e < 4; ++e)
             if (FULL || tok0 + 4 * g + e < T) {
-                qo[lane_off + e * CH_N] = dq[e];
-                ko[lane_off + e * CH_N] = dk[e];
+                qo[lane_off + e * CH_N] = E::e(dq[e]);
+                ko[lane_off + e * CH_N] = E::e(dk[e]);
             }
         __syncthreads();
     };
@@ -323,7 +327,8 @@ template <bool SP> __device__ __forceinline__ void ks_slab_wave(const DfwBwdArgs
 
 // Waves 0, 1: state waves (16 key channels each) and waves 4, 5: the adjoint waves of the same channels, on SIMDs 0
 // and 1; wave 2: matrix wave; waves 3, 6, 7: prep waves.
-template <bool SP> __global__ __launch_bounds__(BW_THREADS) void dfw_chunk_bwd_key_kernel(DfwBwdArgs p, int rows_padded) {
+template <bool SP, typename E> __global__ __launch_bounds__(BW_THREADS) void dfw_chunk_bwd_key_kernel(DfwBwdArgs p, int rows_padded) {
+    typedef typename E::elem elem;
     extern __shared__ __align__(16) unsigned char smem[];
     const int half = (int)blockIdx.x >= rows_padded ? 1 : 0;
     const int64_t b = (int)blockIdx.x - half * rows_padded;
@@ -331,35 +336,35 @@ template <bool SP> __global__ __launch_bounds__(BW_THREADS) void dfw_chunk_bwd_k
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
     const int T = (int)p.T, nstages = (T + DL - 1) / DL;
     const int64_t row = b * p.T * CH_N;
-    const float *const k = reinterpret_cast<const float *>(p.k) + row;
-    const float *const q = reinterpret_cast<const float *>(p.q) + row;
-    const float *const dl = reinterpret_cast<const float *>(p.delta) + row;
-    const float *const go = reinterpret_cast<const float *>(p.g_out) + row;
-    const float *const dv = reinterpret_cast<const float *>(p.d_v) + row;
+    const elem *const k = reinterpret_cast<const elem *>(p.k) + row;
+    const elem *const q = reinterpret_cast<const elem *>(p.q) + row;
+    const elem *const dl = reinterpret_cast<const elem *>(p.delta) + row;
+    const elem *const go = reinterpret_cast<const elem *>(p.g_out) + row;
+    const elem *const dv = reinterpret_cast<const elem *>(p.d_v) + row;
     auto tok0_of = [=](int stage, int bb) { return reverse_tok0(nstages, 1, stage, bb); };
     if (wave < 2) {
-        ks_slab_wave<SP>(p, smem, b, 32 * half + 16 * wave, wave, nstages, lane);
+        ks_slab_wave<SP, E>(p, smem, b, 32 * half + 16 * wave, wave, nstages, lane);
     } else if (wave == 4 || wave == 5) {
-        ks_adjoint_wave<SP>(p, smem, b, 32 * half + 16 * (wave - 4), wave - 4, nstages, lane);
+        ks_adjoint_wave<SP, E>(p, smem, b, 32 * half + 16 * (wave - 4), wave - 4, nstages, lane);
     } else if (wave == 2) {
         ks_structure_wave<SP>(smem, nstages, lane);
     } else if (wave == 3) {
-        const PrepJob jobs[1] = {{dl, KS_DT, KS_NDC, 1.f, true}};
-        prep_wave_jobs<KsRing, 1, 1, SP, 3>(smem, jobs, T, nstages, lane, tok0_of, nullptr);
+        const PrepJob<E> jobs[1] = {{dl, KS_DT, KS_NDC, 1.f, true}};
+        prep_wave_jobs<KsRing, 1, 1, SP, 3, E>(smem, jobs, T, nstages, lane, tok0_of, nullptr);
     } else if (wave == 6) {
-        const PrepJob jobs[2] = {{go, KS_GT, -1, 1.f, false}, {k, -1, KS_KC, 1.f, false}};
-        prep_wave_jobs<KsRing, 1, 2, SP, 3>(smem, jobs, T, nstages, lane, tok0_of, smem + KS_SCRATCH);
+        const PrepJob<E> jobs[2] = {{go, KS_GT, -1, 1.f, false}, {k, -1, KS_KC, 1.f, false}};
+        prep_wave_jobs<KsRing, 1, 2, SP, 3, E>(smem, jobs, T, nstages, lane, tok0_of, smem + KS_SCRATCH);
     } else if (wave == 7) {
-        const PrepJob jobs[2] = {{dv, KS_NUT, -1, -1.f, false}, {q, -1, KS_QC, 1.f, false}};
-        prep_wave_jobs<KsRing, 1, 2, SP, 3>(smem, jobs, T, nstages, lane, tok0_of, smem + KS_SCRATCH + 2 * TM_TILE);
+        const PrepJob<E> jobs[2] = {{dv, KS_NUT, -1, -1.f, false}, {q, -1, KS_QC, 1.f, false}};
+        prep_wave_jobs<KsRing, 1, 2, SP, 3, E>(smem, jobs, T, nstages, lane, tok0_of, smem + KS_SCRATCH + 2 * TM_TILE);
     }
 }
 
 }  // namespace
 
-template <bool SP> static int launch_backward(const DfwBwdArgs &a, hipStream_t stream) {
-    auto value_side = dfw_chunk_bwd_value_kernel<SP>;
-    auto key_side = dfw_chunk_bwd_key_kernel<SP>;
+template <bool SP, typename E> static int launch_backward(const DfwBwdArgs &a, hipStream_t stream) {
+    auto value_side = dfw_chunk_bwd_value_kernel<SP, E>;
+    auto key_side = dfw_chunk_bwd_key_kernel<SP, E>;
     int rc = enable_lds(reinterpret_cast<const void *>(value_side), VsRing::SMEM, "hipFuncSetAttribute(delta-rule backward kernel, value side)");
     if (rc) return rc;
     if ((rc = enable_lds(reinterpret_cast<const void *>(key_side), KS_SMEM, "hipFuncSetAttribute(delta-rule backward kernel, key side)"))) return rc;
@@ -370,11 +375,20 @@ template <bool SP> static int launch_backward(const DfwBwdArgs &a, hipStream_t s
     return check_hip(hipGetLastError(), "dfw_chunk_bwd_key_kernel launch");
 }
 
-int dfw_chunk_backward(const DfwBwdArgs &a, bool split_operands, hipStream_t stream) {
+template <typename E> static int backward_of(const DfwBwdArgs &a, bool split_operands, hipStream_t stream) {
+    return split_operands ? launch_backward<true, E>(a, stream) : launch_backward<false, E>(a, stream);
+}
+
+int dfw_chunk_backward(const DfwBwdArgs &a, int dtype, bool split_operands, hipStream_t stream) {
     if (a.D != CH_N || a.M != CH_N) return fail(T2FW_ERR_UNSUPPORTED, "the block-wise delta-rule kernels take D = M = 64");
     if (a.T * CH_N >= 0x7fffffffLL || a.B > 0x1fffffffLL)
         return fail(T2FW_ERR_UNSUPPORTED, "B=%lld T=%lld is too large for the block-wise delta-rule kernels", (long long)a.B, (long long)a.T);
-    return split_operands ? launch_backward<true>(a, stream) : launch_backward<false>(a, stream);
+    switch (dtype) {
+    case T2FW_F32: return backward_of<ElF32>(a, split_operands, stream);
+    case T2FW_F16: return backward_of<El16<Fp16>>(a, split_operands, stream);
+    case T2FW_BF16: return backward_of<El16<Bf16>>(a, split_operands, stream);
+    default: return fail(T2FW_ERR_UNSUPPORTED, "the block-wise delta-rule kernels take fp32, fp16 and bf16 tensors");
+    }
 }
 
 }  // namespace t2fw

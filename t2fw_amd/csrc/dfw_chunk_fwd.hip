@@ -1,5 +1,5 @@
-// Forward pass of the delta rule on the matrix cores, D = M = 64, fp32 tensors (algebra and precision:
-// dfw_chunk.hpp).  Two workgroups per batch row, one per half of the value channels: the rows S[d, :] of the
+// Forward pass of the delta rule on the matrix cores, D = M = 64, fp32 / fp16 / bf16 tensors (algebra, precision
+// and element types: dfw_chunk.hpp).  Two workgroups per batch row, one per half of the value channels: the rows S[d, :] of the
 // state, and with them the columns of V, Delta and O, never interact.  A workgroup has six waves (eight are launched; two leave at once):
 //   two slab waves    each keeps 16 rows of the state in fp32 accumulators for the whole sequence; per block:
 //                     Delta = Tm V - K' S0^T, O = Q S0^T + Bq Delta, S += Delta^T K; they load V and store O
@@ -74,52 +74,52 @@ template <bool SP> __device__ __forceinline__ void structure_wave(unsigned char 
     }
 }
 
-template <bool SP> __device__ __forceinline__ void slab_wave(const DfwFwdArgs &p, unsigned char *smem, int64_t b, int d0, int nstages, int lane) {
+template <bool SP, typename E> __device__ __forceinline__ void slab_wave(const DfwFwdArgs &p, unsigned char *smem, int64_t b, int d0, int nstages, int lane) {
+    typedef typename E::elem elem;
     const int r = lane & 15, g = lane >> 4, d = d0 + r, T = (int)p.T;
     const floatx4 zero = {0.f, 0.f, 0.f, 0.f};
     // token addresses: a wave-uniform base per block plus the lane's fixed offset (first token 4 g, channel d)
-    const float *const v = reinterpret_cast<const float *>(p.v) + b * p.T * CH_N;
-    float *const out = reinterpret_cast<float *>(p.out) + b * p.T * CH_N;
-    float *const delta = reinterpret_cast<float *>(p.delta) + b * p.T * CH_N;
+    const elem *const v = reinterpret_cast<const elem *>(p.v) + b * p.T * CH_N;
+    elem *const out = reinterpret_cast<elem *>(p.out) + b * p.T * CH_N;
+    elem *const delta = reinterpret_cast<elem *>(p.delta) + b * p.T * CH_N;
     const u32 lane_off = (u32)(4 * g * CH_N + d);
     // S[j][e] = S[d][16 j + 4 g + e]
     floatx4 S[4];
     {
-        const float *s0 = reinterpret_cast<const float *>(p.s0) + (b * CH_N + d) * CH_N + 4 * g;
+        const elem *s0 = reinterpret_cast<const elem *>(p.s0) + (b * CH_N + d) * CH_N + 4 * g;
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            const float4 t = *reinterpret_cast<const float4 *>(s0 + 16 * j);
-            S[j] = floatx4{t.x, t.y, t.z, t.w};
-        }
+        for (int j = 0; j < 4; ++j) S[j] = E::load4(s0 + 16 * j);
     }
     // V of a stage: element [bb][e] is token (stage * DNB + bb) * 16 + 4 g + e; loaded one stage ahead into the
-    // register set the stage before has left
+    // register set the stage before has left, as loaded (converted where the stage uses it)
     // (unconditional loads: tokens at or past T are read from token T - 1 and zeroed where they are used)
-    auto load_v = [&](floatx4 (&x)[DNB], int stage) {
+    struct VRaw {
+        elem x[DNB][4];
+    };
+    auto load_v = [&](VRaw &x, int stage) {
 #pragma unroll
         for (int bb = 0; bb < DNB; ++bb)
 #pragma unroll
-            for (int e = 0; e < 4; ++e) x[bb][e] = v[(size_t)min((stage * DNB + bb) * DL + 4 * g + e, T - 1) * CH_N + d];
+            for (int e = 0; e < 4; ++e) x.x[bb][e] = v[(size_t)min((stage * DNB + bb) * DL + 4 * g + e, T - 1) * CH_N + d];
     };
     // One stage.  FULL: every token of the stage is below T, and the body is free of branches: the waits that
     // the compiler places count outstanding memory operations along every path, so a path that skips stores
     // would make the loads of the next stage wait for the stores of this one.
-    auto stage_body = [&](auto full, int stage, floatx4 (&vcur)[DNB], floatx4 (&vnxt)[DNB]) {
+    auto stage_body = [&](auto full, int stage, VRaw &vraw, VRaw &vnxt) {
         constexpr bool FULL = decltype(full)::value;
         load_v(vnxt, min(stage + 1, nstages - 1));
 #pragma unroll
         for (int bb = 0; bb < DNB; ++bb) {
             const int tok0 = (stage * DNB + bb) * DL;
-            if constexpr (!FULL) {
+            floatx4 vcur;
 #pragma unroll
-                for (int e = 0; e < 4; ++e) vcur[bb][e] = tok0 + 4 * g + e < T ? vcur[bb][e] : 0.f;
-            }
+            for (int e = 0; e < 4; ++e) vcur[e] = (FULL || tok0 + 4 * g + e < T) ? E::f(vraw.x[bb][e]) : 0.f;
             const unsigned char *raw = raw_block(smem, stage, bb);
             const unsigned char *st = st_block(smem, stage, bb);
             const TmTile<SP> QT(raw + FW_QT), KP(st + FW_KP);
             const CmTile<SP> KC(raw + FW_KC);
             // Delta[tok 4g+e][d] = Tm V - K' S0^T: only the second term waits for the state
-            const floatx4 tv = mma16(st_load<SP>(st + FW_TT, lane), split4<SP>(vcur[bb]), zero);
+            const floatx4 tv = mma16(st_load<SP>(st + FW_TT, lane), split4<SP>(vcur), zero);
             const Sp4<SP> sb0 = cat(split4<SP>(S[0]), split4<SP>(S[1])), sb1 = cat(split4<SP>(S[2]), split4<SP>(S[3]));
             const floatx4 ks = mma32(KP.acc_order(r, g, 1), sb1, mma32(KP.acc_order(r, g, 0), sb0, zero));
             const floatx4 dl = tv - ks;
@@ -127,12 +127,12 @@ template <bool SP> __device__ __forceinline__ void slab_wave(const DfwFwdArgs &p
             // O = Q S0^T + Bq Delta
             const floatx4 qs = mma32(QT.acc_order(r, g, 1), sb1, mma32(QT.acc_order(r, g, 0), sb0, zero));
             const floatx4 o = qs + mma16(st_load<SP>(st + FW_BQT, lane), dls, zero);
-            float *const ob = out + (size_t)tok0 * CH_N, *const db = delta + (size_t)tok0 * CH_N;      // wave-uniform
+            elem *const ob = out + (size_t)tok0 * CH_N, *const db = delta + (size_t)tok0 * CH_N;      // wave-uniform
 #pragma unroll
             for (int e = 0; e < 4; ++e)
                 if (FULL || tok0 + 4 * g + e < T) {
-                    ob[lane_off + e * CH_N] = o[e];
-                    db[lane_off + e * CH_N] = dl[e];
+                    ob[lane_off + e * CH_N] = E::e(o[e]);
+                    db[lane_off + e * CH_N] = E::e(dl[e]);
                 }
             // S += Delta^T K
 #pragma unroll
@@ -140,7 +140,7 @@ template <bool SP> __device__ __forceinline__ void slab_wave(const DfwFwdArgs &p
         }
         __syncthreads();
     };
-    floatx4 v_a[DNB], v_b[DNB];
+    VRaw v_a, v_b;
     load_v(v_a, 0);
     __syncthreads();        // ticks 0 and 1: the prep and matrix waves fill the pipeline
     __syncthreads();
@@ -160,22 +160,23 @@ template <bool SP> __device__ __forceinline__ void slab_wave(const DfwFwdArgs &p
     } else if (stage < nstages) {
         stage_body(std::false_type{}, stage, v_a, v_b);
     }
-    float *fin = reinterpret_cast<float *>(p.final_state) + (b * CH_N + d) * CH_N + 4 * g;
+    elem *fin = reinterpret_cast<elem *>(p.final_state) + (b * CH_N + d) * CH_N + 4 * g;
 #pragma unroll
-    for (int j = 0; j < 4; ++j) *reinterpret_cast<float4 *>(fin + 16 * j) = make_float4(S[j][0], S[j][1], S[j][2], S[j][3]);
+    for (int j = 0; j < 4; ++j) E::store4(fin + 16 * j, S[j]);
 }
 
 // blockIdx = half * rows_padded + row with rows_padded a multiple of 8: the two halves of a row land on the
 // same XCD and share its L2 for K and Q, which both read
-template <bool SP> __global__ __launch_bounds__(FW_THREADS) void dfw_chunk_fwd_kernel(DfwFwdArgs p, int rows_padded) {
+template <bool SP, typename E> __global__ __launch_bounds__(FW_THREADS) void dfw_chunk_fwd_kernel(DfwFwdArgs p, int rows_padded) {
+    typedef typename E::elem elem;
     extern __shared__ __align__(16) unsigned char smem[];
     const int half = (int)blockIdx.x >= rows_padded ? 1 : 0;
     const int64_t b = (int)blockIdx.x - half * rows_padded;
     if (b >= p.B) return;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
     const int T = (int)p.T, nstages = (T + DL * DNB - 1) / (DL * DNB);
-    const float *const k = reinterpret_cast<const float *>(p.k) + b * p.T * CH_N;
-    const float *const q = reinterpret_cast<const float *>(p.q) + b * p.T * CH_N;
+    const elem *const k = reinterpret_cast<const elem *>(p.k) + b * p.T * CH_N;
+    const elem *const q = reinterpret_cast<const elem *>(p.q) + b * p.T * CH_N;
     // Every wave that stays executes nstages + 2 workgroup barriers.  Wave i runs on SIMD i % 4: the slab waves,
     // whose chain of dependent steps sets the kernel's duration, get SIMDs 0 and 1 to themselves (waves 4 and 5
     // leave at once; a workgroup barrier waits only for the waves that are left), the matrix waves and the
@@ -183,22 +184,22 @@ template <bool SP> __global__ __launch_bounds__(FW_THREADS) void dfw_chunk_fwd_k
     static_assert(DNB == 2, "one matrix wave per block of a stage");
     auto tok0_of = [](int stage, int bb) { return (stage * DNB + bb) * DL; };
     if (wave < 2)
-        slab_wave<SP>(p, smem, b, 32 * half + 16 * wave, nstages, lane);
+        slab_wave<SP, E>(p, smem, b, 32 * half + 16 * wave, nstages, lane);
     else if (wave < 4)
         structure_wave<SP>(smem, nstages, wave - 2, lane);
     else if (wave == 6) {          // K: token-major, and channel-major derived from it
-        const PrepJob jobs[1] = {{k, FW_KT, FW_KC, 1.f, false}};
-        prep_wave_jobs<FwRing, DNB, 1, SP, 3>(smem, jobs, T, nstages, lane, tok0_of, nullptr);
+        const PrepJob<E> jobs[1] = {{k, FW_KT, FW_KC, 1.f, false}};
+        prep_wave_jobs<FwRing, DNB, 1, SP, 3, E>(smem, jobs, T, nstages, lane, tok0_of, nullptr);
     } else if (wave == 7) {        // Q: token-major
-        const PrepJob jobs[1] = {{q, FW_QT, -1, 1.f, false}};
-        prep_wave_jobs<FwRing, DNB, 1, SP, 3>(smem, jobs, T, nstages, lane, tok0_of, nullptr);
+        const PrepJob<E> jobs[1] = {{q, FW_QT, -1, 1.f, false}};
+        prep_wave_jobs<FwRing, DNB, 1, SP, 3, E>(smem, jobs, T, nstages, lane, tok0_of, nullptr);
     }
 }
 
 }  // namespace
 
-template <bool SP> static int launch_forward(const DfwFwdArgs &a, hipStream_t stream) {
-    auto kern = dfw_chunk_fwd_kernel<SP>;
+template <bool SP, typename E> static int launch_forward(const DfwFwdArgs &a, hipStream_t stream) {
+    auto kern = dfw_chunk_fwd_kernel<SP, E>;
     int rc = enable_lds(reinterpret_cast<const void *>(kern), FW_SMEM, "hipFuncSetAttribute(delta-rule forward kernel)");
     if (rc) return rc;
     const int rows_padded = (int)((a.B + 7) / 8 * 8);
@@ -206,11 +207,20 @@ template <bool SP> static int launch_forward(const DfwFwdArgs &a, hipStream_t st
     return check_hip(hipGetLastError(), "dfw_chunk_fwd_kernel launch");
 }
 
-int dfw_chunk_forward(const DfwFwdArgs &a, bool split_operands, hipStream_t stream) {
+template <typename E> static int forward_of(const DfwFwdArgs &a, bool split_operands, hipStream_t stream) {
+    return split_operands ? launch_forward<true, E>(a, stream) : launch_forward<false, E>(a, stream);
+}
+
+int dfw_chunk_forward(const DfwFwdArgs &a, int dtype, bool split_operands, hipStream_t stream) {
     if (a.D != CH_N || a.M != CH_N) return fail(T2FW_ERR_UNSUPPORTED, "the block-wise delta-rule kernels take D = M = 64");
     if (a.T * CH_N >= 0x7fffffffLL || a.B > 0x1fffffffLL)
         return fail(T2FW_ERR_UNSUPPORTED, "B=%lld T=%lld is too large for the block-wise delta-rule kernels", (long long)a.B, (long long)a.T);
-    return split_operands ? launch_forward<true>(a, stream) : launch_forward<false>(a, stream);
+    switch (dtype) {
+    case T2FW_F32: return forward_of<ElF32>(a, split_operands, stream);
+    case T2FW_F16: return forward_of<El16<Fp16>>(a, split_operands, stream);
+    case T2FW_BF16: return forward_of<El16<Bf16>>(a, split_operands, stream);
+    default: return fail(T2FW_ERR_UNSUPPORTED, "the block-wise delta-rule kernels take fp32, fp16 and bf16 tensors");
+    }
 }
 
 }  // namespace t2fw

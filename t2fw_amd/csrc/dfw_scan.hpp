@@ -21,8 +21,9 @@ struct DfwBwdArgs {
 
 int dfw_forward(const DfwFwdArgs &a, int dtype, hipStream_t stream);
 int dfw_backward(const DfwBwdArgs &a, int dtype, hipStream_t stream);
-// block-wise matrix-core kernels: D = M = 64, fp32 tensors, 16-byte aligned pointers (dfw_chunk_fwd.hip, dfw_chunk_bwd.hip)
-int dfw_chunk_forward(const DfwFwdArgs &a, bool split_operands, hipStream_t stream);
-int dfw_chunk_backward(const DfwBwdArgs &a, bool split_operands, hipStream_t stream);
+// block-wise matrix-core kernels: D = M = 64, fp32 / fp16 / bf16 tensors, 16-byte aligned pointers (dfw_chunk_fwd.hip,
+// dfw_chunk_bwd.hip)
+int dfw_chunk_forward(const DfwFwdArgs &a, int dtype, bool split_operands, hipStream_t stream);
+int dfw_chunk_backward(const DfwBwdArgs &a, int dtype, bool split_operands, hipStream_t stream);
 
 }  // namespace t2fw

@@ -1,5 +1,5 @@
-"""GPU parity of the block-wise matrix-core kernels of the delta rule (D = M = 64, fp32 tensors) against
-the CPU oracle (fp64, same inputs), through the C ABI.  The operands of every contraction are split into a
+"""GPU parity of the block-wise matrix-core kernels of the delta rule (D = M = 64; fp32 tensors, and fp16 / bf16
+ones in the tests at the end) against the CPU oracle (fp64, same inputs), through the C ABI.  The operands of every contraction are split into a
 bf16 head and remainder, so the results are held to the tolerance of the exact per-step kernels
 (tests/test_dfw_gpu.py), not to a 16-bit one; the exact kernels (flag 1) are run on the same inputs."""
 import pytest
@@ -111,6 +111,68 @@ def test_single_bf16_operand_mode(B, T):
         err = (got.double().cpu() - ref.double()).abs().max().item()
         scale = ref.double().abs().max().item()
         assert err <= 1e-2 * scale, "%s: max error %.3e against max|ref| %.3e" % (n, err, scale)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("B,T", [(3, 1), (3, 17), (2, 100), (9, 257), (2, 1024)])
+def test_16_bit_tensors(dtype, B, T):
+    """fp16 / bf16 tensors run the same block-wise kernels (loads and stores convert; all arithmetic as for fp32
+    tensors).  Against the fp64 oracle on the same 16-bit inputs, to the tolerance of the exact per-step kernels
+    for the type; the saved deltas and the final state that the backward starts from are 16-bit there as here.
+    The error of the block-wise kernels stays within twice that of the exact kernels on the same inputs (both are
+    dominated by the rounding of what is stored), and flag 16 selects other kernels."""
+    q, k, v, s, go, gs = make_inputs(B, T, 64, 64, dtype, seed=600 + T)
+    r_out, r_fin, r_grads = dfw_reference_grads(q, k, v, s, go, gs)
+    r_delta = dfw_deltas(q.double(), k.double(), v.double(), s.double())
+    tol = TOL_DFW[dtype]
+    refs = [("outputs", r_out), ("final_state", r_fin), ("delta", r_delta)] + list(zip(NAMES, r_grads))
+    worst = {}
+    for flags in (1, 0, 16):
+        out, fin, delta, grads = run_abi(q, k, v, s, go, gs, flags)
+        got = [out, fin, delta] + grads
+        for (n, r), t in zip(refs, got):
+            assert t.dtype == dtype
+            assert_close(t, r, dtype, "%s (flags %d)" % (n, flags), tol=tol)
+            worst[(flags, n)] = ((t.double().cpu() - r.double()).abs().max() / r.double().abs().max()).item()
+    for n, _ in refs:
+        floor = 2.0 ** (-11 if dtype == torch.float16 else -8)          # one rounding of the largest element
+        assert worst[(0, n)] <= 2.0 * max(worst[(1, n)], floor), (n, worst[(0, n)], worst[(1, n)])
+    if T > 1:
+        assert not torch.equal(run_abi(q, k, v, s, go, gs, 0)[0], run_abi(q, k, v, s, go, gs, 16)[0])
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_16_bit_tensors_through_the_autograd_function(dtype):
+    """DFWFunction on 16-bit tensors: fp16 with the default (split) operands, bf16 with single bf16 operands
+    (flag 16; the wrapper's choice for that type) -- bit-identical to the C-ABI call with those flags, and inside
+    the type's tolerance against the oracle."""
+    from t2fw.functional_dfw import DFWFunction
+    q, k, v, s, go, gs = make_inputs(5, 200, 64, 64, dtype, seed=19)
+    ins = [t.cuda().requires_grad_(True) for t in (q, k, v, s)]
+    out, fin = DFWFunction.apply(*ins)
+    torch.autograd.backward([out, fin], [go.cuda(), gs.cuda()])
+    torch.cuda.synchronize()
+    r_out, r_fin, r_grads = dfw_reference_grads(q, k, v, s, go, gs)
+    assert out.dtype == dtype and fin.dtype == dtype
+    assert_close(out, r_out, dtype, "outputs", tol=TOL_DFW[dtype])
+    assert_close(fin, r_fin, dtype, "final_state", tol=TOL_DFW[dtype])
+    for n, t, r in zip(NAMES, ins, r_grads):
+        assert t.grad.dtype == dtype
+        assert_close(t.grad, r, dtype, n, tol=TOL_DFW[dtype])
+    a_out, a_fin, _, a_grads = run_abi(q, k, v, s, go, gs, flags=16 if dtype == torch.bfloat16 else 0)
+    assert torch.equal(out, a_out) and torch.equal(fin, a_fin)
+    for t, g in zip(ins, a_grads):
+        assert torch.equal(t.grad, g)
+
+
+def test_the_wrapper_s_flag_choice_yields_to_the_environment(monkeypatch):
+    from t2fw_amd import _lib
+    from t2fw_amd.functional_dfw import _dfw_flags
+    monkeypatch.delenv("T2FW_FLAGS", raising=False)
+    assert _dfw_flags(torch.bfloat16) == _lib.FLAG_BF16_OPERANDS
+    assert _dfw_flags(torch.float16) == 0 and _dfw_flags(torch.float32) == 0
+    monkeypatch.setenv("T2FW_FLAGS", "1")
+    assert _dfw_flags(torch.bfloat16) == 1
 
 
 def test_autograd_function_uses_the_block_wise_kernels():
