@@ -350,6 +350,60 @@ def lfw_apply_16bit(value, forget, query, key, f_key, state, dtype=torch.float16
     return LFW16Function.apply(value, forget, query, key, f_key, state, dtype)
 
 
+def lfw_apply_blocked(value, forget, query, key, f_key, state):
+    """``LFWFunction.apply`` for fp16 / bf16 tensors whose value and key widths are not 64, on the matrix-core
+    kernels, which take 64 x 64 states only.  The recurrence does not couple the rows of the state with each
+    other, nor its columns: S[d, k] sees x[d], f[d], k[k], f_key[k] only, and o[d] is a sum over k.  So a
+    D x K state is cut into (D / 64) x (K / 64) blocks of 64 x 64, each block is one independent recurrence on
+    channels 64 i .. 64 i + 63 of the value side and 64 j .. 64 j + 63 of the key side, and the outputs of the
+    blocks of a row of blocks add up.  The blocks go through ``LFWHeadsFunction`` as heads (one launch for all of
+    them); the copies that bring the channels into that layout, the sum over the key blocks and all of their
+    gradients are plain tensor operations.  Widths that are not multiples of 64 are padded (values, keys, queries
+    and the state with zeros, gates with ones): correct, and as expensive as the padded width.
+
+    An explicit choice of the caller, like ``lfw_apply_16bit``: results carry the matrix-core kernels' accuracy
+    (bf16 operands; and one more rounding to the tensors' type per key block in the outputs), where
+    ``LFWFunction.apply`` runs the exact per-step kernels for such shapes.  The reference has one kernel for every
+    shape (t2fw/csrc/lfw_kernel.cu:105-121) and no counterpart of this."""
+    assert value.dtype in (torch.float16, torch.bfloat16), "the matrix-core kernels take fp16 / bf16 tensors"
+    return _blocked(value, forget, query, key, f_key, state)
+
+
+def _blocked(value, forget, query, key, f_key, state):
+    """The decomposition of ``lfw_apply_blocked`` (any tensor type: what it calls decides what runs)."""
+    assert value.shape == forget.shape and query.shape == key.shape and query.shape == f_key.shape
+    B, T, D = value.shape
+    K = query.shape[2]
+    assert tuple(state.shape) == (B, D, K)
+    nd, nk = -(-D // 64), -(-K // 64)
+    Dp, Kp = 64 * nd, 64 * nk
+
+    def widen(t, width, fill):
+        return t if t.shape[-1] == width else torch.nn.functional.pad(t, (0, width - t.shape[-1]), value=fill)
+
+    x, f = widen(value, Dp, 0.0), widen(forget, Dp, 1.0)
+    q, k, fk = widen(query, Kp, 0.0), widen(key, Kp, 0.0), widen(f_key, Kp, 1.0)
+    s = state
+    if Dp != D or Kp != K:
+        s = torch.nn.functional.pad(state, (0, Kp - K, 0, Dp - D))
+    def narrow(out, nxt):
+        if Dp == D and Kp == K:
+            return out, nxt
+        return out[..., :D].contiguous(), nxt[:, :D, :K].contiguous()
+
+    if nd == 1 and nk == 1:
+        return narrow(*LFWFunction.apply(x, f, q, k, fk, s))
+    # head h = i * nk + j: value block i with key block j
+    H = nd * nk
+    value_side = lambda t: t.view(B, T, nd, 1, 64).expand(B, T, nd, nk, 64).reshape(B, T, H, 64).contiguous()
+    key_side = lambda t: t.view(B, T, 1, nk, 64).expand(B, T, nd, nk, 64).reshape(B, T, H, 64).contiguous()
+    sb = s.view(B, nd, 64, nk, 64).permute(0, 1, 3, 2, 4).reshape(B, H, 64, 64).contiguous()
+    out_b, nxt_b = LFWHeadsFunction.apply(value_side(x), value_side(f), key_side(q), key_side(k), key_side(fk), sb)
+    out = out_b.view(B, T, nd, nk, 64).sum(dim=3).reshape(B, T, Dp)
+    nxt = nxt_b.view(B, nd, nk, 64, 64).permute(0, 1, 3, 2, 4).reshape(B, Dp, Kp)
+    return narrow(out, nxt)
+
+
 def lfw_step(x, f, query, key, f_key, state, out=None, inplace=True):
     """One generation step (T = 1) without autograd: x,f [B,D]; query,key,f_key [B,K];
     state [B,D,K] updated in place when ``inplace``.  Returns (out [B,D], state).
