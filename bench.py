@@ -21,7 +21,7 @@ roofline   = algorithmic bytes of the dominant call (the backward: four launches
              this run: `traffic_source` says so).  Against 8 TB/s.
 other_configs = after the headline's timed region (cfg3 only): cfg2, cfg4, cfg3 with the gates of the
              reference's tests, cfg5, the delta rule (default and single-operand mode) and cfg3's shape
-             with float32 tensors, and a 128 x 128 state through lfw_apply_blocked, each briefly.
+             with float32 tensors, and a 128 x 128 state (run as 64 x 64 blocks), each briefly.
 dfw        = the delta-rule kernels (forward + backward) at cfg3's shape in fp32, the dtype the
              reference tests them in (--dfw-bf16-operands: their opt-in single-operand mode;
              --dfw-dtype: 16-bit tensors through the same kernels).
@@ -599,51 +599,51 @@ def bench_float32(args, steps, warmup):
 
 
 def bench_blocked_widths(args, steps, warmup):
-    """A 128 x 128 state (B=24, T=1024, fp16: the state bytes of cfg3) through the autograd API:
-    LFWFunction.apply (exact kernels: the matrix-core kernels take 64 x 64 states) against lfw_apply_blocked
-    (four independent 64 x 64 blocks per row on the matrix-core kernels, the caller's explicit choice), and the
-    second one's error against the first's results."""
+    """A 128 x 128 state (B=24, T=1024, fp16: the state bytes of cfg3) through LFWFunction.apply + autograd:
+    as the library runs it (four independent 64 x 64 blocks per row on the matrix-core kernels) against the exact
+    per-step kernels (T2FW_FLAGS=1), and the first one's error against the second's results."""
     import torch
-    from t2fw_amd import LFWFunction, lfw_apply_blocked
+    from t2fw_amd import LFWFunction
     from t2fw_amd.synthetic import make_config_inputs
     B, T, D, K = 24, 1024, 128, 128
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     os.environ["T2FW_CKPT_INTERVAL"] = str(args.ckpt_interval)
-    os.environ["T2FW_FLAGS"] = "0"
     x, f, q, k, fk, s0, go, gs = make_config_inputs(B, T, D, K, torch.float16, seed=0, gate_mean=2.0)
     leaves = [t.to(dev).requires_grad_(True) for t in (x, f, q, k, fk, s0)]
     go, gs = go.to(dev), gs.to(dev)
 
-    def run(fn, n):
+    def run(n):
         res = None
         for _ in range(n):
             for t in leaves:
                 t.grad = None
-            o, nx = fn(*leaves)
+            o, nx = LFWFunction.apply(*leaves)
             torch.autograd.backward([o, nx], [go, gs])
             res = [o.detach(), nx.detach()] + [t.grad for t in leaves]
         return res
     out, results = {}, {}
-    for name, fn, n in (("exact_kernels", LFWFunction.apply, max(2, steps // 4)), ("blocked", lfw_apply_blocked, steps)):
-        run(fn, warmup)
+    for name, flags, n in (("exact_kernels", "1", max(2, steps // 4)), ("blocks", "0", steps)):
+        os.environ["T2FW_FLAGS"] = flags
+        run(warmup)
         torch.cuda.synchronize()
         t0 = time.perf_counter()
-        results[name] = run(fn, n)
+        results[name] = run(n)
         torch.cuda.synchronize()
         ms = (time.perf_counter() - t0) / n * 1e3
         out[name] = {"value": round(B * T / ms / 1e3, 1), "unit": "Mtokens/s", "ms_per_step": round(ms, 5), "steps": n}
+    # recorded once into a HIP graph and replayed: the GPU time without the host's share
     side = torch.cuda.Stream()
     side.wait_stream(torch.cuda.current_stream())
     with torch.cuda.stream(side):
-        run(lfw_apply_blocked, 1)
+        run(1)
     torch.cuda.current_stream().wait_stream(side)
     torch.cuda.synchronize()
     for t in leaves:
         t.grad = None
     graph = torch.cuda.CUDAGraph()
     with torch.cuda.graph(graph):
-        o, nx = lfw_apply_blocked(*leaves)
+        o, nx = LFWFunction.apply(*leaves)
         torch.autograd.backward([o, nx], [go, gs])
     for _ in range(3):
         graph.replay()
@@ -653,14 +653,14 @@ def bench_blocked_widths(args, steps, warmup):
         graph.replay()
     torch.cuda.synchronize()
     ms = (time.perf_counter() - t0) / steps * 1e3
-    out["blocked"]["graph_replay_ms_per_step"] = round(ms, 5)
-    out["blocked"]["graph_replay_value"] = round(B * T / ms / 1e3, 1)
+    out["blocks"]["graph_replay_ms_per_step"] = round(ms, 5)
+    out["blocks"]["graph_replay_value"] = round(B * T / ms / 1e3, 1)
     worst = max(((a.double() - b.double()).abs().max() / b.double().abs().max()).item()
-                for a, b in zip(results["blocked"], results["exact_kernels"]))
-    out["blocked"]["max_abs_over_max_ref_vs_exact_kernels"] = round(worst, 6)
-    out["blocked"]["tensors"] = ["outputs", "next_state", "d_x", "d_f", "d_q", "d_k", "d_f_key", "d_state"]
-    out["workload"] = ("B=24 T=1024 D=K=128 float16, LFWFunction.apply / lfw_apply_blocked + autograd backward "
-                       "(host and allocations included)")
+                for a, b in zip(results["blocks"], results["exact_kernels"]))
+    out["blocks"]["max_abs_over_max_ref_vs_exact_kernels"] = round(worst, 6)
+    out["blocks"]["tensors"] = ["outputs", "next_state", "d_x", "d_f", "d_q", "d_k", "d_f_key", "d_state"]
+    out["workload"] = ("B=24 T=1024 D=K=128 float16, LFWFunction.apply + autograd backward (host and allocations "
+                       "included): 64 x 64 blocks on the matrix-core kernels / exact per-step kernels")
     return out
 
 

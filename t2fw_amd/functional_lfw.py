@@ -73,6 +73,88 @@ def _dtype_code(dtype):
         raise RuntimeError("t2fw: unsupported dtype %s" % dtype)
 
 
+# ---- widths that are multiples of 64 (other than 64 x 64) as independent 64 x 64 blocks -------------------
+# The recurrence couples neither the rows of the state nor its columns: S[d, k] sees x[d], f[d], k[k], f_key[k]
+# only, and o[d] is a sum over k.  A D x K state is (D / 64) (K / 64) independent 64 x 64 recurrences -- value
+# channels 64 i .. 64 i + 63 with key channels 64 j .. 64 j + 63 -- whose outputs add up over j.  For fp16 / bf16
+# tensors the blocks run as heads (h = i * nk + j) through the head-strided entry points, i.e. on the matrix-core
+# kernels, which take 64 x 64 states only; the exact per-step kernels that would otherwise serve such widths take
+# 4.1 ms for a forward + backward at B=24, T=1024, D=K=128 where the blocks take 0.24 ms.  The reference has one
+# kernel for every shape (t2fw/csrc/lfw_kernel.cu:105-121).
+def _block_counts(value, query, flags):
+    """(D / 64, K / 64) if tensors of these widths run as blocks, else None"""
+    D, K = value.shape[-1], query.shape[-1]
+    if value.dim() != 3 or value.dtype not in (torch.float16, torch.bfloat16) or (flags & _lib.FLAG_FORCE_SCAN):
+        return None
+    if D % 64 or K % 64 or D == 0 or K == 0 or (D == 64 and K == 64):
+        return None
+    return D // 64, K // 64
+
+
+def _value_blocks(t, nd, nk):
+    B, T = t.shape[:2]
+    return t.view(B, T, nd, 1, 64).expand(B, T, nd, nk, 64).reshape(B, T, nd * nk, 64).contiguous()
+
+
+def _key_blocks(t, nd, nk):
+    B, T = t.shape[:2]
+    return t.view(B, T, 1, nk, 64).expand(B, T, nd, nk, 64).reshape(B, T, nd * nk, 64).contiguous()
+
+
+def _state_blocks(s, nd, nk):
+    return s.view(s.shape[0], nd, 64, nk, 64).permute(0, 1, 3, 2, 4).reshape(s.shape[0], nd * nk, 64, 64).contiguous()
+
+
+def _state_from_blocks(sb, nd, nk):
+    return sb.view(sb.shape[0], nd, nk, 64, 64).permute(0, 1, 3, 2, 4).reshape(sb.shape[0], 64 * nd, 64 * nk)
+
+
+def _sum_key_blocks(tb, nd, nk):
+    """[B,T,nd*nk,64] -> [B,T,64*nd]: what the blocks of one row of blocks hold adds up (fp32 accumulation)"""
+    B, T = tb.shape[:2]
+    return tb.view(B, T, nd, nk, 64).sum(dim=3).view(B, T, 64 * nd)
+
+
+def _sum_value_blocks(tb, nd, nk):
+    B, T = tb.shape[:2]
+    return tb.view(B, T, nd, nk, 64).sum(dim=2).view(B, T, 64 * nk)
+
+
+class _BlockedCall:
+    """What a forward call on blocks leaves for its backward call: the block copies of the six inputs (made once,
+    not again in the backward) and the hints of the call underneath.  Travels in the ``hints`` slot."""
+    __slots__ = ("tensors", "hints")
+
+    def __init__(self, tensors, hints):
+        self.tensors = tensors
+        self.hints = hints
+
+
+def _lfw_forward_blocked(value, forget, query, key, f_key, state, need_grad, blocks):
+    nd, nk = blocks
+    tensors = (_value_blocks(value, nd, nk), _value_blocks(forget, nd, nk), _key_blocks(query, nd, nk),
+               _key_blocks(key, nd, nk), _key_blocks(f_key, nd, nk), _state_blocks(state, nd, nk))
+    out_b, nxt_b, ckpt, C, flags, hints = _lfw_forward(*tensors, need_grad, heads=True)
+    kept = _BlockedCall(tensors, hints) if need_grad else None
+    return _sum_key_blocks(out_b, nd, nk), _state_from_blocks(nxt_b, nd, nk), ckpt, C, flags, kept
+
+
+def _lfw_backward_blocked(grad_output, grad_state, value, forget, query, key, f_key, state, ckpt, C, flags, kept, blocks):
+    """The adjoint of the copies is the sum over the blocks that share a channel."""
+    nd, nk = blocks
+    if isinstance(kept, _BlockedCall):
+        tensors, hints = kept.tensors, kept.hints
+    else:
+        tensors = (_value_blocks(value, nd, nk), _value_blocks(forget, nd, nk), _key_blocks(query, nd, nk),
+                   _key_blocks(key, nd, nk), _key_blocks(f_key, nd, nk), _state_blocks(state, nd, nk))
+        hints = None
+    d_xb, d_fb, d_qb, d_kb, d_fkb, d_sb = _lfw_backward(
+        _value_blocks(grad_output, nd, nk), _state_blocks(grad_state, nd, nk), *tensors, ckpt, C, flags, heads=True,
+        hints=hints)
+    return (_sum_key_blocks(d_xb, nd, nk), _sum_key_blocks(d_fb, nd, nk), _sum_value_blocks(d_qb, nd, nk),
+            _sum_value_blocks(d_kb, nd, nk), _sum_value_blocks(d_fkb, nd, nk), _state_from_blocks(d_sb, nd, nk))
+
+
 def _lfw_forward(value, forget, query, key, f_key, state, need_grad, heads=False):
     """Checks as in t2fw/functional_lfw.py:42-49 and t2fw/csrc/lfw.cpp:24-26,36-41, then the forward
     kernels.  heads=False: x,f [B,T,D]; q,k,f_key [B,T,K]; state [B,D,K].  heads=True: x,f [B,T,H,D];
@@ -102,9 +184,13 @@ def _lfw_forward(value, forget, query, key, f_key, state, need_grad, heads=False
         raise RuntimeError("t2fw: inconsistent shapes x %s, query %s, state %s"
                            % (tuple(value.shape), tuple(query.shape), tuple(state.shape)))
     code = _dtype_code(value.dtype)
+    flags = _flags()
+    if not heads:
+        blocks = _block_counts(value, query, flags)
+        if blocks is not None:
+            return _lfw_forward_blocked(value, forget, query, key, f_key, state, need_grad, blocks)
     lib = _lib.load()
     C = _ckpt_interval()
-    flags = _flags()
     dev = value.device
     nc, ws_bytes, _, regions = _sizes(B * H, T, D, K, C, code, flags)
     with _on_device(dev):
@@ -142,6 +228,11 @@ def _lfw_backward(grad_output, grad_state, value, forget, query, key, f_key, sta
     assert grad_output.dtype == value.dtype
     grad_output = grad_output.contiguous()
     grad_state = grad_state.contiguous()
+    if not heads:
+        blocks = _block_counts(value, query, flags)
+        if blocks is not None:
+            return _lfw_backward_blocked(grad_output, grad_state, value, forget, query, key, f_key, state, ckpt, C,
+                                         flags, hints, blocks)
     B, T = value.shape[:2]
     H = value.shape[2] if heads else 1
     D, K = value.shape[-1], query.shape[-1]
@@ -172,7 +263,10 @@ def _lfw_backward(grad_output, grad_state, value, forget, query, key, f_key, sta
 
 class LFWFunction(torch.autograd.Function):
     """Decay update rule S_t = S_{t-1} * (f_t (x) f_key_t) + x_t (x) k_t, o_t = S_t q_t.
-    Inputs are already gated (no sigmoid is applied here), as in the reference."""
+    Inputs are already gated (no sigmoid is applied here), as in the reference.
+    fp16 / bf16 tensors with D = K = 64 run on the matrix-core kernels, those whose widths are other multiples
+    of 64 as independent 64 x 64 blocks on the same kernels (``_block_counts`` above), everything else on the
+    exact per-step kernels; T2FW_FLAGS=1 keeps the exact kernels for every shape."""
 
     @staticmethod
     def forward(ctx, value, forget, query, key, f_key, state):
@@ -350,58 +444,28 @@ def lfw_apply_16bit(value, forget, query, key, f_key, state, dtype=torch.float16
     return LFW16Function.apply(value, forget, query, key, f_key, state, dtype)
 
 
-def lfw_apply_blocked(value, forget, query, key, f_key, state):
-    """``LFWFunction.apply`` for fp16 / bf16 tensors whose value and key widths are not 64, on the matrix-core
-    kernels, which take 64 x 64 states only.  The recurrence does not couple the rows of the state with each
-    other, nor its columns: S[d, k] sees x[d], f[d], k[k], f_key[k] only, and o[d] is a sum over k.  So a
-    D x K state is cut into (D / 64) x (K / 64) blocks of 64 x 64, each block is one independent recurrence on
-    channels 64 i .. 64 i + 63 of the value side and 64 j .. 64 j + 63 of the key side, and the outputs of the
-    blocks of a row of blocks add up.  The blocks go through ``LFWHeadsFunction`` as heads (one launch for all of
-    them); the copies that bring the channels into that layout, the sum over the key blocks and all of their
-    gradients are plain tensor operations.  Widths that are not multiples of 64 are padded (values, keys, queries
-    and the state with zeros, gates with ones): correct, and as expensive as the padded width.
-
-    An explicit choice of the caller, like ``lfw_apply_16bit``: results carry the matrix-core kernels' accuracy
-    (bf16 operands; and one more rounding to the tensors' type per key block in the outputs), where
-    ``LFWFunction.apply`` runs the exact per-step kernels for such shapes.  The reference has one kernel for every
-    shape (t2fw/csrc/lfw_kernel.cu:105-121) and no counterpart of this."""
+def lfw_apply_padded(value, forget, query, key, f_key, state):
+    """``LFWFunction.apply`` for fp16 / bf16 tensors whose value or key width is not a multiple of 64, on the
+    matrix-core kernels: the widths are padded up to the next multiple of 64 (values, keys, queries and the state
+    with zeros, gates with ones -- the padded channels stay zero and add nothing), the padded tensors run as
+    64 x 64 blocks (``LFWFunction.apply`` does that by itself for multiples of 64), and the results are cut back.
+    Correct for any width, and as expensive as the padded width: a 32 x 32 state costs what a 64 x 64 one costs,
+    which is still a quarter of the exact per-step kernels' time at B=96, T=1024.  An explicit choice of the
+    caller, because the results carry the matrix-core kernels' accuracy where ``LFWFunction.apply`` runs the exact
+    kernels for such widths.  Padding, cutting and their gradients are plain tensor operations."""
     assert value.dtype in (torch.float16, torch.bfloat16), "the matrix-core kernels take fp16 / bf16 tensors"
-    return _blocked(value, forget, query, key, f_key, state)
-
-
-def _blocked(value, forget, query, key, f_key, state):
-    """The decomposition of ``lfw_apply_blocked`` (any tensor type: what it calls decides what runs)."""
     assert value.shape == forget.shape and query.shape == key.shape and query.shape == f_key.shape
     B, T, D = value.shape
     K = query.shape[2]
     assert tuple(state.shape) == (B, D, K)
-    nd, nk = -(-D // 64), -(-K // 64)
-    Dp, Kp = 64 * nd, 64 * nk
-
-    def widen(t, width, fill):
-        return t if t.shape[-1] == width else torch.nn.functional.pad(t, (0, width - t.shape[-1]), value=fill)
-
-    x, f = widen(value, Dp, 0.0), widen(forget, Dp, 1.0)
-    q, k, fk = widen(query, Kp, 0.0), widen(key, Kp, 0.0), widen(f_key, Kp, 1.0)
-    s = state
-    if Dp != D or Kp != K:
-        s = torch.nn.functional.pad(state, (0, Kp - K, 0, Dp - D))
-    def narrow(out, nxt):
-        if Dp == D and Kp == K:
-            return out, nxt
-        return out[..., :D].contiguous(), nxt[:, :D, :K].contiguous()
-
-    if nd == 1 and nk == 1:
-        return narrow(*LFWFunction.apply(x, f, q, k, fk, s))
-    # head h = i * nk + j: value block i with key block j
-    H = nd * nk
-    value_side = lambda t: t.view(B, T, nd, 1, 64).expand(B, T, nd, nk, 64).reshape(B, T, H, 64).contiguous()
-    key_side = lambda t: t.view(B, T, 1, nk, 64).expand(B, T, nd, nk, 64).reshape(B, T, H, 64).contiguous()
-    sb = s.view(B, nd, 64, nk, 64).permute(0, 1, 3, 2, 4).reshape(B, H, 64, 64).contiguous()
-    out_b, nxt_b = LFWHeadsFunction.apply(value_side(x), value_side(f), key_side(q), key_side(k), key_side(fk), sb)
-    out = out_b.view(B, T, nd, nk, 64).sum(dim=3).reshape(B, T, Dp)
-    nxt = nxt_b.view(B, nd, nk, 64, 64).permute(0, 1, 3, 2, 4).reshape(B, Dp, Kp)
-    return narrow(out, nxt)
+    Dp, Kp = 64 * -(-D // 64), 64 * -(-K // 64)
+    if Dp == D and Kp == K:
+        return LFWFunction.apply(value, forget, query, key, f_key, state)
+    pad = torch.nn.functional.pad
+    out, nxt = LFWFunction.apply(pad(value, (0, Dp - D)), pad(forget, (0, Dp - D), value=1.0), pad(query, (0, Kp - K)),
+                                 pad(key, (0, Kp - K)), pad(f_key, (0, Kp - K), value=1.0),
+                                 pad(state, (0, Kp - K, 0, Dp - D)))
+    return out[..., :D].contiguous(), nxt[:, :D, :K].contiguous()
 
 
 def lfw_step(x, f, query, key, f_key, state, out=None, inplace=True):

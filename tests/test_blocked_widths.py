@@ -1,7 +1,8 @@
-"""``lfw_apply_blocked``: value / key widths other than 64 as independent 64 x 64 blocks.
+"""Value / key widths other than 64 on the matrix-core kernels: multiples of 64 as independent 64 x 64 blocks
+(what ``LFWFunction.apply`` does by itself for fp16 / bf16 tensors), other widths padded (``lfw_apply_padded``).
 
-CPU: the decomposition itself (which channels go to which block, how outputs, states and gradients come back),
-with the two autograd functions it calls replaced by the oracle's plain-torch recurrence, in float64 against the
+CPU: the decomposition itself -- which channels go to which block, how outputs, states and gradients come back --
+with the two kernel calls replaced by the oracle's plain-torch recurrence on the blocks, in float64, against the
 same recurrence on the undivided tensors.  GPU: the real kernels against the C oracle."""
 import pytest
 import torch
@@ -9,62 +10,75 @@ import torch
 from oracle.lfw_ref import lfw_reference
 from tests.lfw_cases import make_config_inputs
 
-SHAPES = [(128, 64), (64, 128), (128, 128), (192, 64), (64, 64), (32, 32), (100, 70), (1, 1), (65, 64)]
+
+def _fold(t):
+    B, T, H, W = t.shape
+    return t.transpose(1, 2).reshape(B * H, T, W)
 
 
-class _HeadsByOracle:
-    @staticmethod
-    def apply(x, f, q, k, fk, s):
-        B, T, H, _ = x.shape
-        fold = lambda t: t.transpose(1, 2).reshape(B * H, T, 64)
-        out, nxt = lfw_reference(fold(x), fold(f), fold(q), fold(k), fold(fk), s.reshape(B * H, 64, 64))
-        return out.view(B, H, T, 64).transpose(1, 2), nxt.view(B, H, 64, 64)
+def _heads_forward_by_oracle(x, f, q, k, fk, s, need_grad, heads=False):
+    assert heads and x.is_contiguous() and k.is_contiguous() and s.is_contiguous()
+    B, T, H, _ = x.shape
+    out, nxt = lfw_reference(_fold(x), _fold(f), _fold(q), _fold(k), _fold(fk), s.reshape(B * H, 64, 64))
+    return out.view(B, H, T, 64).transpose(1, 2).contiguous(), nxt.view(B, H, 64, 64), "ckpt", 64, 0, None
 
 
-class _RowsByOracle:
-    @staticmethod
-    def apply(x, f, q, k, fk, s):
-        return lfw_reference(x, f, q, k, fk, s)
+def _heads_backward_by_oracle(go, gs, x, f, q, k, fk, s, ckpt, C, flags, heads=False, hints=None):
+    assert heads and ckpt == "ckpt" and go.is_contiguous() and gs.is_contiguous()
+    B, T, H, _ = x.shape
+    leaves = [_fold(t).clone().requires_grad_(True) for t in (x, f, q, k, fk)] + [s.reshape(B * H, 64, 64).clone().requires_grad_(True)]
+    with torch.enable_grad():
+        out, nxt = lfw_reference(*leaves)
+        grads = torch.autograd.grad([out, nxt], leaves, [_fold(go), gs.reshape(B * H, 64, 64)])
+    unfold = lambda t: t.view(B, H, T, 64).transpose(1, 2).contiguous()
+    return tuple(unfold(g) for g in grads[:5]) + (grads[5].view(B, H, 64, 64),)
 
 
-@pytest.mark.parametrize("D,K", SHAPES)
+@pytest.mark.parametrize("D,K", [(128, 64), (64, 128), (128, 128), (192, 64), (64, 192), (256, 128)])
 def test_decomposition_is_the_same_recurrence(monkeypatch, D, K):
     from t2fw_amd import functional_lfw as F
-    monkeypatch.setattr(F, "LFWHeadsFunction", _HeadsByOracle)
-    monkeypatch.setattr(F, "LFWFunction", _RowsByOracle)
+    monkeypatch.setattr(F, "_lfw_forward", _heads_forward_by_oracle)
+    monkeypatch.setattr(F, "_lfw_backward", _heads_backward_by_oracle)
     B, T = 2, 9
     x, f, q, k, fk, s, go, gs = [t.double() for t in make_config_inputs(B, T, D, K, torch.float32, seed=D + K, state_std=0.5)]
-    results = []
-    for fn in (lfw_reference, None):          # None: the decomposition, whatever the tensor type
-        leaves = [t.clone().requires_grad_(True) for t in (x, f, q, k, fk, s)]
-        out, nxt = (fn or F._blocked)(*leaves)
-        torch.autograd.backward([out, nxt], [go, gs])
-        results.append([out.detach(), nxt.detach()] + [t.grad for t in leaves])
-    for a, b in zip(*results):
+    leaves = [t.clone().requires_grad_(True) for t in (x, f, q, k, fk, s)]
+    r_out, r_nxt = lfw_reference(*leaves)
+    torch.autograd.backward([r_out, r_nxt], [go, gs])
+    blocks = (D // 64, K // 64)
+    out, nxt, ckpt, C, flags, hints = F._lfw_forward_blocked(x, f, q, k, fk, s, True, blocks)
+    grads = F._lfw_backward_blocked(go, gs, x, f, q, k, fk, s, ckpt, C, flags, hints, blocks)
+    for a, b in zip([out, nxt] + list(grads), [r_out.detach(), r_nxt.detach()] + [t.grad for t in leaves]):
         assert a.shape == b.shape
         assert torch.allclose(a, b, rtol=1e-12, atol=1e-12)
 
 
-def test_16_bit_tensors_only():
-    from t2fw_amd import lfw_apply_blocked
-    x, f, q, k, fk, s, go, gs = make_config_inputs(1, 3, 128, 64, torch.float32, seed=1)
+def test_which_tensors_run_as_blocks():
+    from t2fw_amd import _lib
+    from t2fw_amd.functional_lfw import _block_counts
+    t = lambda w, dtype=torch.float16: torch.empty(2, 3, w, dtype=dtype)
+    assert _block_counts(t(128), t(64), 0) == (2, 1)
+    assert _block_counts(t(64), t(192), 0) == (1, 3)
+    assert _block_counts(t(256, torch.bfloat16), t(128, torch.bfloat16), 0) == (4, 2)
+    assert _block_counts(t(64), t(64), 0) is None                       # the kernels' own shape
+    assert _block_counts(t(128), t(100), 0) is None and _block_counts(t(32), t(64), 0) is None
+    assert _block_counts(t(128, torch.float32), t(128, torch.float32), 0) is None     # exact kernels
+    assert _block_counts(t(128), t(128), _lib.FLAG_FORCE_SCAN) is None
+
+
+def test_padding_takes_16_bit_tensors_only():
+    from t2fw_amd import lfw_apply_padded
+    x, f, q, k, fk, s, go, gs = make_config_inputs(1, 3, 100, 64, torch.float32, seed=1)
     with pytest.raises(AssertionError):
-        lfw_apply_blocked(x, f, q, k, fk, s)
+        lfw_apply_padded(x, f, q, k, fk, s)
 
 
-@pytest.mark.gpu
-@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
-@pytest.mark.parametrize("D,K", [(128, 64), (64, 128), (128, 128), (192, 64), (32, 32), (100, 70), (65, 64)])
-def test_blocked_widths_on_the_matrix_cores(D, K, dtype):
-    """against the fp64 C oracle at the matrix-core kernels' tolerance (the gate gradients at theirs)"""
+def _check_on_gpu(fn, D, K, dtype, B=3, T=200):
     from oracle import c_oracle
-    from t2fw_amd import lfw_apply_blocked
     from tests.test_lfw_chunk_gpu import NAMES
     from tests.test_lfw_gpu import TOL_CHUNK, TOL_CHUNK_GATE, assert_close
-    B, T = 3, 200
     x, f, q, k, fk, s, go, gs = make_config_inputs(B, T, D, K, dtype, seed=3 * D + K, gate_mean=2.5, state_std=0.3)
     leaves = [t.cuda().requires_grad_(True) for t in (x, f, q, k, fk, s)]
-    out, nxt = lfw_apply_blocked(*leaves)
+    out, nxt = fn(*leaves)
     torch.autograd.backward([out, nxt], [go.cuda(), gs.cuda()])
     torch.cuda.synchronize()
     assert out.shape == (B, T, D) and nxt.shape == (B, D, K) and out.dtype == dtype and out.is_contiguous()
@@ -75,17 +89,61 @@ def test_blocked_widths_on_the_matrix_cores(D, K, dtype):
     for n, t, r in zip(NAMES, leaves, r_grads):
         assert t.grad.shape == t.shape
         assert_close(t.grad, r, dtype, n, tol=TOL_CHUNK_GATE if n in ("d_f", "d_f_key") else TOL_CHUNK)
+    return out
 
 
 @pytest.mark.gpu
-def test_blocked_path_runs_the_matrix_core_kernels_not_the_exact_ones():
-    """128 x 128: different from LFWFunction.apply on the same tensors (exact kernels), by no more than the
-    matrix-core tolerance"""
-    from t2fw_amd import LFWFunction, lfw_apply_blocked
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("D,K", [(128, 64), (64, 128), (128, 128), (192, 64), (256, 128)])
+def test_multiples_of_64_through_the_autograd_function(D, K, dtype):
+    """LFWFunction.apply itself, against the fp64 C oracle at the matrix-core kernels' tolerance"""
+    from t2fw_amd import LFWFunction
+    _check_on_gpu(LFWFunction.apply, D, K, dtype)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("D,K", [(32, 32), (100, 70), (65, 64), (1, 1), (128, 130)])
+def test_other_widths_padded(D, K, dtype):
+    from t2fw_amd import lfw_apply_padded
+    _check_on_gpu(lfw_apply_padded, D, K, dtype)
+
+
+@pytest.mark.gpu
+def test_blocks_run_the_matrix_core_kernels_and_force_scan_the_exact_ones(monkeypatch):
+    """128 x 128: different from the exact kernels' results (T2FW_FLAGS=1) by no more than the matrix-core
+    tolerance, and not equal to them"""
+    from t2fw_amd import LFWFunction
     x, f, q, k, fk, s, go, gs = make_config_inputs(2, 300, 128, 128, torch.float16, seed=77, gate_mean=2.5, state_std=0.3)
     ins = [t.cuda() for t in (x, f, q, k, fk, s)]
-    a, _ = lfw_apply_blocked(*ins)
+    a, _ = LFWFunction.apply(*ins)
+    monkeypatch.setenv("T2FW_FLAGS", "1")
     b, _ = LFWFunction.apply(*ins)
     torch.cuda.synchronize()
     assert not torch.equal(a, b)
     assert (a.double() - b.double()).abs().max() <= 2e-2 * b.double().abs().max()
+
+
+@pytest.mark.gpu
+def test_gated_and_float32_routes_inherit_the_blocks():
+    """LFWGatedFunction and lfw_apply_16bit go through the same calls: 128 x 64 on logits, and float32 tensors
+    narrowed to fp16, against the oracle"""
+    from oracle import c_oracle
+    from t2fw_amd import LFWGatedFunction, lfw_apply_16bit, sigmoid_gates
+    from tests.test_lfw_gpu import TOL_CHUNK, assert_close
+    B, T, D, K = 2, 150, 128, 64
+    g = torch.Generator().manual_seed(4)
+    x, q, k = [(torch.randn(B, T, w, generator=g) * 0.125).half() for w in (D, K, K)]
+    zf, zk = [(torch.randn(B, T, w, generator=g) + 2.5).half() for w in (D, K)]
+    s = (torch.randn(B, D, K, generator=g) * 0.3).half()
+    out, nxt = LFWGatedFunction.apply(x.cuda(), zf.cuda(), q.cuda(), k.cuda(), zk.cuda(), s.cuda())
+    f, fk = [t.cpu() for t in sigmoid_gates(zf.cuda(), zk.cuda())]
+    r_out, r_nxt = c_oracle.lfw_forward(x, f, q, k, fk, s)
+    assert_close(out, r_out, torch.float16, "outputs (logits)", tol=TOL_CHUNK)
+    assert_close(nxt, r_nxt, torch.float16, "next_state (logits)", tol=TOL_CHUNK)
+    x32, f32, q32, k32, fk32, s32, _, _ = make_config_inputs(B, T, D, K, torch.float32, seed=8, gate_mean=2.5, state_std=0.3)
+    out, nxt = lfw_apply_16bit(*[t.cuda() for t in (x32, f32, q32, k32, fk32, s32)])
+    r_out, r_nxt = c_oracle.lfw_forward(x32, f32, q32, k32, fk32, s32)
+    assert out.dtype == torch.float32
+    assert (out.double().cpu() - torch.as_tensor(r_out).double()).abs().max() <= 1e-2 * torch.as_tensor(r_out).double().abs().max()
+    assert (nxt.double().cpu() - torch.as_tensor(r_nxt).double()).abs().max() <= 1e-2 * torch.as_tensor(r_nxt).double().abs().max()
