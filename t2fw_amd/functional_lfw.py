@@ -77,47 +77,53 @@ def _dtype_code(dtype):
 # The recurrence couples neither the rows of the state nor its columns: S[d, k] sees x[d], f[d], k[k], f_key[k]
 # only, and o[d] is a sum over k.  A D x K state is (D / 64) (K / 64) independent 64 x 64 recurrences -- value
 # channels 64 i .. 64 i + 63 with key channels 64 j .. 64 j + 63 -- whose outputs add up over j.  For fp16 / bf16
-# tensors the blocks run as heads (h = i * nk + j) through the head-strided entry points, i.e. on the matrix-core
+# tensors the blocks run as heads through the head-strided entry points, i.e. on the matrix-core
 # kernels, which take 64 x 64 states only; the exact per-step kernels that would otherwise serve such widths take
 # 4.1 ms for a forward + backward at B=24, T=1024, D=K=128 where the blocks take 0.24 ms.  The reference has one
 # kernel for every shape (t2fw/csrc/lfw_kernel.cu:105-121).
 def _block_counts(value, query, flags):
     """(D / 64, K / 64) if tensors of these widths run as blocks, else None"""
     D, K = value.shape[-1], query.shape[-1]
-    if value.dim() != 3 or value.dtype not in (torch.float16, torch.bfloat16) or (flags & _lib.FLAG_FORCE_SCAN):
+    if value.dim() not in (3, 4) or value.dtype not in (torch.float16, torch.bfloat16) or (flags & _lib.FLAG_FORCE_SCAN):
         return None
     if D % 64 or K % 64 or D == 0 or K == 0 or (D == 64 and K == 64):
         return None
     return D // 64, K // 64
 
 
+# Tensors are [B,T,W] or, with a head axis, [B,T,H,W]; states [B,D,K] or [B,H,D,K].  Block (i, j) of head h becomes
+# head (h * nd + i) * nk + j of the 64-wide call.
 def _value_blocks(t, nd, nk):
-    B, T = t.shape[:2]
-    return t.view(B, T, nd, 1, 64).expand(B, T, nd, nk, 64).reshape(B, T, nd * nk, 64).contiguous()
+    lead = t.shape[:-1]
+    return t.view(*lead, nd, 1, 64).expand(*lead, nd, nk, 64).reshape(lead[0], lead[1], -1, 64).contiguous()
 
 
 def _key_blocks(t, nd, nk):
-    B, T = t.shape[:2]
-    return t.view(B, T, 1, nk, 64).expand(B, T, nd, nk, 64).reshape(B, T, nd * nk, 64).contiguous()
+    lead = t.shape[:-1]
+    return t.view(*lead, 1, nk, 64).expand(*lead, nd, nk, 64).reshape(lead[0], lead[1], -1, 64).contiguous()
 
 
 def _state_blocks(s, nd, nk):
-    return s.view(s.shape[0], nd, 64, nk, 64).permute(0, 1, 3, 2, 4).reshape(s.shape[0], nd * nk, 64, 64).contiguous()
+    B = s.shape[0]
+    return s.view(B, -1, nd, 64, nk, 64).permute(0, 1, 2, 4, 3, 5).reshape(B, -1, 64, 64).contiguous()
 
 
-def _state_from_blocks(sb, nd, nk):
-    return sb.view(sb.shape[0], nd, nk, 64, 64).permute(0, 1, 3, 2, 4).reshape(sb.shape[0], 64 * nd, 64 * nk)
+def _state_from_blocks(sb, nd, nk, like):
+    """back to the shape of ``like`` ([B,D,K] or [B,H,D,K])"""
+    B = sb.shape[0]
+    return sb.view(B, -1, nd, nk, 64, 64).permute(0, 1, 2, 4, 3, 5).reshape(like.shape)
 
 
-def _sum_key_blocks(tb, nd, nk):
-    """[B,T,nd*nk,64] -> [B,T,64*nd]: what the blocks of one row of blocks hold adds up (fp32 accumulation)"""
+def _sum_key_blocks(tb, nd, nk, like):
+    """[B,T,heads of blocks,64] -> the shape of ``like`` ([B,T,D] or [B,T,H,D]): what the blocks of one row of
+    blocks hold adds up (fp32 accumulation)"""
     B, T = tb.shape[:2]
-    return tb.view(B, T, nd, nk, 64).sum(dim=3).view(B, T, 64 * nd)
+    return tb.view(B, T, -1, nd, nk, 64).sum(dim=4).reshape(like.shape)
 
 
-def _sum_value_blocks(tb, nd, nk):
+def _sum_value_blocks(tb, nd, nk, like):
     B, T = tb.shape[:2]
-    return tb.view(B, T, nd, nk, 64).sum(dim=2).view(B, T, 64 * nk)
+    return tb.view(B, T, -1, nd, nk, 64).sum(dim=3).reshape(like.shape)
 
 
 class _BlockedCall:
@@ -136,7 +142,7 @@ def _lfw_forward_blocked(value, forget, query, key, f_key, state, need_grad, blo
                _key_blocks(key, nd, nk), _key_blocks(f_key, nd, nk), _state_blocks(state, nd, nk))
     out_b, nxt_b, ckpt, C, flags, hints = _lfw_forward(*tensors, need_grad, heads=True)
     kept = _BlockedCall(tensors, hints) if need_grad else None
-    return _sum_key_blocks(out_b, nd, nk), _state_from_blocks(nxt_b, nd, nk), ckpt, C, flags, kept
+    return _sum_key_blocks(out_b, nd, nk, value), _state_from_blocks(nxt_b, nd, nk, state), ckpt, C, flags, kept
 
 
 def _lfw_backward_blocked(grad_output, grad_state, value, forget, query, key, f_key, state, ckpt, C, flags, kept, blocks):
@@ -151,8 +157,9 @@ def _lfw_backward_blocked(grad_output, grad_state, value, forget, query, key, f_
     d_xb, d_fb, d_qb, d_kb, d_fkb, d_sb = _lfw_backward(
         _value_blocks(grad_output, nd, nk), _state_blocks(grad_state, nd, nk), *tensors, ckpt, C, flags, heads=True,
         hints=hints)
-    return (_sum_key_blocks(d_xb, nd, nk), _sum_key_blocks(d_fb, nd, nk), _sum_value_blocks(d_qb, nd, nk),
-            _sum_value_blocks(d_kb, nd, nk), _sum_value_blocks(d_fkb, nd, nk), _state_from_blocks(d_sb, nd, nk))
+    return (_sum_key_blocks(d_xb, nd, nk, value), _sum_key_blocks(d_fb, nd, nk, value),
+            _sum_value_blocks(d_qb, nd, nk, query), _sum_value_blocks(d_kb, nd, nk, query),
+            _sum_value_blocks(d_fkb, nd, nk, query), _state_from_blocks(d_sb, nd, nk, state))
 
 
 def _lfw_forward(value, forget, query, key, f_key, state, need_grad, heads=False):
@@ -185,10 +192,9 @@ def _lfw_forward(value, forget, query, key, f_key, state, need_grad, heads=False
                            % (tuple(value.shape), tuple(query.shape), tuple(state.shape)))
     code = _dtype_code(value.dtype)
     flags = _flags()
-    if not heads:
-        blocks = _block_counts(value, query, flags)
-        if blocks is not None:
-            return _lfw_forward_blocked(value, forget, query, key, f_key, state, need_grad, blocks)
+    blocks = _block_counts(value, query, flags)
+    if blocks is not None:
+        return _lfw_forward_blocked(value, forget, query, key, f_key, state, need_grad, blocks)
     lib = _lib.load()
     C = _ckpt_interval()
     dev = value.device
@@ -228,11 +234,10 @@ def _lfw_backward(grad_output, grad_state, value, forget, query, key, f_key, sta
     assert grad_output.dtype == value.dtype
     grad_output = grad_output.contiguous()
     grad_state = grad_state.contiguous()
-    if not heads:
-        blocks = _block_counts(value, query, flags)
-        if blocks is not None:
-            return _lfw_backward_blocked(grad_output, grad_state, value, forget, query, key, f_key, state, ckpt, C,
-                                         flags, hints, blocks)
+    blocks = _block_counts(value, query, flags)
+    if blocks is not None:
+        return _lfw_backward_blocked(grad_output, grad_state, value, forget, query, key, f_key, state, ckpt, C,
+                                     flags, hints, blocks)
     B, T = value.shape[:2]
     H = value.shape[2] if heads else 1
     D, K = value.shape[-1], query.shape[-1]

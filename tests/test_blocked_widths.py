@@ -34,20 +34,30 @@ def _heads_backward_by_oracle(go, gs, x, f, q, k, fk, s, ckpt, C, flags, heads=F
     return tuple(unfold(g) for g in grads[:5]) + (grads[5].view(B, H, 64, 64),)
 
 
+@pytest.mark.parametrize("H", [0, 3])
 @pytest.mark.parametrize("D,K", [(128, 64), (64, 128), (128, 128), (192, 64), (64, 192), (256, 128)])
-def test_decomposition_is_the_same_recurrence(monkeypatch, D, K):
+def test_decomposition_is_the_same_recurrence(monkeypatch, D, K, H):
+    """H = 0: [B,T,W] tensors; H = 3: a head axis, [B,T,H,W] tensors and [B,H,D,K] states"""
     from t2fw_amd import functional_lfw as F
     monkeypatch.setattr(F, "_lfw_forward", _heads_forward_by_oracle)
     monkeypatch.setattr(F, "_lfw_backward", _heads_backward_by_oracle)
     B, T = 2, 9
-    x, f, q, k, fk, s, go, gs = [t.double() for t in make_config_inputs(B, T, D, K, torch.float32, seed=D + K, state_std=0.5)]
+    rows = B * max(H, 1)
+    x, f, q, k, fk, s, go, gs = [t.double() for t in make_config_inputs(rows, T, D, K, torch.float32, seed=D + K, state_std=0.5)]
     leaves = [t.clone().requires_grad_(True) for t in (x, f, q, k, fk, s)]
     r_out, r_nxt = lfw_reference(*leaves)
     torch.autograd.backward([r_out, r_nxt], [go, gs])
+    refs = [r_out.detach(), r_nxt.detach()] + [t.grad for t in leaves]
+    if H:       # rows are (batch, head) pairs: the same data with the head axis next to the channels
+        to_heads = lambda t: t.view(B, H, T, -1).transpose(1, 2).contiguous() if t.shape[1] == T and t.dim() == 3 else t.view(B, H, *t.shape[1:])
+        x, f, q, k, fk, go = [t.view(B, H, T, -1).transpose(1, 2).contiguous() for t in (x, f, q, k, fk, go)]
+        s, gs = s.view(B, H, D, K), gs.view(B, H, D, K)
+        refs = [refs[0].view(B, H, T, D).transpose(1, 2), refs[1].view(B, H, D, K)] + \
+               [r.view(B, H, T, -1).transpose(1, 2) for r in refs[2:7]] + [refs[7].view(B, H, D, K)]
     blocks = (D // 64, K // 64)
-    out, nxt, ckpt, C, flags, hints = F._lfw_forward_blocked(x, f, q, k, fk, s, True, blocks)
-    grads = F._lfw_backward_blocked(go, gs, x, f, q, k, fk, s, ckpt, C, flags, hints, blocks)
-    for a, b in zip([out, nxt] + list(grads), [r_out.detach(), r_nxt.detach()] + [t.grad for t in leaves]):
+    out, nxt, ckpt, C, flags, kept = F._lfw_forward_blocked(x, f, q, k, fk, s, True, blocks)
+    grads = F._lfw_backward_blocked(go, gs, x, f, q, k, fk, s, ckpt, C, flags, kept, blocks)
+    for a, b in zip([out, nxt] + list(grads), refs):
         assert a.shape == b.shape
         assert torch.allclose(a, b, rtol=1e-12, atol=1e-12)
 
@@ -63,6 +73,8 @@ def test_which_tensors_run_as_blocks():
     assert _block_counts(t(128), t(100), 0) is None and _block_counts(t(32), t(64), 0) is None
     assert _block_counts(t(128, torch.float32), t(128, torch.float32), 0) is None     # exact kernels
     assert _block_counts(t(128), t(128), _lib.FLAG_FORCE_SCAN) is None
+    heads = lambda w: torch.empty(2, 3, 5, w, dtype=torch.float16)
+    assert _block_counts(heads(128), heads(64), 0) == (2, 1) and _block_counts(heads(64), heads(64), 0) is None
 
 
 def test_padding_takes_16_bit_tensors_only():
@@ -107,6 +119,32 @@ def test_multiples_of_64_through_the_autograd_function(D, K, dtype):
 def test_other_widths_padded(D, K, dtype):
     from t2fw_amd import lfw_apply_padded
     _check_on_gpu(lfw_apply_padded, D, K, dtype)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("D,K", [(128, 64), (128, 128)])
+def test_head_strided_tensors_with_wide_heads(D, K):
+    """LFWHeadsFunction on [B,T,H,D] tensors with D, K multiples of 64: against the oracle on the folded rows"""
+    from oracle import c_oracle
+    from t2fw_amd import LFWHeadsFunction
+    from tests.test_lfw_chunk_gpu import NAMES
+    from tests.test_lfw_gpu import TOL_CHUNK, TOL_CHUNK_GATE, assert_close
+    B, H, T, dtype = 2, 3, 130, torch.float16
+    x, f, q, k, fk, s, go, gs = make_config_inputs(B * H, T, D, K, dtype, seed=D + 7 * K, gate_mean=2.5, state_std=0.3)
+    r_out, r_nxt = c_oracle.lfw_forward(x, f, q, k, fk, s)
+    r_grads = c_oracle.lfw_backward(go, gs, x, f, q, k, fk, s)
+    heads = lambda t: t.view(B, H, T, -1).transpose(1, 2).contiguous()
+    fold = lambda t: t.transpose(1, 2).reshape(B * H, T, -1)
+    leaves = [heads(t).cuda().requires_grad_(True) for t in (x, f, q, k, fk)] + [s.view(B, H, D, K).cuda().requires_grad_(True)]
+    out, nxt = LFWHeadsFunction.apply(*leaves)
+    torch.autograd.backward([out, nxt], [heads(go).cuda(), gs.view(B, H, D, K).cuda()])
+    torch.cuda.synchronize()
+    assert out.shape == (B, T, H, D) and nxt.shape == (B, H, D, K)
+    assert_close(fold(out), r_out, dtype, "outputs", tol=TOL_CHUNK)
+    assert_close(nxt.reshape(B * H, D, K), r_nxt, dtype, "next_state", tol=TOL_CHUNK)
+    for n, t, r in zip(NAMES, leaves, r_grads):
+        g = t.grad.reshape(B * H, D, K) if n == "d_state" else fold(t.grad)
+        assert_close(g, r, dtype, n, tol=TOL_CHUNK_GATE if n in ("d_f", "d_f_key") else TOL_CHUNK)
 
 
 @pytest.mark.gpu
